@@ -1,0 +1,35 @@
+// C entry points of the gfx950 kernel library.  Every function enqueues work on `stream` and returns
+// 0, or a non-zero code (see common.h) without launching when it refuses its arguments.  Pointers are
+// device pointers; matrices are row-major.  `dtype` is 0 for float and 1 for bfloat16.
+#pragma once
+#include <hip/hip_runtime.h>
+
+extern "C" {
+
+int ms_embed(const int* ids, const void* table, float* out, int n_tokens, int hidden, int dtype, hipStream_t stream);
+
+int ms_rms_norm(float* x, const void* delta, int delta_dtype, const float* weight, const int* rows, void* out,
+                int n_rows, int hidden, float eps, int write_back, int dtype, hipStream_t stream);
+
+int ms_residual_add(float* x, const void* delta, long long total, int dtype, hipStream_t stream);
+
+int ms_silu_mul(const void* gate_up, void* out, int n_tokens, int intermediate, int dtype, hipStream_t stream);
+
+int ms_rope_store(void* qkv, const int* positions, const float* inv_freq, const int* slot_mapping, void* k_pages,
+                  void* v_pages, int n_tokens, int num_heads, int num_kv_heads, int head_dim, int rot_dim,
+                  int page_size, int dtype, hipStream_t stream);
+
+int ms_gemm_generic(const void* A, const void* W, const float* bias, void* C, int M, int N, int K, long long lda,
+                    long long ldw, long long ldc, int in_dtype, int out_dtype, int accumulate, hipStream_t stream);
+
+int ms_paged_attention_generic(const void* q, long long q_stride, const void* k_pages, const void* v_pages,
+                               const int* block_table, int table_stride, const int* token_req, const int* positions,
+                               void* out, long long out_stride, int n_tokens, int num_heads, int num_kv_heads,
+                               int head_dim, int page_size, long long num_pages, float scale, int window, int dtype,
+                               hipStream_t stream);
+
+int ms_sample(const float* logits, long long ld, int n_rows, int vocab, const float* temperature, const int* top_k,
+              const float* top_p, const unsigned long long* seeds, const int* draw_index, int* out,
+              hipStream_t stream);
+
+}  // extern "C"

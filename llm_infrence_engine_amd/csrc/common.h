@@ -1,0 +1,50 @@
+// Shared helpers of the gfx950 kernels: element types, conversions, wave/block reductions.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <stdint.h>
+
+#define MS_WAVE 64
+
+// Element type codes of the C entry points.
+enum { MS_F32 = 0, MS_BF16 = 1 };
+
+// Error codes returned by the C entry points (0 = launched).
+enum { MS_OK = 0, MS_BAD_ARG = 1, MS_UNSUPPORTED = 2, MS_LAUNCH_FAILED = 3 };
+
+typedef __hip_bfloat16 bf16;
+
+__device__ __forceinline__ float to_float(float v) { return v; }
+__device__ __forceinline__ float to_float(bf16 v) { return __bfloat162float(v); }
+
+template <typename T> __device__ __forceinline__ T from_float(float v);
+template <> __device__ __forceinline__ float from_float<float>(float v) { return v; }
+template <> __device__ __forceinline__ bf16 from_float<bf16>(float v) { return __float2bfloat16(v); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = MS_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, MS_WAVE);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = MS_WAVE / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, MS_WAVE));
+  return v;
+}
+
+// Sum over a block of up to 1024 threads; every thread gets the result.  `red` holds 16 floats of LDS.
+__device__ __forceinline__ float block_sum(float v, float* red) {
+  const int lane = threadIdx.x & (MS_WAVE - 1), wave = threadIdx.x / MS_WAVE;
+  const int nwaves = (blockDim.x + MS_WAVE - 1) / MS_WAVE;
+  v = wave_sum(v);
+  __syncthreads();  // `red` may still be read from a previous call
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  float t = 0.f;
+  for (int i = 0; i < nwaves; ++i) t += red[i];
+  return t;
+}
+
+static inline int ms_launch_status() {
+  return hipGetLastError() == hipSuccess ? MS_OK : MS_LAUNCH_FAILED;
+}

@@ -1,0 +1,184 @@
+// Row-wise kernels: embedding gather, RMS norm (with the residual sum fused), gated activation,
+// rotary position encoding fused with the write of keys and values into cache pages.
+// The residual stream is float in every mode; sums of squares, the normalisation, rotation angles
+// and the activation are computed in float.
+#include "common.h"
+#include "api.h"
+
+// ------------------------------------------------------------------------------------------------
+// out[n, :] = float(table[ids[n], :])
+template <typename T>
+__global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table, float* __restrict__ out, int H) {
+  const int n = blockIdx.x;
+  const T* row = table + (size_t)ids[n] * H;
+  float* o = out + (size_t)n * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = to_float(row[i]);
+}
+
+extern "C" int ms_embed(const int* ids, const void* table, float* out, int n_tokens, int hidden, int dtype,
+                        hipStream_t stream) {
+  if (n_tokens <= 0) return MS_OK;
+  if (hidden <= 0) return MS_BAD_ARG;
+  dim3 grid(n_tokens), block(256);
+  if (dtype == MS_F32) embed_kernel<float><<<grid, block, 0, stream>>>(ids, (const float*)table, out, hidden);
+  else if (dtype == MS_BF16) embed_kernel<bf16><<<grid, block, 0, stream>>>(ids, (const bf16*)table, out, hidden);
+  else return MS_BAD_ARG;
+  return ms_launch_status();
+}
+
+// ------------------------------------------------------------------------------------------------
+// Row r of the output is the norm of row rows[r] (or r) of x.  With `delta`, x[row] += delta[row]
+// first (written back), which is the residual sum of the layer before.  `delta2` is a second addend.
+// y = w * (x * rsqrt(mean(x^2) + eps)), all in float, rounded once on store.
+template <typename T, typename TD>
+__global__ void rms_norm_kernel(float* __restrict__ x, const TD* __restrict__ delta, const float* __restrict__ w,
+                                const int* __restrict__ rows, T* __restrict__ out, int H, float eps, int write_back) {
+  __shared__ float red[16];
+  extern __shared__ float buf[];  // H floats: the row after the residual sum
+  const int r = blockIdx.x;
+  const int src = rows ? rows[r] : r;
+  float* xr = x + (size_t)src * H;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float v = xr[i];
+    if (delta) {
+      v += to_float(delta[(size_t)src * H + i]);
+      if (write_back) xr[i] = v;
+    }
+    buf[i] = v;
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+  T* o = out + (size_t)r * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = from_float<T>(w[i] * (buf[i] * inv));
+}
+
+extern "C" int ms_rms_norm(float* x, const void* delta, int delta_dtype, const float* weight, const int* rows,
+                           void* out, int n_rows, int hidden, float eps, int write_back, int dtype,
+                           hipStream_t stream) {
+  if (n_rows <= 0) return MS_OK;
+  if (hidden <= 0 || hidden > 16384) return MS_UNSUPPORTED;  // the row is staged in LDS
+  dim3 grid(n_rows), block(hidden >= 1024 ? 256 : 128);
+  size_t lds = (size_t)hidden * sizeof(float);
+#define LAUNCH(T, TD) rms_norm_kernel<T, TD><<<grid, block, lds, stream>>>(x, (const TD*)delta, weight, rows, (T*)out, hidden, eps, write_back)
+  if (dtype == MS_F32) {
+    if (delta && delta_dtype == MS_BF16) return MS_BAD_ARG;
+    LAUNCH(float, float);
+  } else if (dtype == MS_BF16) {
+    if (delta && delta_dtype == MS_F32) LAUNCH(bf16, float);
+    else LAUNCH(bf16, bf16);
+  } else return MS_BAD_ARG;
+#undef LAUNCH
+  return ms_launch_status();
+}
+
+// ------------------------------------------------------------------------------------------------
+// x[n, :] += delta[n, :]  (the residual sum alone, for arrangements that do not fuse it into a norm)
+template <typename TD>
+__global__ void residual_add_kernel(float* __restrict__ x, const TD* __restrict__ delta, size_t total) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < total; i += stride) x[i] += to_float(delta[i]);
+}
+
+extern "C" int ms_residual_add(float* x, const void* delta, long long total, int dtype, hipStream_t stream) {
+  if (total <= 0) return MS_OK;
+  int blocks = (int)((total + 255) / 256);
+  if (blocks > 4096) blocks = 4096;
+  if (dtype == MS_F32) residual_add_kernel<float><<<blocks, 256, 0, stream>>>(x, (const float*)delta, (size_t)total);
+  else if (dtype == MS_BF16) residual_add_kernel<bf16><<<blocks, 256, 0, stream>>>(x, (const bf16*)delta, (size_t)total);
+  else return MS_BAD_ARG;
+  return ms_launch_status();
+}
+
+// ------------------------------------------------------------------------------------------------
+// out[n, i] = silu(gu[n, i]) * gu[n, I + i],  silu(z) = z / (1 + exp(-z))
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total) {
+  size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; idx < total; idx += stride) {
+    const size_t n = idx / I;
+    const int i = (int)(idx - n * I);
+    const float g = to_float(gu[n * 2 * I + i]);
+    const float u = to_float(gu[n * 2 * I + I + i]);
+    out[idx] = from_float<T>(g / (1.0f + expf(-g)) * u);
+  }
+}
+
+extern "C" int ms_silu_mul(const void* gate_up, void* out, int n_tokens, int intermediate, int dtype,
+                           hipStream_t stream) {
+  if (n_tokens <= 0) return MS_OK;
+  if (intermediate <= 0) return MS_BAD_ARG;
+  const size_t total = (size_t)n_tokens * intermediate;
+  int blocks = (int)((total + 255) / 256);
+  if (blocks > 8192) blocks = 8192;
+  if (dtype == MS_F32) silu_mul_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gate_up, (float*)out, intermediate, total);
+  else if (dtype == MS_BF16) silu_mul_kernel<bf16><<<blocks, 256, 0, stream>>>((const bf16*)gate_up, (bf16*)out, intermediate, total);
+  else return MS_BAD_ARG;
+  return ms_launch_status();
+}
+
+// ------------------------------------------------------------------------------------------------
+// One block per token.  qkv[n] = [q heads | k heads | v heads], head_dim values each.
+// The first rot_dim values of every q and k head are rotated with half-split pairing (j, j + rot_dim/2):
+//   x1' = x1 cos - x2 sin,  x2' = x2 cos + x1 sin,  angle = float(position) * inv_freq[j]
+// q is rotated in place.  With pages given, the rotated k and v go to
+// pages[slot / page_size][kv head][slot % page_size][:] for slot = slot_mapping[n] (slot < 0: not stored);
+// k is also rotated in place so that a caller without pages sees it.
+template <typename T>
+__global__ void rope_store_kernel(T* __restrict__ qkv, const int* __restrict__ positions,
+                                  const float* __restrict__ inv_freq, const int* __restrict__ slot_mapping,
+                                  T* __restrict__ k_pages, T* __restrict__ v_pages, int nh, int nkv, int d,
+                                  int rot_dim, int page_size) {
+  const int n = blockIdx.x;
+  T* row = qkv + (size_t)n * (nh + 2 * nkv) * d;
+  const float pos = (float)positions[n];
+  const int half = rot_dim / 2;
+  long long slot = -1;
+  if (k_pages) slot = slot_mapping[n];
+  const long long page = slot >= 0 ? slot / page_size : 0;
+  const int off = slot >= 0 ? (int)(slot % page_size) : 0;
+
+  // rotate q and k heads: work item = (head, j)
+  const int n_rot_heads = nh + nkv;
+  for (int w = threadIdx.x; w < n_rot_heads * half; w += blockDim.x) {
+    const int h = w / half, j = w - h * half;
+    T* x = row + (size_t)h * d;
+    float s, c;
+    sincosf(pos * inv_freq[j], &s, &c);
+    const float x1 = to_float(x[j]), x2 = to_float(x[j + half]);
+    x[j] = from_float<T>(x1 * c - x2 * s);
+    x[j + half] = from_float<T>(x2 * c + x1 * s);
+  }
+  if (slot < 0) return;
+  __syncthreads();
+  // copy k and v heads into the page
+  const T* k = row + (size_t)nh * d;
+  const T* v = k + (size_t)nkv * d;
+  for (int w = threadIdx.x; w < nkv * d; w += blockDim.x) {
+    const int h = w / d, i = w - h * d;
+    const size_t dst = (((size_t)page * nkv + h) * page_size + off) * d + i;
+    k_pages[dst] = k[w];
+    v_pages[dst] = v[w];
+  }
+}
+
+extern "C" int ms_rope_store(void* qkv, const int* positions, const float* inv_freq, const int* slot_mapping,
+                             void* k_pages, void* v_pages, int n_tokens, int num_heads, int num_kv_heads,
+                             int head_dim, int rot_dim, int page_size, int dtype, hipStream_t stream) {
+  if (n_tokens <= 0) return MS_OK;
+  if (num_heads < 0 || num_kv_heads < 0 || head_dim <= 0 || rot_dim < 0 || rot_dim > head_dim || (rot_dim & 1))
+    return MS_BAD_ARG;
+  if ((k_pages == nullptr) != (v_pages == nullptr)) return MS_BAD_ARG;
+  if (k_pages && (page_size <= 0 || slot_mapping == nullptr)) return MS_BAD_ARG;
+  if (rot_dim > 0 && (positions == nullptr || inv_freq == nullptr)) return MS_BAD_ARG;
+  dim3 grid(n_tokens), block(256);
+#define LAUNCH(T) rope_store_kernel<T><<<grid, block, 0, stream>>>((T*)qkv, positions, inv_freq, slot_mapping, (T*)k_pages, (T*)v_pages, num_heads, num_kv_heads, head_dim, rot_dim, page_size)
+  if (dtype == MS_F32) LAUNCH(float);
+  else if (dtype == MS_BF16) LAUNCH(bf16);
+  else return MS_BAD_ARG;
+#undef LAUNCH
+  return ms_launch_status();
+}

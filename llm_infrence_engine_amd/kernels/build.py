@@ -1,0 +1,132 @@
+"""Compiles the HIP sources under ``csrc/`` for gfx950 into one shared library and loads it.
+
+``build()`` always compiles.  ``load()`` takes the library that is there and compiles only when there
+is none, printing a line per file so that a first call in a fresh checkout shows progress.  The
+library sits beside this file; when that folder cannot be written (a read-only checkout) it goes to a
+per-user folder under the system's temporary directory instead.  There is no fallback: without the
+library every op raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+import time
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+PKG = Path(__file__).resolve().parent.parent
+CSRC = PKG / "csrc"
+LIB_NAME = "libminiserve_gfx950.so"
+ARCH = "gfx950"
+# -packed-fp32-ops off: hipcc must not form packed float instructions from scalar code
+FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang",
+         "-packed-fp32-ops", "-Wno-unused-command-line-argument"]
+
+_lib = None
+
+
+class KernelLibraryError(RuntimeError):
+    pass
+
+
+def _hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"),
+                 os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "bin", "hipcc")):
+        if cand and os.path.isfile(cand):
+            return cand
+    raise KernelLibraryError("hipcc not found (looked at $HIPCC, PATH and $ROCM_PATH/bin); the HIP kernels "
+                             "cannot be built and there is no fallback")
+
+
+def _writable(d: Path) -> bool:
+    try:
+        d.mkdir(parents=True, exist_ok=True)
+        probe = d / f".probe{os.getpid()}"
+        probe.write_text("")
+        probe.unlink()
+        return True
+    except OSError:
+        return False
+
+
+def _fallback_dir() -> Path:
+    return Path(tempfile.gettempdir()) / f"llm_infrence_engine_amd-{os.getuid()}"
+
+
+def library_path() -> Path | None:
+    """The built library, or None."""
+    for d in (PKG / "kernels", _fallback_dir()):
+        p = d / LIB_NAME
+        if p.is_file():
+            return p
+    return None
+
+
+def sources() -> list:
+    return sorted(CSRC.glob("*.hip"))
+
+
+def build(verbose: bool = True) -> Path:
+    """Compile every ``csrc/*.hip`` and link the library.  Returns its path."""
+    hipcc = _hipcc()
+    out_dir = PKG / "kernels"
+    if not _writable(out_dir):
+        out_dir = _fallback_dir()
+        if not _writable(out_dir):
+            raise KernelLibraryError(f"neither {PKG / 'kernels'} nor {out_dir} can be written")
+    obj_dir = out_dir / "_build"
+    obj_dir.mkdir(parents=True, exist_ok=True)
+    srcs = sources()
+    if not srcs:
+        raise KernelLibraryError(f"no HIP sources under {CSRC}")
+    t0 = time.time()
+
+    def say(msg):
+        if verbose:
+            print(f"[kernels {time.time() - t0:5.1f}s] {msg}", file=sys.stderr, flush=True)
+
+    say(f"compiling {len(srcs)} HIP sources for {ARCH} with {hipcc}")
+
+    def compile_one(src: Path):
+        obj = obj_dir / (src.stem + ".o")
+        cmd = [hipcc, *FLAGS, "-I", str(CSRC), "-c", str(src), "-o", str(obj)]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise KernelLibraryError(f"hipcc failed on {src.name}:\n{r.stdout}\n{r.stderr}")
+        say(f"compiled {src.name}")
+        return obj
+
+    workers = max(1, min(len(srcs), int(os.environ.get("MAX_JOBS", "0")) or os.cpu_count() or 4, 16))
+    with ThreadPoolExecutor(workers) as pool:
+        objs = list(pool.map(compile_one, srcs))
+    tmp = out_dir / (LIB_NAME + f".tmp{os.getpid()}")
+    r = subprocess.run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", str(tmp), *map(str, objs)],
+                       capture_output=True, text=True)
+    if r.returncode != 0:
+        raise KernelLibraryError(f"linking {LIB_NAME} failed:\n{r.stdout}\n{r.stderr}")
+    os.replace(tmp, out_dir / LIB_NAME)
+    say(f"linked {out_dir / LIB_NAME}")
+    global _lib
+    _lib = None
+    return out_dir / LIB_NAME
+
+
+def load() -> ctypes.CDLL:
+    """The loaded library; built first if it does not exist yet."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    import torch  # noqa: F401  (its HIP runtime must be the one in the process before ours binds to it)
+
+    path = library_path()
+    if path is None:
+        path = build(verbose=True)
+    try:
+        _lib = ctypes.CDLL(str(path))
+    except OSError as e:
+        raise KernelLibraryError(f"cannot load {path}: {e}") from e
+    return _lib

@@ -1,0 +1,231 @@
+"""Python face of the HIP kernel library: one function per kernel, each checking on the host that
+operand shapes, types and devices are what the kernel and its grid assume before anything is launched.
+
+All work goes to torch's current stream.  There is no CPU path: a tensor that is not on the GPU, or a
+missing library, raises.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import build
+
+F32, BF16 = 0, 1
+_CODES = {1: "bad argument", 2: "unsupported size", 3: "launch failed"}
+
+_c_int, _c_ll, _c_float, _c_ptr = ctypes.c_int, ctypes.c_longlong, ctypes.c_float, ctypes.c_void_p
+
+_SIGNATURES = {
+    "ms_embed": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    "ms_rms_norm": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
+    "ms_residual_add": [_c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr],
+    "ms_silu_mul": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    "ms_rope_store": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int,
+                      _c_int, _c_int, _c_ptr],
+    "ms_gemm_generic": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ll, _c_ll, _c_ll, _c_int,
+                        _c_int, _c_int, _c_ptr],
+    "ms_paged_attention_generic": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ll,
+                                   _c_int, _c_int, _c_int, _c_int, _c_int, _c_ll, _c_float, _c_int, _c_int, _c_ptr],
+    "ms_sample": [_c_ptr, _c_ll, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+}
+
+_fn = {}
+
+
+def _get(name):
+    f = _fn.get(name)
+    if f is None:
+        lib = build.load()
+        try:
+            f = getattr(lib, name)
+        except AttributeError as e:
+            raise build.KernelLibraryError(
+                f"{name} is not in {build.library_path()}; the library is older than its sources, build it again") from e
+        f.argtypes = _SIGNATURES[name]
+        f.restype = _c_int
+        _fn[name] = f
+    return f
+
+
+def _call(name, *args):
+    rc = _get(name)(*args)
+    if rc != 0:
+        raise RuntimeError(f"{name} refused its arguments: {_CODES.get(rc, rc)}")
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _code(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return F32
+    if dtype == torch.bfloat16:
+        return BF16
+    raise TypeError(f"kernels take float32 or bfloat16, not {dtype}")
+
+
+def _check(t: torch.Tensor, name: str, dtype=None, shape=None, contiguous=True):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a tensor")
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} is on {t.device}; the kernels run on the GPU only (there is no CPU path)")
+    if dtype is not None and t.dtype != dtype:
+        raise TypeError(f"{name} must be {dtype}, got {t.dtype}")
+    if contiguous and not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous")
+    if shape is not None:
+        if t.dim() != len(shape) or any(s is not None and s != a for s, a in zip(shape, t.shape)):
+            raise ValueError(f"{name} must have shape {list(shape)}, got {list(t.shape)}")
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+# ------------------------------------------------------------------------------------------------
+def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[n] = float(table[ids[n]]).  ids int32 [N] (checked against the table by the caller), out float32 [N, H]."""
+    _check(ids, "ids", torch.int32)
+    _check(table, "table")
+    V, H = table.shape
+    _check(out, "out", torch.float32, (ids.numel(), H))
+    _call("ms_embed", ids.data_ptr(), table.data_ptr(), out.data_ptr(), ids.numel(), H, _code(table.dtype), _stream())
+    return out
+
+
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
+             delta: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None,
+             write_back: bool = True) -> torch.Tensor:
+    """out[r] = weight * normalised(x[rows[r]] (+ delta[rows[r]])).  x float32 [N, H] is the residual stream;
+    with ``delta`` the sum is written back to x (unless ``write_back`` is False)."""
+    _check(x, "x", torch.float32)
+    N, H = x.shape
+    _check(weight, "weight", torch.float32, (H,))
+    n_rows = N
+    if rows is not None:
+        _check(rows, "rows", torch.int32)
+        n_rows = rows.numel()
+    _check(out, "out", None, (n_rows, H))
+    dcode = 0
+    if delta is not None:
+        _check(delta, "delta", None, (N, H))
+        dcode = _code(delta.dtype)
+    _call("ms_rms_norm", x.data_ptr(), _ptr(delta), dcode, weight.data_ptr(), _ptr(rows), out.data_ptr(), n_rows, H,
+          float(eps), int(write_back), _code(out.dtype), _stream())
+    return out
+
+
+def residual_add(x: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
+    _check(x, "x", torch.float32)
+    _check(delta, "delta", None, tuple(x.shape))
+    _call("ms_residual_add", x.data_ptr(), delta.data_ptr(), x.numel(), _code(delta.dtype), _stream())
+    return x
+
+
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[n, i] = silu(gate_up[n, i]) * gate_up[n, I + i]."""
+    _check(gate_up, "gate_up")
+    N, two_i = gate_up.shape
+    if two_i % 2:
+        raise ValueError("gate_up must have an even number of columns")
+    _check(out, "out", gate_up.dtype, (N, two_i // 2))
+    _call("ms_silu_mul", gate_up.data_ptr(), out.data_ptr(), N, two_i // 2, _code(out.dtype), _stream())
+    return out
+
+
+def rope_store(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, rot_dim: int = 0,
+               positions: Optional[torch.Tensor] = None, inv_freq: Optional[torch.Tensor] = None,
+               slot_mapping: Optional[torch.Tensor] = None, k_pages: Optional[torch.Tensor] = None,
+               v_pages: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Rotate q and k of ``qkv`` [N, (nh + 2 nkv) d] in place and store k, v into pages
+    [pages, nkv, page_size, d] at ``slot_mapping`` (page * page_size + offset)."""
+    _check(qkv, "qkv", None, (None, (num_heads + 2 * num_kv_heads) * head_dim))
+    N = qkv.shape[0]
+    page_size = 0
+    if rot_dim:
+        if rot_dim % 2 or rot_dim > head_dim:
+            raise ValueError(f"rot_dim {rot_dim} must be even and at most head_dim {head_dim}")
+        _check(positions, "positions", torch.int32, (N,))
+        _check(inv_freq, "inv_freq", torch.float32, (rot_dim // 2,))
+    if k_pages is not None:
+        _check(k_pages, "k_pages", qkv.dtype, (None, num_kv_heads, None, head_dim))
+        _check(v_pages, "v_pages", qkv.dtype, tuple(k_pages.shape))
+        _check(slot_mapping, "slot_mapping", torch.int32, (N,))
+        page_size = k_pages.shape[2]
+    _call("ms_rope_store", qkv.data_ptr(), _ptr(positions), _ptr(inv_freq), _ptr(slot_mapping), _ptr(k_pages),
+          _ptr(v_pages), N, num_heads, num_kv_heads, head_dim, rot_dim, page_size, _code(qkv.dtype), _stream())
+    return qkv
+
+
+def gemm_generic(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                 accumulate: bool = False) -> torch.Tensor:
+    """out (+)= a @ w.T (+ bias), float accumulation on the vector ALUs.  a [M, K] and out [M, N] may be row
+    slices of wider matrices (unit stride in the last dimension)."""
+    for t, name in ((a, "a"), (w, "w"), (out, "out")):
+        _check(t, name, contiguous=False)
+        if t.dim() != 2 or t.stride(1) != 1:
+            raise ValueError(f"{name} must be a matrix with unit stride along its rows")
+    M, K = a.shape
+    N = w.shape[0]
+    if w.shape[1] != K or tuple(out.shape) != (M, N):
+        raise ValueError(f"shapes do not fit: a {list(a.shape)}, w {list(w.shape)}, out {list(out.shape)}")
+    if a.dtype != w.dtype:
+        raise TypeError(f"a is {a.dtype} but w is {w.dtype}")
+    if bias is not None:
+        _check(bias, "bias", torch.float32, (N,))
+    _call("ms_gemm_generic", a.data_ptr(), w.data_ptr(), _ptr(bias), out.data_ptr(), M, N, K,
+          a.stride(0) if M > 1 else K, w.stride(0) if N > 1 else K, out.stride(0) if M > 1 else N,
+          _code(a.dtype), _code(out.dtype), int(accumulate), _stream())
+    return out
+
+
+def paged_attention_generic(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
+                            token_req: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, num_heads: int,
+                            scale: float, window: Optional[int] = None) -> torch.Tensor:
+    """out[n, h] = softmax(scale * q[n, h] . K[keys visible to n]) V, keys read in place from pages.
+
+    q: [N, >= nh * d] (a row slice of the fused projection is fine), out [N, nh * d],
+    pages [P, nkv, page_size, d], block_table int32 [R, max_pages], token_req / positions int32 [N].
+    Token n sees keys 0..positions[n] of request token_req[n] (the last ``window`` of them if given)."""
+    _check(k_pages, "k_pages")
+    P, nkv, page_size, d = k_pages.shape
+    _check(v_pages, "v_pages", k_pages.dtype, tuple(k_pages.shape))
+    _check(q, "q", k_pages.dtype, contiguous=False)
+    N = q.shape[0]
+    if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < num_heads * d:
+        raise ValueError(f"q must be [N, >= {num_heads * d}] with unit stride along rows, got {list(q.shape)}")
+    _check(out, "out", k_pages.dtype, (N, num_heads * d))
+    _check(block_table, "block_table", torch.int32)
+    if block_table.dim() != 2:
+        raise ValueError("block_table must be [requests, pages]")
+    _check(token_req, "token_req", torch.int32, (N,))
+    _check(positions, "positions", torch.int32, (N,))
+    if num_heads % nkv:
+        raise ValueError(f"{num_heads} query heads cannot share {nkv} key/value heads")
+    _call("ms_paged_attention_generic", q.data_ptr(), q.stride(0) if N > 1 else q.shape[1], k_pages.data_ptr(),
+          v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], token_req.data_ptr(), positions.data_ptr(),
+          out.data_ptr(), num_heads * d, N, num_heads, nkv, d, page_size, P, float(scale), int(window or 0),
+          _code(q.dtype), _stream())
+    return out
+
+
+def sample(logits: torch.Tensor, out: torch.Tensor, temperature: Optional[torch.Tensor] = None,
+           top_k: Optional[torch.Tensor] = None, top_p: Optional[torch.Tensor] = None,
+           seeds: Optional[torch.Tensor] = None, draw_index: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One token per row of float32 logits [M, V].  Without ``temperature`` (or where it is <= 0) the first
+    maximum; else a draw after top-k and top-p, repeatable from (seeds[r], draw_index[r])."""
+    _check(logits, "logits", torch.float32)
+    M, V = logits.shape
+    _check(out, "out", torch.int32, (M,))
+    for t, name, dt in ((temperature, "temperature", torch.float32), (top_k, "top_k", torch.int32),
+                        (top_p, "top_p", torch.float32), (seeds, "seeds", torch.int64),
+                        (draw_index, "draw_index", torch.int32)):
+        if t is not None:
+            _check(t, name, dt, (M,))
+    _call("ms_sample", logits.data_ptr(), V, M, V, _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(seeds),
+          _ptr(draw_index), out.data_ptr(), _stream())
+    return out

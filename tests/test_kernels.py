@@ -1,0 +1,270 @@
+"""Each HIP kernel alone against a plain float reference of the same op, at sizes other than the
+engine's (odd widths, head sizes in steps of 16, vocabularies that are no power of two)."""
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from llm_infrence_engine_amd.kernels import ops
+
+    return ops
+
+
+def tol(dtype):
+    # float: sums of a few hundred products; bfloat16: one rounding of the result (2^-8 relative) on top
+    return dict(atol=2e-5, rtol=2e-5) if dtype == torch.float32 else dict(atol=2e-2, rtol=1.6e-2)
+
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed(ops, dtype):
+    g = torch.Generator().manual_seed(0)
+    table = torch.randn(331, 72, generator=g).to(dtype).to(DEV)
+    ids = torch.randint(0, 331, (13,), generator=g).to(torch.int32).to(DEV)
+    out = torch.empty(13, 72, dtype=torch.float32, device=DEV)
+    ops.embed(ids, table, out)
+    assert torch.equal(out, table[ids.long()].float())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("H", [72, 896, 1500])
+def test_rms_norm(ops, dtype, H):
+    g = torch.Generator().manual_seed(1)
+    x = (torch.randn(9, H, generator=g) * 3).to(DEV)
+    w = (1 + 0.1 * torch.randn(H, generator=g)).to(DEV)
+    out = torch.empty(9, H, dtype=dtype, device=DEV)
+    ops.rms_norm(x, w, 1e-5, out)
+    want = w.double() * (x.double() * torch.rsqrt((x.double() ** 2).mean(-1, keepdim=True) + 1e-5))
+    torch.testing.assert_close(out.double(), want, **tol(dtype))
+    # with the residual sum fused, and rows gathered
+    delta = torch.randn(9, H, generator=g).to(dtype).to(DEV)
+    x2 = x.clone()
+    ops.rms_norm(x2, w, 1e-5, out, delta=delta)
+    s = x.double() + delta.double()
+    torch.testing.assert_close(x2.double(), s, atol=1e-6, rtol=1e-6)
+    want = w.double() * (s * torch.rsqrt((s ** 2).mean(-1, keepdim=True) + 1e-5))
+    torch.testing.assert_close(out.double(), want, **tol(dtype))
+    rows = torch.tensor([7, 0, 3], dtype=torch.int32, device=DEV)
+    out3 = torch.empty(3, H, dtype=dtype, device=DEV)
+    ops.rms_norm(x2, w, 1e-5, out3, rows=rows)
+    torch.testing.assert_close(out3.double(), want[rows.long()], **tol(dtype))
+
+
+def test_rms_norm_eps_inside_root(ops):
+    x = torch.full((1, 16), 1e-6, device=DEV)
+    out = torch.empty(1, 16, device=DEV)
+    ops.rms_norm(x, torch.ones(16, device=DEV), 1e-2, out)
+    torch.testing.assert_close(out, x / math.sqrt(1e-12 + 1e-2), rtol=1e-6, atol=0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_silu_mul(ops, dtype):
+    g = torch.Generator().manual_seed(2)
+    gu = (torch.randn(7, 2 * 200, generator=g) * 2).to(dtype).to(DEV)
+    out = torch.empty(7, 200, dtype=dtype, device=DEV)
+    ops.silu_mul(gu, out)
+    a = gu.double()
+    want = torch.nn.functional.silu(a[:, :200]) * a[:, 200:]
+    torch.testing.assert_close(out.double(), want, **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(1, 331, 72), (5, 64, 120), (70, 200, 896), (130, 151, 50), (3, 1000, 4864)])
+def test_gemm_generic(ops, dtype, M, N, K):
+    g = torch.Generator().manual_seed(3)
+    a = torch.randn(M, K, generator=g).to(dtype).to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(dtype).to(DEV)
+    bias = torch.randn(N, generator=g).to(DEV)
+    want = a.double() @ w.double().T
+    out = torch.empty(M, N, dtype=dtype, device=DEV)
+    ops.gemm_generic(a, w, out)
+    torch.testing.assert_close(out.double(), want, **tol(dtype))
+    ops.gemm_generic(a, w, out, bias=bias)
+    torch.testing.assert_close(out.double(), want + bias.double(), **tol(dtype))
+    acc = torch.randn(M, N, generator=g).to(DEV)
+    acc0 = acc.clone()
+    ops.gemm_generic(a, w, acc, accumulate=True)  # float result whatever the inputs are
+    torch.testing.assert_close(acc.double(), acc0.double() + want, atol=2e-5, rtol=2e-5)
+
+
+def test_gemm_row_does_not_depend_on_the_batch(ops):
+    g = torch.Generator().manual_seed(4)
+    a = torch.randn(77, 192, generator=g).to(DEV)
+    w = torch.randn(331, 192, generator=g).to(DEV)
+    full = torch.empty(77, 331, device=DEV)
+    one = torch.empty(1, 331, device=DEV)
+    ops.gemm_generic(a, w, full)
+    ops.gemm_generic(a[40:41], w, one)
+    assert torch.equal(full[40:41], one)
+
+
+def rope_reference(x, pos, rot, inv):
+    ang = pos.double()[:, None] * inv[None]
+    cos, sin = torch.cat((ang, ang), -1).cos()[:, None], torch.cat((ang, ang), -1).sin()[:, None]
+    xr = x[..., :rot]
+    half = rot // 2
+    rotated = xr * cos + torch.cat((-xr[..., half:], xr[..., :half]), -1) * sin
+    return torch.cat((rotated, x[..., rot:]), -1)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,rot", [(4, 2, 16, 16), (5, 1, 48, 48), (6, 3, 80, 32)])
+def test_rope_store(ops, dtype, nh, nkv, d, rot):
+    g = torch.Generator().manual_seed(5)
+    N, page_size, pages = 11, 4, 9
+    qkv = torch.randn(N, (nh + 2 * nkv) * d, generator=g).to(dtype)
+    pos = torch.tensor([0, 1, 2, 3, 8191, 5, 100, 7, 4000, 9, 10], dtype=torch.int32)
+    slots = torch.randperm(pages * page_size, generator=g)[:N].to(torch.int32)
+    slots[3] = -1
+    theta = 1e6
+    inv_freq = (1.0 / (theta ** (torch.arange(0, rot, 2, dtype=torch.float64) / rot))).float()
+    kp = torch.zeros(pages, nkv, page_size, d, dtype=dtype, device=DEV)
+    vp = torch.zeros_like(kp)
+    dev = qkv.to(DEV)
+    ops.rope_store(dev, nh, nkv, d, rot, pos.to(DEV), inv_freq.to(DEV), slots.to(DEV), kp, vp)
+    x = qkv.double().view(N, nh + 2 * nkv, d)
+    want_q = rope_reference(x[:, :nh], pos, rot, inv_freq.double())
+    want_k = rope_reference(x[:, nh:nh + nkv], pos, rot, inv_freq.double())
+    got = dev.double().cpu().view(N, nh + 2 * nkv, d)
+    # the angle is a float product of position and frequency: at position 8191 its rounding is ~2.4e-4 rad
+    t = dict(atol=2e-3, rtol=0) if dtype == torch.float32 else dict(atol=3e-2, rtol=1.6e-2)
+    torch.testing.assert_close(got[:, :nh], want_q, **t)
+    torch.testing.assert_close(got[:, nh:nh + nkv], want_k, **t)
+    small = pos < 200  # there the float angle is exact to ~1e-5
+    torch.testing.assert_close(got[small][:, :nh], want_q[small], **tol(dtype))
+    assert torch.equal(got[:, nh + nkv:], x[:, nh + nkv:])
+    for n in range(N):
+        s = int(slots[n])
+        if s < 0:
+            continue
+        p, o = divmod(s, page_size)
+        assert torch.equal(kp[p, :, o].cpu().double(), got[n, nh:nh + nkv])
+        assert torch.equal(vp[p, :, o].cpu().double(), x[n, nh + nkv:])
+    used = torch.zeros(pages * page_size, dtype=torch.bool)
+    used[slots[slots >= 0].long()] = True
+    assert (kp.cpu().permute(0, 2, 1, 3).reshape(pages * page_size, -1)[~used] == 0).all()
+
+
+def attention_reference(q, k, v, scale, window=None):
+    """q [nh, T, d], k/v [nkv, S, d] with the T queries at the last T of S positions."""
+    nh, T, d = q.shape
+    S = k.shape[1]
+    rep = nh // k.shape[0]
+    k, v = k.repeat_interleave(rep, 0), v.repeat_interleave(rep, 0)
+    s = torch.einsum("htd,hsd->hts", q, k) * scale
+    i = torch.arange(S - T, S)[:, None]
+    j = torch.arange(S)[None]
+    vis = j <= i
+    if window:
+        vis = vis & (j > i - window)
+    s = s.masked_fill(~vis[None], float("-inf"))
+    return torch.einsum("hts,hsd->htd", s.softmax(-1), v)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("nh,nkv,d,page_size,window", [(4, 2, 16, 4, None), (6, 2, 32, 8, None), (5, 1, 48, 16, None),
+                                                        (3, 3, 80, 4, 7), (8, 2, 128, 16, 40)])
+def test_paged_attention_generic(ops, dtype, nh, nkv, d, page_size, window):
+    """Three requests in one batch: a whole prompt, a portion after a cached prefix, one decoded token;
+    pages handed out in shuffled order and the pool pre-filled with large values that must never be read."""
+    g = torch.Generator().manual_seed(6)
+    ctx = [70, 133, 201]       # keys each request holds after this step
+    qlen = [70, 9, 1]          # its new tokens
+    pages_per = [-(-c // page_size) for c in ctx]
+    P = sum(pages_per) + 5
+    order = torch.randperm(P - 1, generator=g) + 1
+    kp = torch.full((P, nkv, page_size, d), 1e4, dtype=dtype)
+    vp = torch.full((P, nkv, page_size, d), -1e4, dtype=dtype)
+    table = torch.zeros(3, max(pages_per), dtype=torch.int32)
+    scale = 1.0 / math.sqrt(d)
+    q_all, req_all, pos_all, want = [], [], [], []
+    used = 0
+    for r in range(3):
+        k = torch.randn(nkv, ctx[r], d, generator=g).to(dtype)
+        v = torch.randn(nkv, ctx[r], d, generator=g).to(dtype)
+        q = (torch.randn(nh, qlen[r], d, generator=g) * 2).to(dtype)
+        # one far key stands out for the last query of each request
+        far = 3
+        k[:, far] = (q[::nh // nkv, -1].float() * 1.5).to(dtype)
+        pages = order[used:used + pages_per[r]]
+        used += pages_per[r]
+        table[r, :pages_per[r]] = pages.to(torch.int32)
+        for j in range(ctx[r]):
+            kp[pages[j // page_size], :, j % page_size] = k[:, j]
+            vp[pages[j // page_size], :, j % page_size] = v[:, j]
+        q_all.append(q.transpose(0, 1).reshape(qlen[r], nh * d))
+        req_all += [r] * qlen[r]
+        pos_all += list(range(ctx[r] - qlen[r], ctx[r]))
+        want.append(attention_reference(q.double(), k.double(), v.double(), scale, window).transpose(0, 1).reshape(qlen[r], nh * d))
+    q = torch.cat(q_all).to(DEV)
+    N = q.shape[0]
+    # q as a row slice of a wider matrix, as in the fused projection
+    wide = torch.zeros(N, nh * d + 24, dtype=dtype, device=DEV)
+    wide[:, :nh * d] = q
+    out = torch.empty(N, nh * d, dtype=dtype, device=DEV)
+    ops.paged_attention_generic(wide, kp.to(DEV), vp.to(DEV), table.to(DEV),
+                                torch.tensor(req_all, dtype=torch.int32, device=DEV),
+                                torch.tensor(pos_all, dtype=torch.int32, device=DEV), out, nh, scale, window)
+    torch.testing.assert_close(out.double().cpu(), torch.cat(want), **tol(dtype))
+
+
+def test_sample_greedy_and_vectors(ops):
+    lg = torch.tensor([[0.1, 2.0, 0.5], [3.0, 0.0, 0.0], [1.0, 1.0, 1.0]], device=DEV)
+    out = torch.empty(3, dtype=torch.int32, device=DEV)
+    ops.sample(lg, out)
+    assert out.tolist() == [1, 0, 0]  # first maximum on ties
+    g = torch.Generator().manual_seed(7)
+    big = torch.randn(5, 151936, generator=g).to(DEV)
+    out = torch.empty(5, dtype=torch.int32, device=DEV)
+    ops.sample(big, out)
+    assert out.tolist() == big.argmax(-1).tolist()
+
+
+def _draws(ops, logits, n, temperature=1.0, top_k=0, top_p=1.0, seed=0):
+    M = n
+    lg = logits.to(DEV).expand(M, -1).contiguous()
+    out = torch.empty(M, dtype=torch.int32, device=DEV)
+    ops.sample(lg, out, torch.full((M,), temperature, device=DEV), torch.full((M,), top_k, dtype=torch.int32, device=DEV),
+               torch.full((M,), top_p, device=DEV), torch.full((M,), seed, dtype=torch.int64, device=DEV),
+               torch.arange(M, dtype=torch.int32, device=DEV))
+    return out.cpu()
+
+
+def test_sample_distribution_and_filters(ops):
+    # vectors of the reference's tests/test_sampler.py
+    assert set(_draws(ops, torch.tensor([[0.1, 2.0, 0.5]]), 20, top_k=1).tolist()) == {1}
+    assert set(_draws(ops, torch.tensor([[2.0, 1.0, 0.0, -1.0]]), 300, top_p=0.7).tolist()) == {0, 1}
+    assert set(_draws(ops, torch.tensor([[10.0, 0.0, 0.0]]), 50, top_p=1e-4).tolist()) == {0}
+    d = _draws(ops, torch.log(torch.tensor([[0.7, 0.2, 0.1]])), 4000, seed=123)
+    freq = torch.bincount(d, minlength=3).float() / 4000
+    assert torch.allclose(freq, torch.tensor([0.7, 0.2, 0.1]), atol=0.03)
+    # temperature sharpens: T = 0.5 squares the odds
+    d = _draws(ops, torch.log(torch.tensor([[0.5, 0.5 / 3]])), 4000, temperature=0.5, seed=5)
+    assert abs((d == 0).float().mean().item() - 0.9) < 0.03
+    # same seed and draw index, same token; top-k = 2 on a wide row leaves two tokens
+    row = torch.randn(1, 5000, generator=torch.Generator().manual_seed(8))
+    a, b = _draws(ops, row, 64, seed=9), _draws(ops, row, 64, seed=9)
+    assert torch.equal(a, b) and len(set(a.tolist())) > 10
+    top2 = set(row[0].topk(2).indices.tolist())
+    assert set(_draws(ops, row, 200, top_k=2, seed=1).tolist()) == top2
+
+
+def test_ops_refuse_cpu_tensors_and_wrong_shapes(ops):
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        ops.silu_mul(torch.zeros(2, 4), torch.zeros(2, 2))
+    with pytest.raises(ValueError):
+        ops.silu_mul(torch.zeros(2, 4, device=DEV), torch.zeros(2, 3, device=DEV))
+    with pytest.raises(RuntimeError, match="unsupported"):
+        kp = torch.zeros(2, 1, 4, 6, device=DEV)  # head size 6 is no multiple of 4
+        ops.paged_attention_generic(torch.zeros(1, 6, device=DEV), kp, kp, torch.zeros(1, 1, dtype=torch.int32, device=DEV),
+                                    torch.zeros(1, dtype=torch.int32, device=DEV), torch.zeros(1, dtype=torch.int32, device=DEV),
+                                    torch.zeros(1, 6, device=DEV), 1, 1.0)
