@@ -1,0 +1,89 @@
+"""The step function: run a batch of (request, its next tokens) from the cache and return the logits at
+the wanted places.
+
+One call = one forward of the model over exactly the tokens it is given: it allocates the pages they
+need, writes their keys and values, attends over what earlier steps left, and commits the new lengths.
+The reference's counterpart is ``Qwen2.forward(input_ids, cache=view, last_only)`` called once for a
+prefill and once for the decode rows of a step (src/miniserve/paged_engine.py:126-127, 168-170).
+"""
+from __future__ import annotations
+
+from typing import Hashable, List, Optional
+
+import torch
+
+from ..cache import CacheLayout, CacheManager, CachePools
+from ..config.engine_config import EngineConfig
+from ..parts.base import Runtime
+from ..parts.model import Model, RunCache
+from .batch import BatchBuilder, StepEntry
+
+_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+class ModelRunner:
+    def __init__(self, model: Model, page_size: int, num_pages: int, max_requests: int, max_len: int):
+        if model.rt is None:
+            raise RuntimeError("the model has no weights yet; load it first")
+        self.model, self.rt = model, model.rt
+        self.layout = CacheLayout(model.run_needs())
+        self.manager = CacheManager(self.layout, page_size, num_pages, max_requests, max_len)
+        self.pools = CachePools(self.layout, page_size, num_pages, max_requests, self.rt)
+        self.builder = BatchBuilder(self.manager, model.spec.vocab_size, self.rt.device)
+
+    # ------------------------------------------------------------------ requests
+    def add_request(self, req_id: Hashable) -> None:
+        self.manager.add(req_id)
+
+    def free_request(self, req_id: Hashable) -> None:
+        self.manager.free(req_id)
+
+    # ------------------------------------------------------------------ the step
+    @torch.inference_mode()
+    def step(self, entries: List[StepEntry]) -> torch.Tensor:
+        """Float logits [wanted places, vocabulary], in the order of the entries and of their ``want``."""
+        m = self.manager
+        seen = set()
+        for e in entries:
+            if e.req_id in seen:
+                raise ValueError(f"request {e.req_id!r} appears twice in one step")
+            seen.add(e.req_id)
+            if not m.has(e.req_id):
+                m.add(e.req_id)
+        for e in entries:
+            m.grow(e.req_id, m.computed(e.req_id) + len(e.tokens))
+        ctx, tables, slots = self.builder.build(entries)
+        if self.layout.state_runs:
+            self.pools.zero_state([r for r, s in zip(ctx.state_slots_host, ctx.start_pos_host) if s == 0])
+        caches = []
+        for i in range(len(self.model.spec.order)):
+            g = self.layout.run_group[i]
+            kv = self.pools.kv_view(i, tables[g], slots[g]) if g is not None else None
+            state = self.pools.state_view(i) if i in self.layout.state_needs else None
+            caches.append(RunCache(kv, state))
+        logits = self.model.forward(ctx, caches)
+        for e in entries:
+            m.advance(e.req_id, m.computed(e.req_id) + len(e.tokens))
+        return logits
+
+
+def load_runner(model_dir, dtype: str = "bfloat16", device: str = "cuda:0", page_size: int = 16,
+                num_pages: Optional[int] = None, max_requests: int = 32, max_len: int = 1024) -> ModelRunner:
+    """Model folder -> a runner with an empty cache.  The model class is chosen by config.json."""
+    from ..config import load_config
+    from ..weights import CheckpointReader
+
+    if dtype not in _DTYPES:
+        raise ValueError(f"dtype must be 'bfloat16' or 'float32', got {dtype!r}")
+    dev = torch.device(device)
+    if dev.type != "cuda":
+        raise RuntimeError(f"the engine runs on the GPU only (device {device!r} was asked for); there is no CPU path")
+    if not torch.cuda.is_available():
+        raise RuntimeError("no GPU is visible to this process; the engine has no CPU path")
+    config = load_config(model_dir)
+    model = Model(config.to_spec())
+    model.load(CheckpointReader(model_dir), Runtime(dev, _DTYPES[dtype]))
+    model.config = config
+    if num_pages is None:
+        num_pages = max_requests * (-(-max_len // page_size))
+    return ModelRunner(model, page_size, num_pages, max_requests, max_len)

@@ -229,3 +229,10 @@ def sample(logits: torch.Tensor, out: torch.Tensor, temperature: Optional[torch.
     _call("ms_sample", logits.data_ptr(), V, M, V, _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(seeds),
           _ptr(draw_index), out.data_ptr(), _stream())
     return out
+
+
+def paged_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor, ctx,
+                    out: torch.Tensor, num_heads: int, scale: float, window: Optional[int] = None) -> torch.Tensor:
+    """Attention of a step's tokens (``ctx`` is its StepContext) over the pages; picks the kernel."""
+    return paged_attention_generic(q, k_pages, v_pages, block_table, ctx.token_req, ctx.positions, out, num_heads,
+                                   scale, window)

@@ -1,0 +1,77 @@
+"""Grouped-query attention over the paged cache.
+
+q, k, v projections (one packed matrix product), position encoding fused with the cache store, causal
+attention read in place from the pages, output projection.  Query head h uses key/value head
+h // (num_heads // num_kv_heads) (src/miniserve/model.py:137-139).  Scores, softmax and the weighted
+sum are float.  ``window`` limits a query to the last ``window`` keys (None: all).
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..kernels import linear, ops
+from ..weights.spec import TensorSpec
+from .base import KVNeed, Mixer, register_part
+
+
+class GQAttention(Mixer):
+    def __init__(self, prefix: str, position, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 scale: float, qkv_bias: bool = True, out_bias: bool = False, window: Optional[int] = None):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} query heads cannot share {num_kv_heads} key/value heads")
+        if head_dim % 16 or head_dim > 256:
+            raise ValueError(f"head_dim {head_dim} is not supported: the attention kernels take multiples of 16 up to 256")
+        if window is not None and window <= 0:
+            raise ValueError("window must be positive")
+        self.prefix, self.position = prefix, position
+        self.hidden_size, self.num_heads, self.num_kv_heads, self.head_dim = hidden_size, num_heads, num_kv_heads, head_dim
+        self.scale, self.qkv_bias, self.out_bias, self.window = float(scale), qkv_bias, out_bias, window
+
+    # ---- weights
+    def tensor_specs(self):
+        p, H, d = self.prefix, self.hidden_size, self.head_dim
+        specs = []
+        for name, heads in (("q_proj", self.num_heads), ("k_proj", self.num_kv_heads), ("v_proj", self.num_kv_heads)):
+            specs.append(TensorSpec(f"{p}{name}.weight", (heads * d, H)))
+            if self.qkv_bias:
+                specs.append(TensorSpec(f"{p}{name}.bias", (heads * d,), "bias"))
+        specs.append(TensorSpec(f"{p}o_proj.weight", (H, self.num_heads * d)))
+        if self.out_bias:
+            specs.append(TensorSpec(f"{p}o_proj.bias", (H,), "bias"))
+        return specs
+
+    def load(self, get, rt):
+        self.rt = rt
+        by_name = {s.name: s for s in self.tensor_specs()}
+        p = self.prefix
+        w = [get(by_name[f"{p}{n}.weight"]) for n in ("q_proj", "k_proj", "v_proj")]
+        self.w_qkv = linear.prepare_weight(torch.cat(w, dim=0))
+        self.b_qkv = torch.cat([get(by_name[f"{p}{n}.bias"]) for n in ("q_proj", "k_proj", "v_proj")]).contiguous() \
+            if self.qkv_bias else None
+        self.w_o = linear.prepare_weight(get(by_name[f"{p}o_proj.weight"]))
+        self.b_o = get(by_name[f"{p}o_proj.bias"]) if self.out_bias else None
+        if self.position is not None:
+            self.position.load(get, rt)
+
+    # ---- cache
+    def cache_need(self):
+        return KVNeed(self.num_kv_heads, self.head_dim, self.window)
+
+    # ---- step
+    def forward(self, h, ctx, kv, state):
+        if kv is None:
+            raise RuntimeError("attention needs a key/value cache view")
+        nh, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
+        qkv = linear.linear(h, self.w_qkv, bias=self.b_qkv)
+        if self.position is not None:
+            self.position.encode_and_store(qkv, nh, nkv, d, ctx, kv)
+        elif kv.store:
+            ops.rope_store(qkv, nh, nkv, d, 0, None, None, kv.slot_mapping, kv.k_pages, kv.v_pages)
+        out = self.rt.empty(ctx.num_tokens, nh * d)
+        ops.paged_attention(qkv, kv.k_pages, kv.v_pages, kv.block_table, ctx, out, nh, self.scale, self.window)
+        return linear.linear(out, self.w_o, bias=self.b_o)
+
+
+register_part("mixer", "gqa_attention", GQAttention)

@@ -1,0 +1,208 @@
+"""Interfaces of the parts a model is assembled from, and the registries that name them.
+
+A part is built from the sizes and constants in its ``PartSpec`` alone and never learns which model
+it is in.  Five kinds are chosen layer by layer:
+
+``Norm``              forward(x, delta, rows, write_back) -> activations         (x: the float residual stream)
+``PositionEncoding``  encode_and_store(qkv, nh, nkv, d, ctx, kv)                 (belongs to a mixer)
+``Mixer``             forward(h, ctx, kv, state) -> [N, hidden]                  (attention here)
+``FeedForward``       forward(h, ctx) -> [N, hidden]
+``Block``             forward(x, pending, ctx, kv, state) -> pending             (the arrangement of the four)
+
+plus ``Embedding`` and ``Head`` at the model's ends.  Every part lists the checkpoint tensors it wants
+(``tensor_specs``) and takes them in ``load``.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Callable, Dict, List, Optional, Tuple
+
+import torch
+
+from ..weights.spec import TensorSpec
+
+
+# ------------------------------------------------------------------------------------------------ runtime data
+@dataclass
+class Runtime:
+    """Where a model lives and the type of its matrices and activations."""
+
+    device: torch.device
+    dtype: torch.dtype
+
+    def empty(self, *shape, dtype=None) -> torch.Tensor:
+        return torch.empty(shape, dtype=dtype or self.dtype, device=self.device)
+
+
+@dataclass(frozen=True)
+class KVNeed:
+    """A mixer that keeps keys and values: pages of [num_kv_heads, page_size, head_dim], all keys of a
+    request (``window`` None) or the last ``window`` of them."""
+
+    num_kv_heads: int
+    head_dim: int
+    window: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """A mixer that keeps state of fixed size per request: one tensor of ``shape`` and ``dtype`` in a slot
+    that the request holds from admission to its end.  The slot is zero when the request's first portion runs."""
+
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass
+class KVView:
+    """One run's pages of its cache group, with the group's tables for the step's requests."""
+
+    k_pages: torch.Tensor      # [pages, nkv, page_size, d]
+    v_pages: torch.Tensor
+    block_table: torch.Tensor  # int32 [R, max pages]
+    slot_mapping: torch.Tensor  # int32 [N]: page * page_size + offset of each token
+    store: bool = True         # False: the run reads another run's cache and writes nothing
+    window: Optional[int] = None
+
+
+@dataclass
+class StateView:
+    """One run's state slots: ``slots[state_slots[r]]`` belongs to request row r of the step."""
+
+    slots: torch.Tensor        # [num_slots, *shape]
+
+
+@dataclass
+class StepContext:
+    """Everything a step's kernels need to know about its batch: N tokens of R requests, flattened.
+    Device tensors are int32.  A request's tokens are consecutive; token n of request row r has absolute
+    position ``positions[n]`` and sees the keys 0..positions[n] of that request."""
+
+    num_tokens: int
+    num_requests: int
+    token_ids: torch.Tensor      # [N]
+    positions: torch.Tensor      # [N]
+    token_req: torch.Tensor      # [N] request row of each token
+    q_start: torch.Tensor        # [R + 1] first token of each request's portion
+    context_lens: torch.Tensor   # [R] keys each request holds once this step's tokens are stored
+    state_slots: torch.Tensor    # [R] slot of each request's fixed-size state
+    logit_rows: torch.Tensor     # [M] tokens whose logits are wanted
+    max_q_len: int = 0
+    max_context_len: int = 0
+    # host copies for parts written in plain tensor code (tests' toy parts) and for kernel choice
+    q_lens_host: List[int] = field(default_factory=list)
+    start_pos_host: List[int] = field(default_factory=list)
+    state_slots_host: List[int] = field(default_factory=list)
+
+    @property
+    def decode_only(self) -> bool:
+        return self.max_q_len == 1
+
+
+# ------------------------------------------------------------------------------------------------ part interfaces
+Getter = Callable[[TensorSpec], torch.Tensor]
+
+
+class Part:
+    def tensor_specs(self) -> List[TensorSpec]:
+        return []
+
+    def load(self, get: Getter, rt: Runtime) -> None:
+        """Take the tensors listed by ``tensor_specs`` (``get`` returns them placed on the device)."""
+        self.rt = rt
+
+
+class Norm(Part):
+    def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor] = None,
+                rows: Optional[torch.Tensor] = None, write_back: bool = True) -> torch.Tensor:
+        """Normalised activations of the float residual stream ``x`` [N, H].  With ``delta`` the sum
+        x + delta is formed first (and kept in x unless ``write_back`` is False); with ``rows`` only
+        those rows are produced."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def encode_and_store(self, qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
+                         ctx: StepContext, kv: Optional[KVView]) -> None:
+        """Encode positions into the q and k parts of ``qkv`` [N, (nh + 2 nkv) d] in place and, if ``kv``
+        stores, put k and v into its pages."""
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def cache_need(self) -> Optional[KVNeed]:
+        return None
+
+    def state_need(self) -> Optional[StateNeed]:
+        return None
+
+    def forward(self, h: torch.Tensor, ctx: StepContext, kv: Optional[KVView],
+                state: Optional[StateView]) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, h: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block(Part):
+    """The arrangement of a layer's parts.  ``pending`` is an addend of the residual stream that the
+    previous layer left unsummed so that the next norm can fuse the sum; a block returns its own."""
+
+    def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm, feed_forward_norm: Norm):
+        self.mixer, self.feed_forward = mixer, feed_forward
+        self.mixer_norm, self.feed_forward_norm = mixer_norm, feed_forward_norm
+
+    def parts(self) -> List[Part]:
+        return [self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward]
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [s for p in self.parts() for s in p.tensor_specs()]
+
+    def load(self, get: Getter, rt: Runtime) -> None:
+        self.rt = rt
+        for p in self.parts():
+            p.load(get, rt)
+
+    def forward(self, x: torch.Tensor, pending: Optional[torch.Tensor], ctx: StepContext,
+                kv: Optional[KVView], state: Optional[StateView]) -> Optional[torch.Tensor]:
+        raise NotImplementedError
+
+
+class Embedding(Part):
+    def forward(self, ctx: StepContext) -> torch.Tensor:
+        """The float residual stream [N, H] of the step's tokens."""
+        raise NotImplementedError
+
+
+class Head(Part):
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        """Float logits [M, V] of normalised rows h [M, H]."""
+        raise NotImplementedError
+
+
+# ------------------------------------------------------------------------------------------------ registries
+_REGISTRIES: Dict[str, Dict[str, type]] = {
+    "norm": {}, "position": {}, "mixer": {}, "feed_forward": {}, "block": {}, "embedding": {}, "head": {},
+}
+
+
+def register_part(category: str, kind: str, cls: type) -> type:
+    """Make ``cls`` buildable from ``PartSpec(kind=...)``.  Its constructor takes ``prefix`` and the spec's
+    params as keywords (a mixer also ``position``, a built PositionEncoding or None)."""
+    if category not in _REGISTRIES:
+        raise KeyError(f"no part category {category!r}; there are {sorted(_REGISTRIES)}")
+    _REGISTRIES[category][kind] = cls
+    return cls
+
+
+def part_class(category: str, kind: str) -> type:
+    reg = _REGISTRIES[category]
+    if kind not in reg:
+        raise KeyError(f"no {category} part named {kind!r}; registered: {sorted(reg)}")
+    return reg[kind]
+
+
+def build_part(category: str, spec, **extra):
+    return part_class(category, spec.kind)(prefix=spec.prefix, **dict(spec.params), **extra)

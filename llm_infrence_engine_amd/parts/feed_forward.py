@@ -1,0 +1,34 @@
+"""Dense gated feed-forward: down(silu(gate(x)) * up(x)), no biases (src/miniserve/model.py:155-165).
+Gate and up are one packed matrix product; the activation is float."""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import linear, ops
+from ..weights.spec import TensorSpec
+from .base import FeedForward, register_part
+
+
+class SwiGLU(FeedForward):
+    def __init__(self, prefix: str, hidden_size: int, intermediate_size: int):
+        self.prefix, self.hidden_size, self.intermediate_size = prefix, hidden_size, intermediate_size
+
+    def tensor_specs(self):
+        p, H, I = self.prefix, self.hidden_size, self.intermediate_size
+        return [TensorSpec(p + "gate_proj.weight", (I, H)), TensorSpec(p + "up_proj.weight", (I, H)),
+                TensorSpec(p + "down_proj.weight", (H, I))]
+
+    def load(self, get, rt):
+        self.rt = rt
+        g, u, d = (get(s) for s in self.tensor_specs())
+        self.w_gate_up = linear.prepare_weight(torch.cat((g, u), dim=0))
+        self.w_down = linear.prepare_weight(d)
+
+    def forward(self, h, ctx):
+        gu = linear.linear(h, self.w_gate_up)
+        act = self.rt.empty(h.shape[0], self.intermediate_size)
+        ops.silu_mul(gu, act)
+        return linear.linear(act, self.w_down)
+
+
+register_part("feed_forward", "swiglu", SwiGLU)

@@ -1,0 +1,96 @@
+"""A model assembled from a ``ModelSpec``: embedding, layers in the order the spec gives, final norm, head.
+
+The same layer may run more than once and a run may read an earlier run's cache; each run that keeps a
+cache of its own is one entry of the cache manager's groups.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional
+
+import torch
+
+from ..config.spec import ModelSpec
+from ..weights.reader import CheckpointReader, place
+from ..weights.spec import TensorSpec
+from . import attention, blocks, ends, feed_forward, norms, positions  # noqa: F401  (register the built-in parts)
+from .base import KVView, Runtime, StateView, StepContext, build_part, part_class
+
+
+@dataclass
+class RunCache:
+    """What one run of a layer was given by the cache manager for this step."""
+
+    kv: Optional[KVView] = None
+    state: Optional[StateView] = None
+
+
+class Model:
+    def __init__(self, spec: ModelSpec):
+        self.spec = spec
+        self.embedding = build_part("embedding", spec.embedding)
+        self.layers = []
+        for ls in spec.layers:
+            position = build_part("position", ls.position) if ls.position is not None else None
+            mixer = build_part("mixer", ls.mixer, position=position)
+            ff = build_part("feed_forward", ls.feed_forward)
+            n1 = build_part("norm", ls.mixer_norm)
+            n2 = build_part("norm", ls.feed_forward_norm)
+            self.layers.append(part_class("block", ls.block)(mixer, ff, n1, n2))
+        self.final_norm = build_part("norm", spec.final_norm)
+        self.head = build_part("head", spec.head)
+        self.rt: Optional[Runtime] = None
+
+    # ------------------------------------------------------------------ weights
+    def _parts(self):
+        return [self.embedding, *self.layers, self.final_norm, self.head]
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        """Every tensor the model wants, each name once (a tied head names the embedding's)."""
+        seen, out = set(), []
+        for p in self._parts():
+            for s in p.tensor_specs():
+                if s.name not in seen:
+                    seen.add(s.name)
+                    out.append(s)
+        return out
+
+    def ignorable_tensors(self) -> List[str]:
+        return list(getattr(self.head, "ignorable", lambda: [])())
+
+    def load(self, reader: CheckpointReader, rt: Runtime) -> "Model":
+        reader.check(self.tensor_specs(), self.ignorable_tensors())
+        placed: Dict[str, torch.Tensor] = {}
+
+        def get(spec: TensorSpec) -> torch.Tensor:
+            if spec.name not in placed:
+                placed[spec.name] = place(reader.get(spec.name), spec, rt.dtype, rt.device)
+            return placed[spec.name]
+
+        for p in self._parts():
+            p.load(get, rt)
+        self.rt = rt
+        reader.close()
+        return self
+
+    # ------------------------------------------------------------------ cache needs, run by run
+    def run_needs(self):
+        """For every entry of the order: (KVNeed or None, StateNeed or None, cache_of)."""
+        out = []
+        for run in self.spec.order:
+            mixer = self.layers[run.layer].mixer
+            out.append((mixer.cache_need(), mixer.state_need(), run.cache_of))
+        return out
+
+    # ------------------------------------------------------------------ one step
+    def forward(self, ctx: StepContext, caches: List[RunCache]) -> torch.Tensor:
+        """Float logits [M, V] at ``ctx.logit_rows``.  Runs only the step's tokens, from the cache."""
+        x = self.embedding.forward(ctx)
+        pending = None
+        for i, run in enumerate(self.spec.order):
+            c = caches[i]
+            pending = self.layers[run.layer].forward(x, pending, ctx, c.kv, c.state)
+        if ctx.logit_rows.numel() == 0:
+            return torch.empty(0, self.spec.vocab_size, dtype=torch.float32, device=x.device)
+        h = self.final_norm.forward(x, delta=pending, rows=ctx.logit_rows, write_back=False)
+        return self.head.forward(h)

@@ -1,0 +1,47 @@
+"""Rotary position encoding with half-split pairing.
+
+inv_freq[j] = theta^(-2j/rotary_dim); the pair (j, j + rotary_dim/2) of every q and k head turns by
+position * inv_freq[j] (src/miniserve/model.py:83-98).  Angles, sines and cosines are float in every
+mode; the frequencies are derived in double on the host and rounded once.  The rotation is fused with
+the store of k and v into the cache pages.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from .base import PositionEncoding, register_part
+
+
+class RotaryHalf(PositionEncoding):
+    def __init__(self, prefix: str, head_dim: int, rotary_dim: int, theta: float):
+        if rotary_dim % 2 or not 0 < rotary_dim <= head_dim:
+            raise ValueError(f"rotary_dim {rotary_dim} must be even and within head_dim {head_dim}")
+        self.head_dim, self.rotary_dim, self.theta = head_dim, rotary_dim, float(theta)
+
+    def load(self, get, rt):
+        self.rt = rt
+        j = torch.arange(0, self.rotary_dim, 2, dtype=torch.float64)
+        self.inv_freq = (1.0 / (self.theta ** (j / self.rotary_dim))).to(torch.float32).to(rt.device)
+
+    def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, ctx, kv):
+        store = kv is not None and kv.store
+        ops.rope_store(qkv, num_heads, num_kv_heads, head_dim, self.rotary_dim, ctx.positions, self.inv_freq,
+                       kv.slot_mapping if store else None, kv.k_pages if store else None,
+                       kv.v_pages if store else None)
+
+
+class NoPosition(PositionEncoding):
+    """No encoding: k and v are stored as they are."""
+
+    def __init__(self, prefix: str = ""):
+        pass
+
+    def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, ctx, kv):
+        if kv is not None and kv.store:
+            ops.rope_store(qkv, num_heads, num_kv_heads, head_dim, 0, None, None, kv.slot_mapping, kv.k_pages,
+                           kv.v_pages)
+
+
+register_part("position", "rotary_half", RotaryHalf)
+register_part("position", "none", NoPosition)

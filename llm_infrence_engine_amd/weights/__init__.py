@@ -1,0 +1,5 @@
+from .random_init import random_tensors, write_random_model
+from .reader import CheckpointReader, WeightsError, place
+from .spec import TensorSpec
+
+__all__ = ["CheckpointReader", "WeightsError", "TensorSpec", "place", "random_tensors", "write_random_model"]

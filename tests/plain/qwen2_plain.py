@@ -50,6 +50,13 @@ def read_weights(model_dir, dtype=torch.float64) -> dict:
     return out
 
 
+# --------------------------------------------------------------------------- rounding
+def rounded(x: torch.Tensor, act_dtype) -> torch.Tensor:
+    """x as an engine that stores activations in ``act_dtype`` would hold it (None: exact).  Used only to
+    measure how far a faithful reduced-precision computation strays from the exact one."""
+    return x if act_dtype is None else x.to(act_dtype).to(x.dtype)
+
+
 # --------------------------------------------------------------------------- parts
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     """x * rsqrt(mean(x^2) + eps) * weight; eps inside the root (src/miniserve/model.py:69-73)."""
@@ -106,7 +113,7 @@ def causal_attention(q, k, v, window=None) -> torch.Tensor:
     return torch.einsum("hts,hsd->htd", torch.softmax(scores, dim=-1), v)
 
 
-def attention_block(x, w, prefix, cfg, cos, sin) -> torch.Tensor:
+def attention_block(x, w, prefix, cfg, cos, sin, act_dtype=None) -> torch.Tensor:
     """Projections with q/k/v bias, rotation of q and k, attention, output projection without bias
     (src/miniserve/model.py:121-152)."""
     T = x.shape[0]
@@ -114,37 +121,42 @@ def attention_block(x, w, prefix, cfg, cos, sin) -> torch.Tensor:
     q = x @ w[prefix + "q_proj.weight"].T + w[prefix + "q_proj.bias"]
     k = x @ w[prefix + "k_proj.weight"].T + w[prefix + "k_proj.bias"]
     v = x @ w[prefix + "v_proj.weight"].T + w[prefix + "v_proj.bias"]
-    q = q.view(T, nh, d).transpose(0, 1)
-    k = k.view(T, nkv, d).transpose(0, 1)
-    v = v.view(T, nkv, d).transpose(0, 1)
-    q = apply_rope(q, cos, sin)
-    k = apply_rope(k, cos, sin)
-    out = causal_attention(q, k, v)
+    q = rounded(q, act_dtype).view(T, nh, d).transpose(0, 1)
+    k = rounded(k, act_dtype).view(T, nkv, d).transpose(0, 1)
+    v = rounded(v, act_dtype).view(T, nkv, d).transpose(0, 1)
+    q = rounded(apply_rope(q, cos, sin), act_dtype)
+    k = rounded(apply_rope(k, cos, sin), act_dtype)
+    out = rounded(causal_attention(q, k, v), act_dtype)
     out = out.transpose(0, 1).reshape(T, nh * d)
-    return out @ w[prefix + "o_proj.weight"].T
+    return rounded(out @ w[prefix + "o_proj.weight"].T, act_dtype)
 
 
-def swiglu_mlp(x, w, prefix) -> torch.Tensor:
+def swiglu_mlp(x, w, prefix, act_dtype=None) -> torch.Tensor:
     """down(silu(gate(x)) * up(x)), no biases (src/miniserve/model.py:164-165)."""
-    g = x @ w[prefix + "gate_proj.weight"].T
-    u = x @ w[prefix + "up_proj.weight"].T
-    return (g * torch.sigmoid(g) * u) @ w[prefix + "down_proj.weight"].T
+    g = rounded(x @ w[prefix + "gate_proj.weight"].T, act_dtype)
+    u = rounded(x @ w[prefix + "up_proj.weight"].T, act_dtype)
+    return rounded(rounded(g * torch.sigmoid(g) * u, act_dtype) @ w[prefix + "down_proj.weight"].T, act_dtype)
 
 
-def decoder_layer(x, w, i, cfg, cos, sin) -> torch.Tensor:
+def decoder_layer(x, w, i, cfg, cos, sin, act_dtype=None) -> torch.Tensor:
     """Two pre-norm residual branches (src/miniserve/model.py:184-185)."""
     p = f"model.layers.{i}."
     eps = cfg["rms_norm_eps"]
-    x = x + attention_block(rms_norm(x, w[p + "input_layernorm.weight"], eps), w, p + "self_attn.", cfg, cos, sin)
-    x = x + swiglu_mlp(rms_norm(x, w[p + "post_attention_layernorm.weight"], eps), w, p + "mlp.")
+    h = rounded(rms_norm(x, w[p + "input_layernorm.weight"], eps), act_dtype)
+    x = x + attention_block(h, w, p + "self_attn.", cfg, cos, sin, act_dtype)
+    h = rounded(rms_norm(x, w[p + "post_attention_layernorm.weight"], eps), act_dtype)
+    x = x + swiglu_mlp(h, w, p + "mlp.", act_dtype)
     return x
 
 
-def forward(w: dict, cfg: dict, token_ids, position_offset: int = 0) -> torch.Tensor:
+def forward(w: dict, cfg: dict, token_ids, position_offset: int = 0, act_dtype=None) -> torch.Tensor:
     """Logits [T, V] of one whole sequence (src/miniserve/model.py:222-237).
 
     ``position_offset`` shifts every position by a constant; the reference always starts at 0,
     the offset exists for the invariance test (only distances between positions matter).
+    ``act_dtype`` (None: exact) rounds every activation that a reduced-precision engine stores between two
+    kernels to that type, leaving the residual stream and the logits alone: a measure of the noise such an
+    engine cannot avoid, never an expected value.
     """
     dtype = w["model.embed_tokens.weight"].dtype
     ids = torch.as_tensor(token_ids, dtype=torch.long)
@@ -152,8 +164,8 @@ def forward(w: dict, cfg: dict, token_ids, position_offset: int = 0) -> torch.Te
     x = w["model.embed_tokens.weight"][ids]
     cos, sin = rope_cos_sin(positions, cfg["head_dim"], cfg["rope_theta"], dtype)
     for i in range(cfg["num_layers"]):
-        x = decoder_layer(x, w, i, cfg, cos, sin)
-    x = rms_norm(x, w["model.norm.weight"], cfg["rms_norm_eps"])
+        x = decoder_layer(x, w, i, cfg, cos, sin, act_dtype)
+    x = rounded(rms_norm(x, w["model.norm.weight"], cfg["rms_norm_eps"]), act_dtype)
     head = w["model.embed_tokens.weight"] if cfg["tie_word_embeddings"] else w["lm_head.weight"]
     return x @ head.T
 
