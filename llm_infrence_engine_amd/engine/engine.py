@@ -1,0 +1,163 @@
+"""The serving loop: scheduler above, step function below, sampler beside.
+
+Public face after the reference's ``Engine`` / ``PagedEngine`` (src/miniserve/engine.py:94-205,
+src/miniserve/paged_engine.py:24-80): ``add_request``, ``has_work``, ``cancel``, ``step``,
+``run_until_idle``, ``finished``, ``steps``, ``stats``; and ``generate`` after
+src/miniserve/generate.py:85-135.
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+from typing import Callable, List, Optional, Sequence
+
+import torch
+
+from ..config.engine_config import EngineConfig
+from ..parts.model import Model
+from ..sampling import Sampler
+from .batch import StepEntry
+from .request import Request, StepRecord
+from .runner import ModelRunner
+from .scheduler import Scheduler
+
+
+class Engine:
+    def __init__(self, model: Model, num_blocks: Optional[int] = None, block_size: int = 16, max_seqs: int = 32,
+                 max_len: int = 1024, max_num_batched_tokens: int = 2048, max_prefill_chunk: Optional[int] = None,
+                 on_token: Optional[Callable[[Request, int], None]] = None,
+                 on_finish: Optional[Callable[[Request], None]] = None,
+                 clock: Callable[[], float] = time.perf_counter, hip_graphs: bool = False):
+        dtype = {torch.float32: "float32", torch.bfloat16: "bfloat16"}[model.rt.dtype]
+        self.config = EngineConfig(dtype=dtype, block_size=block_size, num_blocks=num_blocks, max_seqs=max_seqs,
+                                   max_len=max_len, max_num_batched_tokens=max_num_batched_tokens,
+                                   max_prefill_chunk=max_prefill_chunk, hip_graphs=hip_graphs,
+                                   device=str(model.rt.device))
+        self.model = model
+        self.runner = ModelRunner(model, block_size, self.config.resolved_num_blocks(), max_seqs, max_len)
+        self.scheduler = Scheduler(self.runner.manager, self.config, clock, on_token, on_finish)
+        self.sampler = Sampler(model.rt.device)
+        self.clock = clock
+        self.steps: List[StepRecord] = []
+        self.peak_running = 0
+        self.peak_pages_in_use = 0
+        self.prefill_tokens_computed = 0
+
+    # ------------------------------------------------------------------ the reference's public face
+    def add_request(self, req: Request) -> Request:
+        vocab = self.model.spec.vocab_size
+        for t in req.prompt_ids:
+            if not 0 <= t < vocab:
+                raise ValueError(f"token id {t} is outside the vocabulary of {vocab}")
+        return self.scheduler.add_request(req)
+
+    def has_work(self) -> bool:
+        return self.scheduler.has_work()
+
+    def cancel(self, req: Request) -> None:
+        self.scheduler.cancel(req)
+
+    @property
+    def finished(self) -> List[Request]:
+        return self.scheduler.finished
+
+    @property
+    def running(self) -> List[Request]:
+        return self.scheduler.running
+
+    @property
+    def waiting(self):
+        return self.scheduler.waiting
+
+    @property
+    def preemptions(self) -> int:
+        return self.scheduler.preemptions
+
+    def step(self) -> StepRecord:
+        t0 = self.clock()
+        sched = self.scheduler.schedule()
+        useful = 0
+        if not sched and self.scheduler.has_work():
+            raise RuntimeError("the scheduler could place no request although work is waiting")
+        if sched:
+            entries, rows = [], []
+            for s in sched:
+                toks = s.request.tokens[s.start:s.start + s.count]
+                entries.append(StepEntry(s.request.id, toks, [s.count - 1] if s.sample else []))
+                if s.sample:
+                    rows.append(s.request)
+            logits = self.runner.step(entries)
+            useful = self.scheduler.commit(sched, self.sampler.sample(logits, rows))
+        n_decode = sum(1 for s in sched if s.count == 1 and s.start > 0)
+        n_prefill = sum(s.count for s in sched) - n_decode
+        self.prefill_tokens_computed += n_prefill
+        self.peak_running = max(self.peak_running, len(self.scheduler.running))
+        in_use = max((g.allocator.num_in_use() for g in self.runner.manager.groups), default=0)
+        self.peak_pages_in_use = max(self.peak_pages_in_use, in_use)
+        rec = StepRecord(n_prefill, n_decode, useful, self.clock() - t0, self.scheduler.last_preempted,
+                         self.scheduler.last_admitted)
+        self.steps.append(rec)
+        return rec
+
+    def run_until_idle(self) -> None:
+        while self.has_work():
+            self.step()
+
+    def stats(self) -> dict:
+        m = self.runner.manager
+        return {
+            "prefill_tokens_computed": self.prefill_tokens_computed,
+            "preemptions": self.scheduler.preemptions,
+            "peak_running": self.peak_running,
+            "peak_blocks_in_use": self.peak_pages_in_use,
+            "pool_blocks": m.num_pages,
+            "pool_mib": self.runner.pools.total_bytes() / 2 ** 20,
+        }
+
+
+# ---------------------------------------------------------------------------------------------- one sequence
+@dataclass
+class GenerationResult:
+    """As the reference's (src/miniserve/generate.py:19-37)."""
+
+    token_ids: List[int]
+    prompt_len: int
+    ttft: float
+    total_time: float
+    step_times: List[float] = field(default_factory=list)
+    finish_reason: str = "length"
+    cache_bytes: int = 0
+
+    @property
+    def decode_tps(self) -> float:
+        t = sum(self.step_times)
+        return len(self.step_times) / t if t > 0 else 0.0
+
+    @property
+    def ms_per_token(self) -> float:
+        return 1000 * sum(self.step_times) / len(self.step_times) if self.step_times else 0.0
+
+
+def generate(model: Model, prompt_ids: Sequence[int], max_new_tokens: int = 64, eos_ids: Sequence[int] = (),
+             temperature: float = 0.0, top_k: int = 0, top_p: float = 1.0, seed: Optional[int] = None,
+             block_size: int = 16) -> GenerationResult:
+    """Generate from one prompt and measure, with the reference's option names
+    (src/miniserve/generate.py:85-135).  The stop id is not part of the output."""
+    need = len(prompt_ids) + max_new_tokens
+    eng = Engine(model, num_blocks=-(-need // block_size), block_size=block_size, max_seqs=1, max_len=need,
+                 max_num_batched_tokens=max(need, 1))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    req = eng.add_request(Request(list(prompt_ids), max_new_tokens, tuple(eos_ids), temperature, top_k, top_p, seed))
+    marks = []
+    while eng.has_work():
+        n = len(req.output_ids)
+        eng.step()
+        if len(req.output_ids) > n:
+            marks.append(time.perf_counter())
+    total = time.perf_counter() - t0
+    per_token = model.config.kv_bytes_per_token(model.rt.dtype.itemsize) if hasattr(model, "config") else 0
+    return GenerationResult(
+        token_ids=list(req.output_ids), prompt_len=len(prompt_ids), ttft=(marks[0] - t0) if marks else total,
+        total_time=total, step_times=[b - a for a, b in zip(marks, marks[1:])],
+        finish_reason=req.finish_reason or "length", cache_bytes=per_token * (len(prompt_ids) + len(req.output_ids)))

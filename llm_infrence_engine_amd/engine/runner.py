@@ -13,12 +13,8 @@ from typing import Hashable, List, Optional
 import torch
 
 from ..cache import CacheLayout, CacheManager, CachePools
-from ..config.engine_config import EngineConfig
-from ..parts.base import Runtime
 from ..parts.model import Model, RunCache
 from .batch import BatchBuilder, StepEntry
-
-_DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
 
 
 class ModelRunner:
@@ -69,21 +65,10 @@ class ModelRunner:
 
 def load_runner(model_dir, dtype: str = "bfloat16", device: str = "cuda:0", page_size: int = 16,
                 num_pages: Optional[int] = None, max_requests: int = 32, max_len: int = 1024) -> ModelRunner:
-    """Model folder -> a runner with an empty cache.  The model class is chosen by config.json."""
-    from ..config import load_config
-    from ..weights import CheckpointReader
+    """Model folder -> a runner with an empty cache."""
+    from ..loading import load_model
 
-    if dtype not in _DTYPES:
-        raise ValueError(f"dtype must be 'bfloat16' or 'float32', got {dtype!r}")
-    dev = torch.device(device)
-    if dev.type != "cuda":
-        raise RuntimeError(f"the engine runs on the GPU only (device {device!r} was asked for); there is no CPU path")
-    if not torch.cuda.is_available():
-        raise RuntimeError("no GPU is visible to this process; the engine has no CPU path")
-    config = load_config(model_dir)
-    model = Model(config.to_spec())
-    model.load(CheckpointReader(model_dir), Runtime(dev, _DTYPES[dtype]))
-    model.config = config
+    model = load_model(model_dir, dtype, device)
     if num_pages is None:
         num_pages = max_requests * (-(-max_len // page_size))
     return ModelRunner(model, page_size, num_pages, max_requests, max_len)

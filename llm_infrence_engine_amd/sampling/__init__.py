@@ -1,0 +1,3 @@
+from .sampler import Sampler, SamplingParams
+
+__all__ = ["Sampler", "SamplingParams"]

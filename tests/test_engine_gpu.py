@@ -1,0 +1,173 @@
+"""The engine above the step function, on the GPU: greedy generation through the entry points against the
+plain implementation, the scheduler under page pressure, sampling options, long decoding and the first
+tokens of a sequence."""
+import json
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from tests.conftest import ROOT, TINY
+from tests.plain import qwen2_plain as P
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def eng():
+    import llm_infrence_engine_amd as e
+
+    return e
+
+
+@pytest.fixture(scope="module", params=["A", "B"])
+def tiny(request, tmp_path_factory, eng):
+    from llm_infrence_engine_amd.config import config_from_dict
+
+    name = request.param
+    d = tmp_path_factory.mktemp(f"gen{name}")
+    eng.write_random_model(d, config_from_dict(TINY[name]), seed=3, dtype="float32", std=0.1)
+    cfg, w = P.read_config(d), P.read_weights(d, torch.float64)
+    return name, str(d), cfg, w
+
+
+def prompts_for(name, vocab):
+    lengths = [5, 11, 17] if name == "A" else [1, 9, 23, 40]
+    rng = np.random.default_rng(7)
+    return [[int(t) for t in rng.integers(0, vocab, n)] for n in lengths]
+
+
+def test_greedy_generation_matches_plain(tiny, eng):
+    """The configurations' own workloads: A decodes 8 tokens per prompt with pages of 4; B 12 tokens with
+    prompts cut into portions of 7 and pages of 8."""
+    name, d, cfg, w = tiny
+    prompts = prompts_for(name, cfg["vocab_size"])
+    n_new = 8 if name == "A" else 12
+    want = [P.greedy_generate(w, cfg, p, n_new) for p in prompts]
+    kw = dict(block_size=4, max_len=64) if name == "A" else dict(block_size=8, max_len=64, max_prefill_chunk=7)
+    llm = eng.LLM(d, dtype="float32", **kw)
+    got = llm.generate(prompts, eng.SamplingParams(max_new_tokens=n_new))
+    assert [o.token_ids for o in got] == want
+    assert all(o.finish_reason == "length" for o in got)
+    llm.engine.runner.manager.check_invariants()
+    assert all(g.allocator.num_in_use() == 0 for g in llm.engine.runner.manager.groups)
+    # one prompt alone through generate(), with the reference's option names
+    r = eng.generate(llm.model, prompts[1], max_new_tokens=n_new)
+    assert r.token_ids == want[1] and r.finish_reason == "length" and r.prompt_len == len(prompts[1])
+    assert len(r.step_times) == n_new - 1 and r.cache_bytes > 0
+
+
+def test_stop_id_is_not_emitted(tiny, eng):
+    name, d, cfg, w = tiny
+    p = prompts_for(name, cfg["vocab_size"])[1]
+    full = P.greedy_generate(w, cfg, p, 8)
+    stop = full[3]
+    model = eng.load_model(d, "float32")
+    r = eng.generate(model, p, max_new_tokens=8, eos_ids=[stop])
+    assert r.finish_reason == "stop" and r.token_ids == full[:full.index(stop)]
+
+
+def test_preemption_under_page_pressure_keeps_outputs(tiny, eng):
+    """A pool too small for everybody: requests are preempted and recomputed, outputs do not change, and
+    every page comes back (the reference's tests/test_paged.py:247-259)."""
+    name, d, cfg, w = tiny
+    rng = np.random.default_rng(11)
+    prompts = [[int(t) for t in rng.integers(0, cfg["vocab_size"], n)] for n in (9, 14, 6, 11, 8)]
+    want = [P.greedy_generate(w, cfg, p, 10) for p in prompts]
+    model = eng.load_model(d, "float32")
+    e = eng.Engine(model, num_blocks=15, block_size=4, max_seqs=4, max_len=32, max_num_batched_tokens=12)
+    reqs = [e.add_request(eng.Request(p, max_new_tokens=10)) for p in prompts]
+    while e.has_work():
+        e.step()
+        e.runner.manager.check_invariants()
+    assert e.preemptions > 0
+    assert [r.output_ids for r in reqs] == want
+    assert all(g.allocator.num_in_use() == 0 for g in e.runner.manager.groups)
+    assert e.stats()["preemptions"] == e.preemptions
+
+
+def test_mid_flight_join_and_cancel(tiny, eng):
+    name, d, cfg, w = tiny
+    ps = prompts_for(name, cfg["vocab_size"])
+    want = [P.greedy_generate(w, cfg, p, 6) for p in ps[:2]]
+    model = eng.load_model(d, "float32")
+    e = eng.Engine(model, block_size=4, max_seqs=3, max_len=64)
+    a = e.add_request(eng.Request(ps[0], max_new_tokens=6))
+    e.step(); e.step()
+    b = e.add_request(eng.Request(ps[1], max_new_tokens=6))   # joins while a is decoding
+    c = e.add_request(eng.Request(ps[2], max_new_tokens=40))
+    e.step()
+    e.cancel(c)
+    e.run_until_idle()
+    assert a.output_ids == want[0] and b.output_ids == want[1]
+    assert c.finish_reason == "abort" and c not in e.finished
+    assert a.arrival_time <= a.admitted_time <= a.first_token_time <= a.finish_time
+    assert all(g.allocator.num_in_use() == 0 for g in e.runner.manager.groups)
+
+
+def test_long_decoding_and_first_tokens(tiny, eng):
+    """Decode 150 tokens one by one from a 3-token prompt in bfloat16 and float32: the first tokens of a
+    sequence and positions far past several pages, checked against the plain logits along the way."""
+    from llm_infrence_engine_amd.engine import StepEntry, load_runner
+
+    name, d, cfg, w = tiny
+    rng = np.random.default_rng(5)
+    toks = [int(t) for t in rng.integers(0, cfg["vocab_size"], 153)]
+    exact = P.forward(w, cfg, toks).numpy()
+    noise = np.abs(P.forward(w, cfg, toks, act_dtype=torch.bfloat16).numpy() - exact).max()
+    for dtype, bound in (("float32", 1e-3), ("bfloat16", 3.0 * noise)):
+        r = load_runner(d, dtype=dtype, page_size=8, num_pages=24, max_requests=2, max_len=160)
+        first = r.step([StepEntry("x", toks[:3], [0, 1, 2])]).cpu().numpy()
+        assert np.abs(first - exact[:3]).max() < bound
+        for p in range(3, len(toks)):
+            row = r.step([StepEntry("x", [toks[p]], [0])]).cpu().numpy()[0]
+            assert np.abs(row - exact[p]).max() < bound, f"{dtype} position {p}"
+
+
+def test_sampling_through_the_engine(tiny, eng):
+    name, d, cfg, w = tiny
+    p = prompts_for(name, cfg["vocab_size"])[1]
+    llm = eng.LLM(d, dtype="float32", block_size=4, max_len=64)
+    sp = eng.SamplingParams(max_new_tokens=12, temperature=1.0, seed=42)
+    a = llm.generate([p, p], [sp, sp])
+    assert a[0].token_ids == a[1].token_ids                      # same seed, same tokens
+    b = llm.generate([p], eng.SamplingParams(max_new_tokens=12, temperature=1.0, seed=43))
+    assert b[0].token_ids != a[0].token_ids
+    greedy = P.greedy_generate(w, cfg, p, 12)
+    k1 = llm.generate([p], eng.SamplingParams(max_new_tokens=12, temperature=1.5, top_k=1, seed=1))
+    assert k1[0].token_ids == greedy                             # top_k = 1 is greedy
+    tiny_p = llm.generate([p], eng.SamplingParams(max_new_tokens=12, temperature=1.0, top_p=1e-6, seed=1))
+    assert tiny_p[0].token_ids == greedy                         # the most likely token always stays
+
+
+def test_rejects_impossible_requests(tiny, eng):
+    name, d, cfg, w = tiny
+    model = eng.load_model(d, "float32")
+    e = eng.Engine(model, num_blocks=4, block_size=4, max_seqs=2, max_len=64)
+    with pytest.raises(ValueError, match="empty"):
+        e.add_request(eng.Request([]))
+    with pytest.raises(ValueError, match="max_len"):
+        e.add_request(eng.Request([1] * 60, max_new_tokens=10))
+    with pytest.raises(ValueError, match="never fit"):
+        e.add_request(eng.Request([1] * 10, max_new_tokens=10))
+    with pytest.raises(ValueError, match="vocabulary"):
+        e.add_request(eng.Request([cfg["vocab_size"]], max_new_tokens=1))
+
+
+def test_command_line(tiny, tmp_path):
+    name, d, cfg, w = tiny
+    p = prompts_for(name, cfg["vocab_size"])[0]
+    want = P.greedy_generate(w, cfg, p, 5)
+    r = subprocess.run([sys.executable, "-m", "llm_infrence_engine_amd", "--model", d, "--dtype", "float32",
+                        "--prompt-ids", ",".join(map(str, p)), "--max-new-tokens", "5", "--max-len", "64"],
+                       capture_output=True, text=True, cwd=str(ROOT), timeout=300)
+    assert r.returncode == 0, r.stderr
+    assert json.loads(r.stdout.strip().splitlines()[-1])["token_ids"] == want
+
+
+def test_engine_refuses_the_cpu(tiny, eng):
+    name, d, cfg, w = tiny
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        eng.load_model(d, "float32", device="cpu")
