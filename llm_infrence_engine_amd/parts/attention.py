@@ -40,11 +40,13 @@ class GQAttention(Mixer):
         specs.append(TensorSpec(f"{p}o_proj.weight", (H, self.num_heads * d)))
         if self.out_bias:
             specs.append(TensorSpec(f"{p}o_proj.bias", (H,), "bias"))
+        if self.position is not None:
+            specs += self.position.tensor_specs()
         return specs
 
     def load(self, get, rt):
         self.rt = rt
-        by_name = {s.name: s for s in self.tensor_specs()}
+        by_name = {s.name: s for s in GQAttention.tensor_specs(self)}
         p = self.prefix
         w = [get(by_name[f"{p}{n}.weight"]) for n in ("q_proj", "k_proj", "v_proj")]
         self.w_qkv = linear.prepare_weight(torch.cat(w, dim=0))

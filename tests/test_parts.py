@@ -1,0 +1,383 @@
+"""Each part alone against the plain implementation, and the generality of the assembly: a toy architecture
+defined here (a mixer with state of its own, a routed feed-forward, another position encoding, a windowed
+layer, a layer that runs twice, a run that reads another run's cache) is registered, written to a model
+folder, loaded by name and stepped in portions, without touching the framework's files."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from tests.plain import qwen2_plain as P
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def fw():
+    import llm_infrence_engine_amd as root
+    from llm_infrence_engine_amd import cache, config, engine, parts, weights
+    from llm_infrence_engine_amd.kernels import ops
+
+    class NS:
+        pass
+    ns = NS()
+    ns.root, ns.cache, ns.config, ns.engine, ns.parts, ns.weights, ns.ops = root, cache, config, engine, parts, weights, ops
+    return ns
+
+
+def rt_for(fw, dtype):
+    return fw.parts.Runtime(torch.device(DEV), dtype)
+
+
+def getter(tensors, fw, rt):
+    return lambda spec: fw.weights.place(tensors[spec.name], spec, rt.dtype, rt.device)
+
+
+def random_for(part, seed, fw, std=0.3):
+    return fw.weights.random_tensors(part.tensor_specs(), seed, std=std, dtype="float32")
+
+
+def single_request_ctx(fw, need, n_tokens, start, page_size, rt, total):
+    """A step context and cache view for one request that already holds ``start`` tokens."""
+    layout = fw.cache.CacheLayout([(need, None, None)])
+    m = fw.cache.CacheManager(layout, page_size, 40, 2, 256)
+    pools = fw.cache.CachePools(layout, page_size, 40, 2, rt)
+    b = fw.engine.BatchBuilder(m, 1000, rt.device)
+    return m, pools, b
+
+
+# ------------------------------------------------------------------------------------------------ parts alone
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_part(fw, dtype):
+    part = fw.parts.build_part("norm", fw.config.PartSpec("rms_norm", "n.", {"size": 200, "eps": 3e-4}))
+    t = random_for(part, 0, fw)
+    rt = rt_for(fw, dtype)
+    part.load(getter(t, fw, rt), rt)
+    x = torch.randn(6, 200, device=DEV) * 2
+    want = P.rms_norm(x.double().cpu(), t["n.weight"].double(), 3e-4)
+    got = part.forward(x)
+    assert got.dtype == dtype
+    torch.testing.assert_close(got.double().cpu(), want, atol=2e-5 if dtype == torch.float32 else 3e-2, rtol=1e-2)
+
+
+def test_feed_forward_part(fw):
+    part = fw.parts.build_part("feed_forward", fw.config.PartSpec("swiglu", "m.", {"hidden_size": 72, "intermediate_size": 200}))
+    t = random_for(part, 1, fw, std=0.2)
+    rt = rt_for(fw, torch.float32)
+    part.load(getter(t, fw, rt), rt)
+    h = torch.randn(5, 72, device=DEV)
+    want = P.swiglu_mlp(h.double().cpu(), {k: v.double() for k, v in t.items()}, "m.")
+    torch.testing.assert_close(part.forward(h, None).double().cpu(), want, atol=1e-4, rtol=1e-4)
+
+
+def test_embedding_and_head_parts(fw):
+    emb = fw.parts.build_part("embedding", fw.config.PartSpec("token_embedding", "e.", {"vocab_size": 331, "hidden_size": 72}))
+    head = fw.parts.build_part("head", fw.config.PartSpec("lm_head", "h.", {"hidden_size": 72, "vocab_size": 331, "tied_to": "e.weight"}))
+    t = random_for(emb, 2, fw)
+    rt = rt_for(fw, torch.bfloat16)
+    placed = {}
+
+    def get(spec):
+        if spec.name not in placed:
+            placed[spec.name] = fw.weights.place(t[spec.name], spec, rt.dtype, rt.device)
+        return placed[spec.name]
+    emb.load(get, rt); head.load(get, rt)
+    assert head.weight.data_ptr() == emb.weight.data_ptr()     # tied: one matrix (the reference's tests/test_model_parity.py:29-31)
+    assert head.ignorable() == ["h.weight"]
+
+    class Ctx:
+        num_tokens = 4
+        token_ids = torch.tensor([0, 330, 7, 7], dtype=torch.int32, device=DEV)
+    x = emb.forward(Ctx)
+    assert x.dtype == torch.float32 and torch.equal(x.cpu(), t["e.weight"].bfloat16().float()[[0, 330, 7, 7]])
+    h = torch.randn(3, 72, device=DEV).bfloat16()
+    logits = head.forward(h)
+    assert logits.dtype == torch.float32 and logits.shape == (3, 331)
+    torch.testing.assert_close(logits.cpu().double(), h.double().cpu() @ t["e.weight"].bfloat16().double().T, atol=1e-4, rtol=1e-4)
+
+
+@pytest.mark.parametrize("nh,nkv,d,window,page_size", [(6, 2, 32, None, 8), (5, 5, 48, 9, 4), (4, 1, 16, None, 16)])
+def test_attention_part_in_portions(fw, nh, nkv, d, window, page_size):
+    """The mixer alone, fed 50 tokens as 23 + 2 + 24 + 1, against the plain attention block."""
+    H, T = 40, 50
+    pos = fw.parts.build_part("position", fw.config.PartSpec("rotary_half", "", {"head_dim": d, "rotary_dim": d, "theta": 500.0}))
+    spec = fw.config.PartSpec("gqa_attention", "a.", {"hidden_size": H, "num_heads": nh, "num_kv_heads": nkv, "head_dim": d,
+                                                      "scale": 1 / math.sqrt(d), "qkv_bias": True, "out_bias": False, "window": window})
+    part = fw.parts.build_part("mixer", spec, position=pos)
+    t = random_for(part, 3, fw, std=0.4)
+    rt = rt_for(fw, torch.float32)
+    part.load(getter(t, fw, rt), rt)
+    assert part.cache_need() == fw.parts.KVNeed(nkv, d, window)
+    h = torch.randn(T, H)
+    w = {k: v.double() for k, v in t.items()}
+    cfg = {"num_heads": nh, "num_kv_heads": nkv, "head_dim": d}
+    cos, sin = P.rope_cos_sin(torch.arange(T), d, 500.0)
+    if window is None:
+        want = P.attention_block(h.double(), w, "a.", cfg, cos, sin)
+    else:  # the plain block has no window: assemble it from the plain pieces
+        q = (h.double() @ w["a.q_proj.weight"].T + w["a.q_proj.bias"]).view(T, nh, d).transpose(0, 1)
+        k = (h.double() @ w["a.k_proj.weight"].T + w["a.k_proj.bias"]).view(T, nkv, d).transpose(0, 1)
+        v = (h.double() @ w["a.v_proj.weight"].T + w["a.v_proj.bias"]).view(T, nkv, d).transpose(0, 1)
+        o = P.causal_attention(P.apply_rope(q, cos, sin), P.apply_rope(k, cos, sin), v, window=window)
+        want = o.transpose(0, 1).reshape(T, nh * d) @ w["a.o_proj.weight"].T
+    layout = fw.cache.CacheLayout([(part.cache_need(), None, None)])
+    m = fw.cache.CacheManager(layout, page_size, 20, 2, 64)
+    pools = fw.cache.CachePools(layout, page_size, 20, 2, rt)
+    pools.kv[0].fill_(1e4)                                   # what a reused page may hold must not matter
+    builder = fw.engine.BatchBuilder(m, 1000, rt.device)
+    m.add("x")
+    got, p = [], 0
+    for n in (23, 2, 24, 1):
+        m.grow("x", p + n)
+        ctx, tables, slots = builder.build([fw.engine.StepEntry("x", [1] * n, [])])
+        got.append(part.forward(h[p:p + n].to(DEV), ctx, pools.kv_view(0, tables[0], slots[0]), None).cpu())
+        p += n
+        m.advance("x", p)
+    torch.testing.assert_close(torch.cat(got).double(), want, atol=2e-4, rtol=2e-4)
+
+
+# ------------------------------------------------------------------------------------------------ a toy architecture
+def register_toys(fw):
+    from dataclasses import dataclass
+
+    parts, cfgm, ops = fw.parts, fw.config, fw.ops
+    TensorSpec = fw.weights.TensorSpec
+
+    class ToyDecay(parts.Mixer):
+        """state <- decay * state + W_in h_t ;  out_t = W_out state   (state of fixed size per request)"""
+
+        def __init__(self, prefix, position, hidden_size, state_size, decay):
+            self.prefix, self.H, self.S, self.decay = prefix, hidden_size, state_size, decay
+
+        def tensor_specs(self):
+            return [TensorSpec(self.prefix + "in.weight", (self.S, self.H)), TensorSpec(self.prefix + "out.weight", (self.H, self.S))]
+
+        def load(self, get, rt):
+            self.rt = rt
+            self.w_in, self.w_out = (get(s).float() for s in self.tensor_specs())
+
+        def state_need(self):
+            return parts.StateNeed((self.S,), torch.float32)
+
+        def forward(self, h, ctx, kv, state):
+            assert kv is None
+            hin = h.float() @ self.w_in.T
+            out = torch.empty_like(h)
+            o = 0
+            for n, slot in zip(ctx.q_lens_host, ctx.state_slots_host):
+                s = state.slots[slot].clone()
+                for t in range(n):
+                    s = self.decay * s + hin[o + t]
+                    out[o + t] = (self.w_out @ s).to(h.dtype)
+                state.slots[slot] = s
+                o += n
+            return out
+
+    class ToyRouted(parts.FeedForward):
+        """router logits in float -> softmax -> the best expert alone, weighted by its probability"""
+
+        def __init__(self, prefix, hidden_size, intermediate_size, num_experts):
+            self.prefix, self.H, self.I, self.E = prefix, hidden_size, intermediate_size, num_experts
+
+        def tensor_specs(self):
+            return [TensorSpec(self.prefix + "router.weight", (self.E, self.H), keep32=True),
+                    TensorSpec(self.prefix + "up.weight", (self.E * self.I, self.H)),
+                    TensorSpec(self.prefix + "down.weight", (self.E * self.H, self.I))]
+
+        def load(self, get, rt):
+            self.rt = rt
+            self.router, self.up, self.down = (get(s).float() for s in self.tensor_specs())
+
+        def forward(self, h, ctx):
+            x = h.float()
+            prob = (x @ self.router.T).softmax(-1)
+            best = prob.argmax(-1)
+            out = torch.zeros_like(x)
+            for e in range(self.E):
+                rows = (best == e).nonzero().flatten()
+                if rows.numel():
+                    a = torch.relu(x[rows] @ self.up[e * self.I:(e + 1) * self.I].T)
+                    out[rows] = (a @ self.down[e * self.H:(e + 1) * self.H].T) * prob[rows, e:e + 1]
+            return out.to(h.dtype)
+
+    class ToyOffset(parts.PositionEncoding):
+        """adds table[position % period] to every q and k head (absolute, not rotary)"""
+
+        def __init__(self, prefix, head_dim, period):
+            self.prefix, self.d, self.period = prefix, head_dim, period
+
+        def tensor_specs(self):
+            return [TensorSpec(self.prefix + "table", (self.period, self.d))]
+
+        def load(self, get, rt):
+            self.rt = rt
+            self.table = get(self.tensor_specs()[0])
+
+        def encode_and_store(self, qkv, nh, nkv, d, ctx, kv):
+            v = qkv.view(qkv.shape[0], nh + 2 * nkv, d)
+            v[:, :nh + nkv] += self.table[(ctx.positions.long() % self.period)][:, None, :]
+            if kv is not None and kv.store:
+                ops.rope_store(qkv, nh, nkv, d, 0, None, None, kv.slot_mapping, kv.k_pages, kv.v_pages)
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        vocab_size: int
+        width: int
+        heads: int
+        kv_heads: int
+        head_size: int
+        inner: int
+        experts: int
+        state_size: int
+        decay: float
+        window: int
+        eps: float
+
+        @classmethod
+        def from_dict(cls, d):
+            return cls(**{k: d[k] for k in cls.__dataclass_fields__})
+
+        def to_dict(self):
+            d = {k: getattr(self, k) for k in self.__dataclass_fields__}
+            d["architectures"] = ["ToyForCausalLM"]
+            return d
+
+        def to_spec(self):
+            H, d = self.width, self.head_size
+            PartSpec, LayerSpec, Run = cfgm.PartSpec, cfgm.LayerSpec, cfgm.Run
+            norm = lambda p: PartSpec("rms_norm", p, {"size": H, "eps": self.eps})
+
+            def attn(p, window, position):
+                return dict(mixer=PartSpec("gqa_attention", p + "attn.", {
+                    "hidden_size": H, "num_heads": self.heads, "num_kv_heads": self.kv_heads, "head_dim": d,
+                    "scale": 1 / math.sqrt(d), "qkv_bias": False, "out_bias": True, "window": window}), position=position)
+            rotary = PartSpec("rotary_half", "", {"head_dim": d, "rotary_dim": d // 2, "theta": 100.0})
+            dense = lambda p: PartSpec("swiglu", p + "ff.", {"hidden_size": H, "intermediate_size": self.inner})
+            routed = lambda p: PartSpec("toy_routed", p + "ff.", {"hidden_size": H, "intermediate_size": self.inner, "num_experts": self.experts})
+            layers = []
+            for i, (mix, ff) in enumerate([
+                    (attn("l0.", self.window, rotary), dense("l0.")),
+                    (dict(mixer=PartSpec("toy_decay", "l1.mix.", {"hidden_size": H, "state_size": self.state_size, "decay": self.decay})), routed("l1.")),
+                    (attn("l2.", None, PartSpec("toy_offset", "l2.pos.", {"head_dim": d, "period": 7})), routed("l2.")),
+                    (attn("l3.", self.window - 1, rotary), dense("l3."))]):
+                p = f"l{i}."
+                layers.append(LayerSpec(block="pre_norm_residual", feed_forward=ff, mixer_norm=norm(p + "n1."),
+                                        feed_forward_norm=norm(p + "n2."), **mix))
+            # layer 1 runs twice (two states), the last run reads the keys and values that run 0 stored
+            order = (Run(0), Run(1), Run(2), Run(1), Run(3, cache_of=0))
+            return cfgm.ModelSpec("ToyForCausalLM", H, self.vocab_size,
+                                  PartSpec("token_embedding", "emb.", {"vocab_size": self.vocab_size, "hidden_size": H}),
+                                  tuple(layers), order, norm("final."),
+                                  PartSpec("lm_head", "head.", {"hidden_size": H, "vocab_size": self.vocab_size, "tied_to": None}))
+
+    parts.register_part("mixer", "toy_decay", ToyDecay)
+    parts.register_part("feed_forward", "toy_routed", ToyRouted)
+    parts.register_part("position", "toy_offset", ToyOffset)
+    cfgm.register_architecture("ToyForCausalLM", ToyConfig)
+    return ToyConfig
+
+
+def toy_plain(w, c, ids):
+    """The toy model whole, in double, written out here from the toy parts' one-line definitions."""
+    T, H, d, nh, nkv = len(ids), c.width, c.head_size, c.heads, c.kv_heads
+    x = w["emb.weight"][ids]
+    pos = torch.arange(T)
+    cos, sin = P.rope_cos_sin(pos, d // 2, 100.0)
+
+    def rot(t):  # partial rotary: the first half of each head
+        return torch.cat((P.apply_rope(t[..., :d // 2], cos, sin), t[..., d // 2:]), -1)
+
+    def attn(h, p, window, position, kv=None):
+        q = (h @ w[p + "attn.q_proj.weight"].T).view(T, nh, d).transpose(0, 1)
+        k = (h @ w[p + "attn.k_proj.weight"].T).view(T, nkv, d).transpose(0, 1)
+        v = (h @ w[p + "attn.v_proj.weight"].T).view(T, nkv, d).transpose(0, 1)
+        if position == "rotary":
+            q, k = rot(q), rot(k)
+        else:
+            off = w["l2.pos.table"][pos % 7]
+            q, k = q + off, k + off
+        if kv is not None:
+            k, v = kv
+        o = P.causal_attention(q, k, v, window=window).transpose(0, 1).reshape(T, nh * d)
+        return o @ w[p + "attn.o_proj.weight"].T + w[p + "attn.o_proj.bias"], (k, v)
+
+    def decay(h):
+        s = torch.zeros(c.state_size, dtype=h.dtype)
+        out = []
+        for t in range(T):
+            s = c.decay * s + w["l1.mix.in.weight"] @ h[t]
+            out.append(w["l1.mix.out.weight"] @ s)
+        return torch.stack(out)
+
+    def dense(h, p):
+        return P.swiglu_mlp(h, {"gate_proj.weight": w[p + "ff.gate_proj.weight"], "up_proj.weight": w[p + "ff.up_proj.weight"],
+                                "down_proj.weight": w[p + "ff.down_proj.weight"]}, "")
+
+    def routed(h, p):
+        prob = (h @ w[p + "ff.router.weight"].T).softmax(-1)
+        best = prob.argmax(-1)
+        out = torch.zeros_like(h)
+        for t in range(T):
+            e = int(best[t])
+            a = torch.relu(w[p + "ff.up.weight"][e * c.inner:(e + 1) * c.inner] @ h[t])
+            out[t] = (w[p + "ff.down.weight"][e * H:(e + 1) * H] @ a) * prob[t, e]
+        return out
+
+    n = lambda t, p: P.rms_norm(t, w[p + "weight"], c.eps)
+    a, kv0 = attn(n(x, "l0.n1."), "l0.", c.window, "rotary"); x = x + a
+    x = x + dense(n(x, "l0.n2."), "l0.")
+    for _ in (0,):
+        x = x + decay(n(x, "l1.n1.")); x = x + routed(n(x, "l1.n2."), "l1.")
+    a, _ = attn(n(x, "l2.n1."), "l2.", None, "offset"); x = x + a
+    x = x + routed(n(x, "l2.n2."), "l2.")
+    x = x + decay(n(x, "l1.n1.")); x = x + routed(n(x, "l1.n2."), "l1.")
+    a, _ = attn(n(x, "l3.n1."), "l3.", c.window - 1, "rotary", kv=kv0); x = x + a
+    x = x + dense(n(x, "l3.n2."), "l3.")
+    return n(x, "final.") @ w["head.weight"].T
+
+
+def test_toy_architecture_is_registered_built_and_stepped(fw, tmp_path):
+    ToyConfig = register_toys(fw)
+    cfg = ToyConfig(vocab_size=101, width=40, heads=4, kv_heads=2, head_size=16, inner=56, experts=3, state_size=24,
+                    decay=0.8, window=6, eps=1e-5)
+    d = fw.root.write_random_model(tmp_path / "toy", cfg, seed=4, dtype="float32", std=0.25)
+    assert type(fw.root.load_config(d)).__name__ == "ToyConfig"
+    runner = fw.engine.load_runner(d, dtype="float32", page_size=4, num_pages=40, max_requests=3, max_len=64)
+    lay = runner.layout
+    assert len(lay.group_keys) == 2 and lay.state_runs == [1, 3] and lay.run_stores == [True, False, True, False, False]
+    assert lay.run_group[4] == lay.run_group[0] and lay.run_entry[4] == lay.run_entry[0]
+    w = P.read_weights(d, torch.float64)
+    rng = np.random.default_rng(0)
+    seqs = {r: [int(t) for t in rng.integers(0, 101, n)] for r, n in (("a", 37), ("b", 22), ("c", 9))}
+    want = {r: toy_plain(w, cfg, torch.tensor(t)).numpy() for r, t in seqs.items()}
+    Entry = fw.engine.StepEntry
+    # a whole; then b and c in portions beside each other, with a's slot and pages used again by c
+    got = runner.step([Entry("a", seqs["a"], list(range(37)))]).cpu().numpy()
+    assert np.abs(got - want["a"]).max() < 1e-3
+    runner.free_request("a")
+    out = {"b": [], "c": []}
+    cuts = {"b": [5, 2, 14, 1], "c": [2, 6, 1]}
+    pos = {"b": 0, "c": 0}
+    for i in range(4):
+        entries = []
+        for r in ("b", "c"):
+            if i < len(cuts[r]):
+                n = cuts[r][i]
+                entries.append(Entry(r, seqs[r][pos[r]:pos[r] + n], list(range(n))))
+        logits = runner.step(entries).cpu().numpy()
+        o = 0
+        for e in entries:
+            out[e.req_id].append(logits[o:o + len(e.tokens)])
+            o += len(e.tokens)
+            pos[e.req_id] += len(e.tokens)
+        runner.manager.check_invariants()
+    for r in ("b", "c"):
+        assert np.abs(np.concatenate(out[r]) - want[r]).max() < 1e-3, r
+    # the windowed group has given pages back along the way; the full group has not
+    full = [i for i, k in enumerate(lay.group_keys) if k.window is None][0]
+    held = runner.manager.pages_held("b")
+    assert len(held[full]) == 6 and len(held[1 - full]) < 6
+    runner.free_request("b"); runner.free_request("c")
+    assert all(g.allocator.num_in_use() == 0 for g in runner.manager.groups)
