@@ -39,15 +39,6 @@ def random_for(part, seed, fw, std=0.3):
     return fw.weights.random_tensors(part.tensor_specs(), seed, std=std, dtype="float32")
 
 
-def single_request_ctx(fw, need, n_tokens, start, page_size, rt, total):
-    """A step context and cache view for one request that already holds ``start`` tokens."""
-    layout = fw.cache.CacheLayout([(need, None, None)])
-    m = fw.cache.CacheManager(layout, page_size, 40, 2, 256)
-    pools = fw.cache.CachePools(layout, page_size, 40, 2, rt)
-    b = fw.engine.BatchBuilder(m, 1000, rt.device)
-    return m, pools, b
-
-
 # ------------------------------------------------------------------------------------------------ parts alone
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_norm_part(fw, dtype):
@@ -328,8 +319,7 @@ def toy_plain(w, c, ids):
     n = lambda t, p: P.rms_norm(t, w[p + "weight"], c.eps)
     a, kv0 = attn(n(x, "l0.n1."), "l0.", c.window, "rotary"); x = x + a
     x = x + dense(n(x, "l0.n2."), "l0.")
-    for _ in (0,):
-        x = x + decay(n(x, "l1.n1.")); x = x + routed(n(x, "l1.n2."), "l1.")
+    x = x + decay(n(x, "l1.n1.")); x = x + routed(n(x, "l1.n2."), "l1.")
     a, _ = attn(n(x, "l2.n1."), "l2.", None, "offset"); x = x + a
     x = x + routed(n(x, "l2.n2."), "l2.")
     x = x + decay(n(x, "l1.n1.")); x = x + routed(n(x, "l1.n2."), "l1.")
