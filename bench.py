@@ -1,0 +1,174 @@
+"""Decode and prefill throughput of the engine on one MI355X, with roofline fractions.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Default run: the layer sizes of the Qwen2.5-0.5B configuration with random weights in bfloat16, a batch
+of 8 requests with 512-token prompts, K timed decode steps through the whole engine (scheduler, step
+function, sampler).  One JSON line is printed: ``value`` is decoded tokens a second; ``prefill`` is one
+2,048-token prompt in one step; ``roofline`` prices the decode step against HBM bandwidth (every weight it
+uses once plus the cache of the live requests); ``points`` holds decode throughput at batch 1 and 64.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import tempfile
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# MI355X published peaks
+HBM_GBS = 8000.0
+PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "fp8": 5000.0, "fp32": 157.3}
+
+# Qwen2.5-0.5B's config.json sizes (BASELINE.json configs[2])
+MODEL = {
+    "architectures": ["Qwen2ForCausalLM"], "num_hidden_layers": 24, "hidden_size": 896, "num_attention_heads": 14,
+    "num_key_value_heads": 2, "intermediate_size": 4864, "vocab_size": 151936, "rope_theta": 1000000.0,
+    "rms_norm_eps": 1e-6, "tie_word_embeddings": True,
+}
+PROMPT_LEN = 512
+CONTEXT_LIMIT = 8192
+BLOCK_SIZE = 16
+PREFILL_TOKENS = 2048
+# the reference's own decode at batch 8: CUDA-graph step of 6.0 ms on an A10, context 128 (docs/RESULTS.md:38)
+BASELINE_TOKS = 8 / 6.0e-3
+
+
+def decode_bytes(cfg, batch, context, bytes_per_value=2):
+    """Bytes a decode step has to read: every weight it uses once (the embedding table counts once, as the
+    tied head) and the keys and values of the live requests."""
+    H, I, V, d = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size, cfg.head_dim
+    nh, nkv, L = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.num_hidden_layers
+    per_layer = (nh + 2 * nkv) * d * H + H * nh * d + 3 * H * I
+    weights = (L * per_layer + V * H) * bytes_per_value + (L * ((nh + 2 * nkv) * d + 2 * H) + H) * 4
+    return weights + batch * context * cfg.kv_bytes_per_token(bytes_per_value)
+
+
+def prefill_flops(cfg, tokens):
+    H, I, V, d = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size, cfg.head_dim
+    nh, nkv, L = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.num_hidden_layers
+    linear = 2 * tokens * L * ((nh + 2 * nkv) * d * H + H * nh * d + 3 * H * I) + 2 * V * H  # head: one row
+    attention = L * 4 * nh * d * tokens * (tokens + 1) // 2
+    return linear + attention
+
+
+def run_decode(eng_mod, model, batch, steps, warmup, vocab, seed):
+    """Prefill ``batch`` prompts, then time ``steps`` decode steps of the engine.  Returns seconds per step."""
+    import numpy as np
+    import torch
+
+    rng = np.random.default_rng(seed)
+    budget = max(4096, batch)
+    extra = -(-batch * PROMPT_LEN // budget) + 2     # requests admitted first decode while the others prefill
+    need = PROMPT_LEN + warmup + steps + extra
+    pages = batch * (-(-need // BLOCK_SIZE) + 1)
+    e = eng_mod.Engine(model, num_blocks=pages, block_size=BLOCK_SIZE, max_seqs=batch, max_len=CONTEXT_LIMIT,
+                       max_num_batched_tokens=budget)
+    for _ in range(batch):
+        e.add_request(eng_mod.Request([int(t) for t in rng.integers(0, vocab, PROMPT_LEN)],
+                                      max_new_tokens=warmup + steps + extra))
+    while any(r.num_tokens - r.num_computed > 1 for r in e.running) or e.waiting:
+        e.step()                                   # prompts in portions under the budget; first tokens sampled
+    for _ in range(warmup):
+        e.step()
+    assert len(e.running) == batch and all(r.num_tokens - r.num_computed == 1 for r in e.running)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        e.step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    assert all(rec.decode_batch == batch and rec.n_prefill_tokens == 0 for rec in e.steps[-steps:])
+    mean_context = PROMPT_LEN + warmup + (steps + 1) / 2
+    return dt, mean_context
+
+
+def run_prefill(eng_mod, model, vocab, seed, repeats=5):
+    import numpy as np
+    import torch
+
+    from llm_infrence_engine_amd.engine import ModelRunner, StepEntry
+
+    rng = np.random.default_rng(seed)
+    runner = ModelRunner(model, BLOCK_SIZE, PREFILL_TOKENS // BLOCK_SIZE + 1, 1, PREFILL_TOKENS + BLOCK_SIZE)
+    best = None
+    for i in range(repeats + 1):
+        toks = [int(t) for t in rng.integers(0, vocab, PREFILL_TOKENS)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        runner.step([StepEntry("p", toks, [PREFILL_TOKENS - 1])])
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        runner.free_request("p")
+        if i > 0:                                   # the first run warms up
+            best = dt if best is None else min(best, dt)
+    return best
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=MODEL["num_hidden_layers"],
+                    help="fewer layers than the configuration has, if memory or time needs it (both numbers are reported)")
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points and the prefill")
+    a = ap.parse_args()
+    if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print(f"bench.py measures one GPU; --gpus {a.gpus} is not supported by this single-GPU engine")
+        return 2
+
+    import torch
+
+    import llm_infrence_engine_amd as eng
+    from llm_infrence_engine_amd.config import config_from_dict
+
+    d = dict(MODEL)
+    d["num_hidden_layers"] = a.layers
+    cfg = config_from_dict(d)
+    with tempfile.TemporaryDirectory() as folder:
+        eng.write_random_model(folder, cfg, seed=0, dtype="bfloat16")
+        model = eng.load_model(folder, "bfloat16", "cuda:0")
+    vocab = cfg.vocab_size
+
+    dt, ctx = run_decode(eng, model, a.batch, a.steps, a.warmup, vocab, seed=1)
+    value = a.batch / dt
+    gbs = decode_bytes(cfg, a.batch, ctx) / dt / 1e9
+    out = {
+        "metric": "decode_tokens_per_s", "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1,
+        "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": round(value / BASELINE_TOKS, 2), "dtype": "bf16", "data": "synthetic",
+        "config": {
+            "model": "Qwen2.5-0.5B shape, random weights", "layers": a.layers, "layers_of_config": MODEL["num_hidden_layers"],
+            "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
+            "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": vocab, "tied": True,
+            "global_batch": a.batch, "prompt_len": PROMPT_LEN, "seq_len": CONTEXT_LIMIT, "block_size": BLOCK_SIZE,
+            "prefill_tokens": PREFILL_TOKENS, "parallelism": "single_gpu",
+            "baseline": "reference CUDA-graph decode, batch 8, ctx 128, A10 bf16: 6.0 ms/step",
+        },
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_GBS, 4)},
+    }
+    if not a.no_points:
+        pt = run_prefill(eng, model, vocab, seed=2)
+        tf = prefill_flops(cfg, PREFILL_TOKENS) / pt / 1e12
+        out["prefill"] = {"value": round(PREFILL_TOKENS / pt, 1), "tokens": PREFILL_TOKENS, "ms": round(pt * 1e3, 3),
+                          "frac": round(tf / PEAK_TFLOPS["bf16"], 4)}
+        points = {}
+        for b in (1, 64):
+            steps = min(a.steps, 128)
+            dtb, _ = run_decode(eng, model, b, steps, min(a.warmup, 8), vocab, seed=3 + b)
+            points[f"decode_b{b}"] = round(b / dtb, 1)
+        out["points"] = points
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
