@@ -8,8 +8,11 @@ extern "C" {
 
 int ms_embed(const int* ids, const void* table, float* out, int n_tokens, int hidden, int dtype, hipStream_t stream);
 
-int ms_rms_norm(float* x, const void* delta, int delta_dtype, const float* weight, const int* rows, void* out,
-                int n_rows, int hidden, float eps, int write_back, int dtype, hipStream_t stream);
+int ms_rms_norm(float* x, const void* delta, int delta_dtype, int n_partials, long long partial_stride,
+                const float* weight, const int* rows, void* out, int n_rows, int hidden, float eps, int write_back,
+                int dtype, hipStream_t stream);
+
+int ms_bias_add(void* x, const float* bias, int n_rows, int width, int dtype, hipStream_t stream);
 
 int ms_residual_add(float* x, const void* delta, long long total, int dtype, hipStream_t stream);
 
@@ -21,6 +24,11 @@ int ms_rope_store(void* qkv, const int* positions, const float* inv_freq, const 
 
 int ms_gemm_generic(const void* A, const void* W, const float* bias, void* C, int M, int N, int K, long long lda,
                     long long ldw, long long ldc, int in_dtype, int out_dtype, int accumulate, hipStream_t stream);
+
+int ms_gemm_skinny_splits(int K, int splits);
+
+int ms_gemm_skinny(const void* A, long long lda, const void* W, long long ldw, const float* bias, void* out,
+                   long long ldo, int M, int N, int K, int epilogue, int splits, int out_dtype, hipStream_t stream);
 
 int ms_paged_attention_generic(const void* q, long long q_stride, const void* k_pages, const void* v_pages,
                                const int* block_table, int table_stride, const int* token_req, const int* positions,

@@ -28,10 +28,12 @@ extern "C" int ms_embed(const int* ids, const void* table, float* out, int n_tok
 
 // ------------------------------------------------------------------------------------------------
 // Row r of the output is the norm of row rows[r] (or r) of x.  With `delta`, x[row] += delta[row]
-// first (written back), which is the residual sum of the layer before.  `delta2` is a second addend.
+// first (written back), which is the residual sum of the layer before; delta may come as n_partials
+// partial sums [n_partials, N, H], added in order.
 // y = w * (x * rsqrt(mean(x^2) + eps)), all in float, rounded once on store.
 template <typename T, typename TD>
-__global__ void rms_norm_kernel(float* __restrict__ x, const TD* __restrict__ delta, const float* __restrict__ w,
+__global__ void rms_norm_kernel(float* __restrict__ x, const TD* __restrict__ delta, int n_partials,
+                                size_t partial_stride, const float* __restrict__ w,
                                 const int* __restrict__ rows, T* __restrict__ out, int H, float eps, int write_back) {
   __shared__ float red[16];
   extern __shared__ float buf[];  // H floats: the row after the residual sum
@@ -42,7 +44,7 @@ __global__ void rms_norm_kernel(float* __restrict__ x, const TD* __restrict__ de
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
     float v = xr[i];
     if (delta) {
-      v += to_float(delta[(size_t)src * H + i]);
+      for (int p = 0; p < n_partials; ++p) v += to_float(delta[p * partial_stride + (size_t)src * H + i]);
       if (write_back) xr[i] = v;
     }
     buf[i] = v;
@@ -54,14 +56,15 @@ __global__ void rms_norm_kernel(float* __restrict__ x, const TD* __restrict__ de
   for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = from_float<T>(w[i] * (buf[i] * inv));
 }
 
-extern "C" int ms_rms_norm(float* x, const void* delta, int delta_dtype, const float* weight, const int* rows,
-                           void* out, int n_rows, int hidden, float eps, int write_back, int dtype,
-                           hipStream_t stream) {
+extern "C" int ms_rms_norm(float* x, const void* delta, int delta_dtype, int n_partials, long long partial_stride,
+                           const float* weight, const int* rows, void* out, int n_rows, int hidden, float eps,
+                           int write_back, int dtype, hipStream_t stream) {
   if (n_rows <= 0) return MS_OK;
+  if (delta && (n_partials < 1 || partial_stride < 0)) return MS_BAD_ARG;
   if (hidden <= 0 || hidden > 16384) return MS_UNSUPPORTED;  // the row is staged in LDS
   dim3 grid(n_rows), block(hidden >= 1024 ? 256 : 128);
   size_t lds = (size_t)hidden * sizeof(float);
-#define LAUNCH(T, TD) rms_norm_kernel<T, TD><<<grid, block, lds, stream>>>(x, (const TD*)delta, weight, rows, (T*)out, hidden, eps, write_back)
+#define LAUNCH(T, TD) rms_norm_kernel<T, TD><<<grid, block, lds, stream>>>(x, (const TD*)delta, n_partials, (size_t)partial_stride, weight, rows, (T*)out, hidden, eps, write_back)
   if (dtype == MS_F32) {
     if (delta && delta_dtype == MS_BF16) return MS_BAD_ARG;
     LAUNCH(float, float);
@@ -93,7 +96,28 @@ extern "C" int ms_residual_add(float* x, const void* delta, long long total, int
 }
 
 // ------------------------------------------------------------------------------------------------
-// out[n, i] = silu(gu[n, i]) * gu[n, I + i],  silu(z) = z / (1 + exp(-z))
+// x[n, :] += bias[:]  (for a product that came without its bias)
+template <typename T>
+__global__ void bias_add_kernel(T* __restrict__ x, const float* __restrict__ bias, int width, size_t total) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < total; i += stride) x[i] = from_float<T>(to_float(x[i]) + bias[i % width]);
+}
+
+extern "C" int ms_bias_add(void* x, const float* bias, int n_rows, int width, int dtype, hipStream_t stream) {
+  if (n_rows <= 0) return MS_OK;
+  if (width <= 0) return MS_BAD_ARG;
+  const size_t total = (size_t)n_rows * width;
+  int blocks = (int)((total + 255) / 256);
+  if (blocks > 8192) blocks = 8192;
+  if (dtype == MS_F32) bias_add_kernel<float><<<blocks, 256, 0, stream>>>((float*)x, bias, width, total);
+  else if (dtype == MS_BF16) bias_add_kernel<bf16><<<blocks, 256, 0, stream>>>((bf16*)x, bias, width, total);
+  else return MS_BAD_ARG;
+  return ms_launch_status();
+}
+
+// ------------------------------------------------------------------------------------------------
+// out[n, i] = silu(gu[n, 2i]) * gu[n, 2i + 1],  silu(z) = z / (1 + exp(-z)): gate and up interleaved
 template <typename T>
 __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total) {
   size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -101,8 +125,8 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, i
   for (; idx < total; idx += stride) {
     const size_t n = idx / I;
     const int i = (int)(idx - n * I);
-    const float g = to_float(gu[n * 2 * I + i]);
-    const float u = to_float(gu[n * 2 * I + I + i]);
+    const float g = to_float(gu[n * 2 * I + 2 * i]);
+    const float u = to_float(gu[n * 2 * I + 2 * i + 1]);
     out[idx] = from_float<T>(g / (1.0f + expf(-g)) * u);
   }
 }

@@ -1,0 +1,147 @@
+// out[M,N] = A[M,K] . W[N,K]^T for few rows (M <= 64, a decode step's tokens), bfloat16 in, float accumulation
+// on the matrix cores (v_mfma_f32_16x16x32_bf16).  The product is bound by reading W once from HBM, so
+// the kernel is shaped for memory parallelism: a block owns 16 output features and a slice of K; its four
+// waves take interleaved 32-wide k-steps, each lane streaming 16 bytes of one weight row per step, and add
+// their accumulators through LDS in a fixed order.  The weight tile is the MFMA's A operand and the
+// activation tile its B operand, so a lane ends up with 4 consecutive output features of one token.
+//
+// Epilogues: plain (+ bias) to bfloat16 or float; gated activation over interleaved rows (2j: gate j,
+// 2j+1: up j) writing silu(gate) * up; float partial sums [splits, M, N] when K is split over blocks
+// (whoever consumes them adds them up in order, so results do not depend on timing).
+#include "common.h"
+#include "api.h"
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+enum { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_PARTIAL = 2 };
+
+template <int MT, int EPI, typename TO>
+__global__ void __launch_bounds__(256)
+gemm_skinny_kernel(const bf16* __restrict__ A, size_t lda, const bf16* __restrict__ W, size_t ldw,
+                   const float* __restrict__ bias, TO* __restrict__ out, size_t ldo, int M, int N, int K,
+                   int steps_per_split) {
+  __shared__ f32x4 red[3][MT][MS_WAVE];
+  const int lane = threadIdx.x & (MS_WAVE - 1), wave = threadIdx.x / MS_WAVE;
+  const int col = lane & 15, kq = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const int total_steps = (K + 31) / 32;
+  const int step_begin = blockIdx.y * steps_per_split;
+  const int step_end = min(total_steps, step_begin + steps_per_split);
+
+  const int wn = min(n0 + col, N - 1);  // rows past the end repeat the last one; their results are not stored
+  const bf16* wrow = W + (size_t)wn * ldw + kq * 8;
+  const bf16* arow[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) arow[t] = A + (size_t)min(t * 16 + col, M - 1) * lda + kq * 8;
+
+  f32x4 acc[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll 4
+  for (int s = step_begin + wave; s < step_end; s += 4) {
+    const int k = s * 32;
+    bf16x8 wv = {0, 0, 0, 0, 0, 0, 0, 0};
+    const bool in = k + kq * 8 < K;  // K is a multiple of 8: a lane's 8 values are all inside or all outside
+    if (in) wv = *reinterpret_cast<const bf16x8*>(wrow + k);
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      bf16x8 av = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (in) av = *reinterpret_cast<const bf16x8*>(arow[t] + k);
+      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, av, acc[t], 0, 0, 0);
+    }
+  }
+
+  if (wave > 0) {
+#pragma unroll
+    for (int t = 0; t < MT; ++t) red[wave - 1][t][lane] = acc[t];
+  }
+  __syncthreads();
+  if (wave > 0) return;
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int w = 0; w < 3; ++w) acc[t] += red[w][t][lane];
+
+  // lane holds out[m = t*16 + col][n = n0 + kq*4 + r], r = 0..3
+  const int nb = n0 + kq * 4;
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int m = t * 16 + col;
+    if (m >= M) continue;
+    if (EPI == EPI_SWIGLU) {
+      // rows nb, nb+1 are (gate, up) of feature nb/2; rows nb+2, nb+3 of feature nb/2 + 1
+#pragma unroll
+      for (int p = 0; p < 2; ++p) {
+        if (nb + 2 * p + 1 < N) {
+          const float g = acc[t][2 * p], u = acc[t][2 * p + 1];
+          out[(size_t)m * ldo + nb / 2 + p] = from_float<TO>(g / (1.0f + expf(-g)) * u);
+        }
+      }
+    } else {
+      TO* o = out + (EPI == EPI_PARTIAL ? (size_t)blockIdx.y * M * ldo : 0) + (size_t)m * ldo + nb;
+      const bool add_bias = bias != nullptr && (EPI != EPI_PARTIAL || blockIdx.y == 0);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        if (nb + r < N) o[r] = from_float<TO>(acc[t][r] + (add_bias ? bias[nb + r] : 0.f));
+      }
+    }
+  }
+}
+
+template <int EPI, typename TO>
+int launch_mt(const bf16* A, size_t lda, const bf16* W, size_t ldw, const float* bias, TO* out, size_t ldo, int M,
+              int N, int K, int splits, hipStream_t stream) {
+  const int total_steps = (K + 31) / 32;
+  const int per = (total_steps + splits - 1) / splits;
+  dim3 grid((N + 15) / 16, (total_steps + per - 1) / per), block(256);
+#define GO(MT) gemm_skinny_kernel<MT, EPI, TO><<<grid, block, 0, stream>>>(A, lda, W, ldw, bias, out, ldo, M, N, K, per)
+  if (M <= 16) GO(1);
+  else if (M <= 32) GO(2);
+  else if (M <= 48) GO(3);
+  else GO(4);
+#undef GO
+  return ms_launch_status();
+}
+
+}  // namespace
+
+// The number of partial sums that ms_gemm_skinny writes for `splits` asked for (a split never is empty).
+extern "C" int ms_gemm_skinny_splits(int K, int splits) {
+  const int total_steps = (K + 31) / 32;
+  if (splits < 1) splits = 1;
+  const int per = (total_steps + splits - 1) / splits;
+  return (total_steps + per - 1) / per;
+}
+
+// epilogue 0: out[M,N] (out_dtype float or bfloat16) = product + bias
+// epilogue 1: out[M,N/2] bfloat16 = silu(gate) * up over interleaved rows of W (no bias)
+// epilogue 2: out[splits,M,N] float partial sums (bias goes into split 0); `splits` as ms_gemm_skinny_splits gives
+extern "C" int ms_gemm_skinny(const void* A, long long lda, const void* W, long long ldw, const float* bias, void* out,
+                              long long ldo, int M, int N, int K, int epilogue, int splits, int out_dtype,
+                              hipStream_t stream) {
+  if (M <= 0 || N <= 0) return MS_OK;
+  if (M > 64) return MS_UNSUPPORTED;
+  if (K <= 0 || K % 8 || lda % 8 || ldw % 8 || lda < K || ldw < K) return MS_UNSUPPORTED;
+  if (((uintptr_t)A | (uintptr_t)W) % 16) return MS_UNSUPPORTED;
+  const bf16* a = (const bf16*)A;
+  const bf16* w = (const bf16*)W;
+  if (epilogue == EPI_STORE) {
+    if (ldo < N) return MS_BAD_ARG;
+    if (out_dtype == MS_BF16) return launch_mt<EPI_STORE, bf16>(a, lda, w, ldw, bias, (bf16*)out, ldo, M, N, K, 1, stream);
+    if (out_dtype == MS_F32) return launch_mt<EPI_STORE, float>(a, lda, w, ldw, bias, (float*)out, ldo, M, N, K, 1, stream);
+    return MS_BAD_ARG;
+  }
+  if (epilogue == EPI_SWIGLU) {
+    if (N % 2 || ldo < N / 2 || out_dtype != MS_BF16 || bias) return MS_BAD_ARG;
+    return launch_mt<EPI_SWIGLU, bf16>(a, lda, w, ldw, nullptr, (bf16*)out, ldo, M, N, K, 1, stream);
+  }
+  if (epilogue == EPI_PARTIAL) {
+    if (ldo < N || out_dtype != MS_F32 || splits < 1) return MS_BAD_ARG;
+    return launch_mt<EPI_PARTIAL, float>(a, lda, w, ldw, bias, (float*)out, ldo, M, N, K, splits, stream);
+  }
+  return MS_BAD_ARG;
+}

@@ -1,6 +1,12 @@
 """Matrix products of the model: out = a @ w.T (+ bias).  Picks the kernel by type and shape.
 
-float32 always goes to the vector-ALU kernel (a true 32-bit product).  bfloat16 accumulates in float.
+float32          the vector-ALU kernel: a true 32-bit product, whatever the shape.
+bfloat16, few rows (a decode step)   the weight-streaming matrix-core kernel, with the bias, the gated
+                 activation or split-K partial sums as its epilogue.
+bfloat16, many rows (prompt portions)  the library's matrix product (hipBLASLt through torch.mm), as the
+                 reference uses a library for every product (F.linear, src/miniserve/model.py:123-165);
+                 shapes it cannot take fall back to the vector-ALU kernel.
+All accumulate in float.
 """
 from __future__ import annotations
 
@@ -10,14 +16,63 @@ import torch
 
 from . import ops
 
+_mm_out_dtype_ok = None  # whether torch.mm can write float from bfloat16 inputs (found out at first use)
+
 
 def prepare_weight(w: torch.Tensor) -> torch.Tensor:
     """The layout the kernels read: [out features, in features], rows contiguous."""
     return w.contiguous()
 
 
+def interleave_rows(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """Rows a0, b0, a1, b1, ...: the packing of gate and up that the gated epilogue reads."""
+    return torch.stack((a, b), dim=1).reshape(2 * a.shape[0], a.shape[1]).contiguous()
+
+
+def _library_mm(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> Optional[torch.Tensor]:
+    global _mm_out_dtype_ok
+    if out_dtype == a.dtype:
+        return torch.mm(a, w.t())
+    if _mm_out_dtype_ok is None:
+        try:
+            torch.mm(a[:1], w[:1].t(), out_dtype=out_dtype)
+            _mm_out_dtype_ok = True
+        except (TypeError, RuntimeError):
+            _mm_out_dtype_ok = False
+    return torch.mm(a, w.t(), out_dtype=out_dtype) if _mm_out_dtype_ok else None
+
+
 def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
-           out_dtype: Optional[torch.dtype] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    if out is None:
-        out = torch.empty((a.shape[0], w.shape[0]), dtype=out_dtype or a.dtype, device=a.device)
+           out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """[M, K] x [N, K] -> [M, N] in ``out_dtype`` (default: a's type)."""
+    out_dtype = out_dtype or a.dtype
+    if a.dtype == torch.bfloat16:
+        if ops.skinny_ok(a, w):
+            return ops.gemm_skinny(a, w, bias, ops.EPI_STORE, out_dtype=out_dtype)
+        if a.shape[0] > ops.SKINNY_MAX_ROWS and a.is_contiguous():
+            out = _library_mm(a, w, out_dtype)
+            if out is not None:
+                return ops.bias_add(out, bias) if bias is not None else out
+    out = torch.empty((a.shape[0], w.shape[0]), dtype=out_dtype, device=a.device)
     return ops.gemm_generic(a, w, out, bias=bias)
+
+
+def linear_residual(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """A product that is about to be added to the residual stream: [M, N], or float partial sums [S, M, N]
+    over slices of K that the next norm adds up in order (few rows: more blocks to pull the weights)."""
+    if a.dtype == torch.bfloat16 and ops.skinny_ok(a, w):
+        n_tiles = -(-w.shape[0] // 16)
+        steps = -(-a.shape[1] // 32)
+        splits = max(1, min(-(-512 // n_tiles), steps // 4))
+        if splits > 1:
+            return ops.gemm_skinny(a, w, bias, ops.EPI_PARTIAL, splits=splits)
+    return linear(a, w, bias)
+
+
+def linear_swiglu(a: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
+    """silu(a @ gate.T) * (a @ up.T) for ``w_gate_up`` = interleave_rows(gate, up): [M, I]."""
+    if a.dtype == torch.bfloat16 and ops.skinny_ok(a, w_gate_up):
+        return ops.gemm_skinny(a, w_gate_up, None, ops.EPI_SWIGLU)
+    gu = linear(a, w_gate_up)
+    act = torch.empty((a.shape[0], w_gate_up.shape[0] // 2), dtype=a.dtype, device=a.device)
+    return ops.silu_mul(gu, act)

@@ -20,7 +20,12 @@ _c_int, _c_ll, _c_float, _c_ptr = ctypes.c_int, ctypes.c_longlong, ctypes.c_floa
 
 _SIGNATURES = {
     "ms_embed": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
-    "ms_rms_norm": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
+    "ms_rms_norm": [_c_ptr, _c_ptr, _c_int, _c_int, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int,
+                    _c_int, _c_ptr],
+    "ms_bias_add": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    "ms_gemm_skinny_splits": [_c_int, _c_int],
+    "ms_gemm_skinny": [_c_ptr, _c_ll, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int,
+                       _c_int, _c_ptr],
     "ms_residual_add": [_c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr],
     "ms_silu_mul": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "ms_rope_store": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int,
@@ -101,7 +106,8 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tenso
              delta: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None,
              write_back: bool = True) -> torch.Tensor:
     """out[r] = weight * normalised(x[rows[r]] (+ delta[rows[r]])).  x float32 [N, H] is the residual stream;
-    with ``delta`` the sum is written back to x (unless ``write_back`` is False)."""
+    with ``delta`` ([N, H], or partial sums [S, N, H] added in order) the sum is written back to x (unless
+    ``write_back`` is False)."""
     _check(x, "x", torch.float32)
     N, H = x.shape
     _check(weight, "weight", torch.float32, (H,))
@@ -110,13 +116,25 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tenso
         _check(rows, "rows", torch.int32)
         n_rows = rows.numel()
     _check(out, "out", None, (n_rows, H))
-    dcode = 0
+    dcode, n_partials = 0, 1
     if delta is not None:
-        _check(delta, "delta", None, (N, H))
+        if delta.dim() == 3:
+            n_partials = delta.shape[0]
+            _check(delta, "delta", None, (n_partials, N, H))
+        else:
+            _check(delta, "delta", None, (N, H))
         dcode = _code(delta.dtype)
-    _call("ms_rms_norm", x.data_ptr(), _ptr(delta), dcode, weight.data_ptr(), _ptr(rows), out.data_ptr(), n_rows, H,
-          float(eps), int(write_back), _code(out.dtype), _stream())
+    _call("ms_rms_norm", x.data_ptr(), _ptr(delta), dcode, n_partials, N * H, weight.data_ptr(), _ptr(rows),
+          out.data_ptr(), n_rows, H, float(eps), int(write_back), _code(out.dtype), _stream())
     return out
+
+
+def bias_add(x: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+    """x[n, :] += bias, in place."""
+    _check(x, "x")
+    _check(bias, "bias", torch.float32, (x.shape[-1],))
+    _call("ms_bias_add", x.data_ptr(), bias.data_ptr(), x.numel() // x.shape[-1], x.shape[-1], _code(x.dtype), _stream())
+    return x
 
 
 def residual_add(x: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
@@ -127,7 +145,7 @@ def residual_add(x: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
 
 
 def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out[n, i] = silu(gate_up[n, i]) * gate_up[n, I + i]."""
+    """out[n, i] = silu(gate_up[n, 2i]) * gate_up[n, 2i + 1]: gate and up columns interleaved."""
     _check(gate_up, "gate_up")
     N, two_i = gate_up.shape
     if two_i % 2:
@@ -180,6 +198,50 @@ def gemm_generic(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Opti
     _call("ms_gemm_generic", a.data_ptr(), w.data_ptr(), _ptr(bias), out.data_ptr(), M, N, K,
           a.stride(0) if M > 1 else K, w.stride(0) if N > 1 else K, out.stride(0) if M > 1 else N,
           _code(a.dtype), _code(out.dtype), int(accumulate), _stream())
+    return out
+
+
+SKINNY_MAX_ROWS = 64
+EPI_STORE, EPI_SWIGLU, EPI_PARTIAL = 0, 1, 2
+
+
+def skinny_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether the few-rows matrix-core kernel takes this product."""
+    return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.shape[0] <= SKINNY_MAX_ROWS
+            and a.shape[1] % 8 == 0 and a.stride(1) == 1 and w.is_contiguous()
+            and (a.shape[0] == 1 or a.stride(0) % 8 == 0) and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+
+
+def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, epilogue: int = EPI_STORE,
+                splits: int = 1, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """a [M <= 64, K] @ w [N, K].T on the matrix cores, bfloat16 in.  Epilogues: EPI_STORE -> [M, N] (+ bias);
+    EPI_SWIGLU -> [M, N / 2] = silu(even rows' products) * odd rows' products; EPI_PARTIAL -> float [S, M, N]
+    partial sums over slices of K (bias in the first), to be added in order by the consumer."""
+    _check(a, "a", torch.bfloat16, contiguous=False)
+    _check(w, "w", torch.bfloat16)
+    if a.dim() != 2 or w.dim() != 2 or a.shape[1] != w.shape[1]:
+        raise ValueError(f"shapes do not fit: a {list(a.shape)}, w {list(w.shape)}")
+    if not skinny_ok(a, w):
+        raise ValueError(f"the few-rows kernel takes at most {SKINNY_MAX_ROWS} rows of bfloat16 with K a multiple of 8 "
+                         f"and 16-byte aligned rows; got a {list(a.shape)} strides {a.stride()}")
+    M, K = a.shape
+    N = w.shape[0]
+    if bias is not None:
+        _check(bias, "bias", torch.float32, (N,))
+    if epilogue == EPI_STORE:
+        out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+        ldo = N
+    elif epilogue == EPI_SWIGLU:
+        if N % 2 or bias is not None:
+            raise ValueError("the gated epilogue needs an even number of weight rows and no bias")
+        out, ldo, out_dtype = torch.empty((M, N // 2), dtype=torch.bfloat16, device=a.device), N // 2, torch.bfloat16
+    elif epilogue == EPI_PARTIAL:
+        splits = _get("ms_gemm_skinny_splits")(K, splits)
+        out, ldo, out_dtype = torch.empty((splits, M, N), dtype=torch.float32, device=a.device), N, torch.float32
+    else:
+        raise ValueError(f"unknown epilogue {epilogue}")
+    _call("ms_gemm_skinny", a.data_ptr(), a.stride(0) if M > 1 else K, w.data_ptr(), K, _ptr(bias), out.data_ptr(), ldo,
+          M, N, K, epilogue, splits, _code(out_dtype), _stream())
     return out
 
 

@@ -73,7 +73,7 @@ class GQAttention(Mixer):
             ops.rope_store(qkv, nh, nkv, d, 0, None, None, kv.slot_mapping, kv.k_pages, kv.v_pages)
         out = self.rt.empty(ctx.num_tokens, nh * d)
         ops.paged_attention(qkv, kv.k_pages, kv.v_pages, kv.block_table, ctx, out, nh, self.scale, self.window)
-        return linear.linear(out, self.w_o, bias=self.b_o)
+        return linear.linear_residual(out, self.w_o, bias=self.b_o)
 
 
 register_part("mixer", "gqa_attention", GQAttention)

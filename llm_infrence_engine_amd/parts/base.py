@@ -6,7 +6,7 @@ it is in.  Five kinds are chosen layer by layer:
 ``Norm``              forward(x, delta, rows, write_back) -> activations         (x: the float residual stream)
 ``PositionEncoding``  encode_and_store(qkv, nh, nkv, d, ctx, kv)                 (belongs to a mixer)
 ``Mixer``             forward(h, ctx, kv, state) -> [N, hidden]                  (attention here)
-``FeedForward``       forward(h, ctx) -> [N, hidden]
+``FeedForward``       forward(h, ctx) -> [N, hidden]    (both may return float partial sums [S, N, hidden])
 ``Block``             forward(x, pending, ctx, kv, state) -> pending             (the arrangement of the four)
 
 plus ``Embedding`` and ``Head`` at the model's ends.  Every part lists the checkpoint tensors it wants

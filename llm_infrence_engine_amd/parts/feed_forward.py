@@ -1,10 +1,9 @@
 """Dense gated feed-forward: down(silu(gate(x)) * up(x)), no biases (src/miniserve/model.py:155-165).
-Gate and up are one packed matrix product; the activation is float."""
+Gate and up are one packed matrix product (rows interleaved so that the activation can be the product's
+epilogue); the activation is float."""
 from __future__ import annotations
 
-import torch
-
-from ..kernels import linear, ops
+from ..kernels import linear
 from ..weights.spec import TensorSpec
 from .base import FeedForward, register_part
 
@@ -21,14 +20,11 @@ class SwiGLU(FeedForward):
     def load(self, get, rt):
         self.rt = rt
         g, u, d = (get(s) for s in self.tensor_specs())
-        self.w_gate_up = linear.prepare_weight(torch.cat((g, u), dim=0))
+        self.w_gate_up = linear.interleave_rows(g, u)
         self.w_down = linear.prepare_weight(d)
 
     def forward(self, h, ctx):
-        gu = linear.linear(h, self.w_gate_up)
-        act = self.rt.empty(h.shape[0], self.intermediate_size)
-        ops.silu_mul(gu, act)
-        return linear.linear(act, self.w_down)
+        return linear.linear_residual(linear.linear_swiglu(h, self.w_gate_up), self.w_down)
 
 
 register_part("feed_forward", "swiglu", SwiGLU)

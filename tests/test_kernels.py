@@ -73,7 +73,7 @@ def test_silu_mul(ops, dtype):
     out = torch.empty(7, 200, dtype=dtype, device=DEV)
     ops.silu_mul(gu, out)
     a = gu.double()
-    want = torch.nn.functional.silu(a[:, :200]) * a[:, 200:]
+    want = torch.nn.functional.silu(a[:, 0::2]) * a[:, 1::2]
     torch.testing.assert_close(out.double(), want, **tol(dtype))
 
 
@@ -268,3 +268,66 @@ def test_ops_refuse_cpu_tensors_and_wrong_shapes(ops):
         ops.paged_attention_generic(torch.zeros(1, 6, device=DEV), kp, kp, torch.zeros(1, 1, dtype=torch.int32, device=DEV),
                                     torch.zeros(1, dtype=torch.int32, device=DEV), torch.zeros(1, dtype=torch.int32, device=DEV),
                                     torch.zeros(1, 6, device=DEV), 1, 1.0)
+
+
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 33, 64])
+@pytest.mark.parametrize("N,K", [(1152, 896), (331, 72), (896, 4864), (50, 200)])
+def test_gemm_skinny(ops, M, N, K):
+    g = torch.Generator().manual_seed(M * 1000 + N)
+    a = torch.randn(M, K, generator=g).bfloat16().to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16().to(DEV)
+    bias = torch.randn(N, generator=g).to(DEV)
+    want = a.double() @ w.double().T
+    out = ops.gemm_skinny(a, w, bias)
+    torch.testing.assert_close(out.double(), want + bias.double(), **tol(torch.bfloat16))
+    f = ops.gemm_skinny(a, w, None, out_dtype=torch.float32)
+    assert f.dtype == torch.float32
+    torch.testing.assert_close(f.double(), want, atol=2e-5, rtol=2e-5)
+    for splits in (2, 5):
+        parts = ops.gemm_skinny(a, w, bias, ops.EPI_PARTIAL, splits=splits)
+        assert parts.dim() == 3 and parts.shape[1:] == (M, N) and parts.shape[0] <= splits
+        torch.testing.assert_close(parts.double().sum(0), want + bias.double(), atol=2e-5, rtol=2e-5)
+    if N % 2 == 0:
+        act = ops.gemm_skinny(a, w, None, ops.EPI_SWIGLU)
+        wantact = torch.nn.functional.silu(want[:, 0::2]) * want[:, 1::2]
+        torch.testing.assert_close(act.double(), wantact, **tol(torch.bfloat16))
+    # a row slice of a wider matrix, and the same row alone: the same bits whatever else is in the batch
+    wide = torch.zeros(M, K + 8, dtype=torch.bfloat16, device=DEV)
+    wide[:, :K] = a
+    assert torch.equal(ops.gemm_skinny(wide[:, :K], w, bias), out)
+    assert torch.equal(ops.gemm_skinny(a[M - 1:], w, bias), out[M - 1:])
+
+
+def test_gemm_skinny_refuses_what_it_cannot_take(ops):
+    a = torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ValueError, match="at most 64 rows"):
+        ops.gemm_skinny(a, w)
+    with pytest.raises(ValueError, match="multiple of 8"):
+        ops.gemm_skinny(a[:4, :60], w[:, :60].contiguous())
+
+
+def test_linear_picks_a_kernel_for_every_shape(ops):
+    from llm_infrence_engine_amd.kernels import linear
+
+    g = torch.Generator().manual_seed(11)
+    for dtype in DTYPES:
+        for M, N, K in [(3, 40, 72), (100, 40, 72), (200, 331, 120), (5, 33, 60), (70, 33, 60)]:
+            a = torch.randn(M, K, generator=g).to(dtype).to(DEV)
+            w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(dtype).to(DEV)
+            b = torch.randn(N, generator=g).to(DEV)
+            want = a.double() @ w.double().T + b.double()
+            torch.testing.assert_close(linear.linear(a, w, b).double(), want, **tol(dtype))
+            lg = linear.linear(a, w, b, out_dtype=torch.float32)
+            assert lg.dtype == torch.float32
+            torch.testing.assert_close(lg.double(), want, **(tol(torch.float32) if dtype == torch.float32 or M <= 64 else tol(dtype)))
+            r = linear.linear_residual(a, w, b)
+            r = r.double().sum(0) if r.dim() == 3 else r.double()
+            torch.testing.assert_close(r, want, **tol(dtype))
+        for M in (4, 90):
+            a = torch.randn(M, 72, generator=g).to(dtype).to(DEV)
+            gate = (torch.randn(50, 72, generator=g) / 8).to(dtype).to(DEV)
+            up = (torch.randn(50, 72, generator=g) / 8).to(dtype).to(DEV)
+            got = linear.linear_swiglu(a, linear.interleave_rows(gate, up))
+            want = torch.nn.functional.silu(a.double() @ gate.double().T) * (a.double() @ up.double().T)
+            torch.testing.assert_close(got.double(), want, **tol(dtype))
