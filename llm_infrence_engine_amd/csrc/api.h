@@ -20,7 +20,7 @@ int ms_silu_mul(const void* gate_up, void* out, int n_tokens, int intermediate, 
 
 int ms_rope_store(void* qkv, const int* positions, const float* inv_freq, const int* slot_mapping, void* k_pages,
                   void* v_pages, int n_tokens, int num_heads, int num_kv_heads, int head_dim, int rot_dim,
-                  int page_size, int dtype, hipStream_t stream);
+                  int page_size, int v_transposed, int dtype, hipStream_t stream);
 
 int ms_gemm_generic(const void* A, const void* W, const float* bias, void* C, int M, int N, int K, long long lda,
                     long long ldw, long long ldc, int in_dtype, int out_dtype, int accumulate, hipStream_t stream);
@@ -33,8 +33,22 @@ int ms_gemm_skinny(const void* A, long long lda, const void* W, long long ldw, c
 int ms_paged_attention_generic(const void* q, long long q_stride, const void* k_pages, const void* v_pages,
                                const int* block_table, int table_stride, const int* token_req, const int* positions,
                                void* out, long long out_stride, int n_tokens, int num_heads, int num_kv_heads,
-                               int head_dim, int page_size, long long num_pages, float scale, int window, int dtype,
-                               hipStream_t stream);
+                               int head_dim, int page_size, long long num_pages, float scale, int window,
+                               int v_transposed, int dtype, hipStream_t stream);
+
+int ms_attention_mfma_supported(int head_dim, int page_size);
+
+int ms_paged_attention_mfma(const void* q, long long q_stride, const void* k_pages, const void* vt_pages,
+                            const int* block_table, int table_stride, const int* q_start, const int* context_lens,
+                            void* out, long long out_stride, int n_requests, int max_q_len, int num_heads,
+                            int num_kv_heads, int head_dim, int page_size, float scale, int window, hipStream_t stream);
+
+int ms_paged_attention_mfma_decode(const void* q, long long q_stride, const void* k_pages, const void* vt_pages,
+                                   const int* block_table, int table_stride, const int* q_start,
+                                   const int* context_lens, void* out, long long out_stride, void* part_o,
+                                   void* part_ml, int n_requests, int num_heads, int num_kv_heads, int head_dim,
+                                   int page_size, float scale, int window, int keys_per_split, int n_splits,
+                                   hipStream_t stream);
 
 int ms_sample(const float* logits, long long ld, int n_rows, int vocab, const float* temperature, const int* top_k,
               const float* top_p, const unsigned long long* seeds, const int* draw_index, int* out,

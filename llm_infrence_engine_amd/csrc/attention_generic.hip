@@ -18,7 +18,7 @@ paged_attention_generic_kernel(const T* __restrict__ q, size_t q_stride, const T
                                const T* __restrict__ v_pages, const int* __restrict__ block_table, int table_stride,
                                const int* __restrict__ token_req, const int* __restrict__ positions,
                                T* __restrict__ out, size_t out_stride, int n_tokens, int nh, int nkv, int d,
-                               int page_size, float scale, int window) {
+                               int page_size, float scale, int window, int v_transposed) {
   __shared__ float qs[WAVES][MAX_D];
   const int lane = threadIdx.x & (MS_WAVE - 1), wave = threadIdx.x / MS_WAVE;
   const long long item = (long long)blockIdx.x * WAVES + wave;
@@ -71,11 +71,14 @@ paged_attention_generic_kernel(const T* __restrict__ q, size_t q_stride, const T
     for (int jj = 0; jj < count; ++jj) {
       const float pj = __shfl(p, jj, MS_WAVE);
       const int vrow = __shfl(row, jj, MS_WAVE);
-      const T* vp = v_pages + (size_t)vrow * d;
+      // value pages are [page][kv head][slot][dim], or transposed [page][kv head][dim][slot]
+      const T* vp = v_transposed ? v_pages + (size_t)(vrow / page_size) * page_size * d + vrow % page_size
+                                 : v_pages + (size_t)vrow * d;
+      const int vs = v_transposed ? page_size : 1;
 #pragma unroll
       for (int c = 0; c < MAX_D / MS_WAVE; ++c) {
         const int i = lane + c * MS_WAVE;
-        if (i < d) acc[c] = fmaf(pj, to_float(vp[i]), acc[c]);
+        if (i < d) acc[c] = fmaf(pj, to_float(vp[(size_t)i * vs]), acc[c]);
       }
     }
   }
@@ -94,8 +97,8 @@ extern "C" int ms_paged_attention_generic(const void* q, long long q_stride, con
                                           const int* block_table, int table_stride, const int* token_req,
                                           const int* positions, void* out, long long out_stride, int n_tokens,
                                           int num_heads, int num_kv_heads, int head_dim, int page_size,
-                                          long long num_pages, float scale, int window, int dtype,
-                                          hipStream_t stream) {
+                                          long long num_pages, float scale, int window, int v_transposed,
+                                          int dtype, hipStream_t stream) {
   if (n_tokens <= 0) return MS_OK;
   if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads || page_size <= 0 || table_stride <= 0)
     return MS_BAD_ARG;
@@ -103,7 +106,7 @@ extern "C" int ms_paged_attention_generic(const void* q, long long q_stride, con
   if (num_pages * num_kv_heads * page_size >= (1ll << 31)) return MS_UNSUPPORTED;  // row index is an int
   const long long items = (long long)n_tokens * num_heads;
   dim3 grid((unsigned)((items + WAVES - 1) / WAVES)), block(WAVES * MS_WAVE);
-#define LAUNCH(T) paged_attention_generic_kernel<T><<<grid, block, 0, stream>>>((const T*)q, (size_t)q_stride, (const T*)k_pages, (const T*)v_pages, block_table, table_stride, token_req, positions, (T*)out, (size_t)out_stride, n_tokens, num_heads, num_kv_heads, head_dim, page_size, scale, window)
+#define LAUNCH(T) paged_attention_generic_kernel<T><<<grid, block, 0, stream>>>((const T*)q, (size_t)q_stride, (const T*)k_pages, (const T*)v_pages, block_table, table_stride, token_req, positions, (T*)out, (size_t)out_stride, n_tokens, num_heads, num_kv_heads, head_dim, page_size, scale, window, v_transposed)
   if (dtype == MS_F32) LAUNCH(float);
   else if (dtype == MS_BF16) LAUNCH(bf16);
   else return MS_BAD_ARG;

@@ -1,0 +1,318 @@
+// Paged causal attention on the matrix cores (v_mfma_f32_16x16x32_bf16), bfloat16 in, float softmax.
+//
+// One wave owns NT*16 *columns* of one (request, key/value head): a column is a (token, query head of the
+// group) pair, so every key and value that is loaded serves all query heads that share it, and in a prompt
+// portion also NT*16/group consecutive tokens.  Keys are walked in blocks of 32:
+//
+//   S^T[key, col]  = K[key, :] . Q^T[:, col]        A operand: 16 keys x 32 dims, read in place from the
+//                                                   page (a lane reads 16 contiguous bytes of one key);
+//                                                   B operand: the query, kept in registers
+//   online softmax per column in float (scores are in log2 units: scale * log2(e) is folded in)
+//   O^T[dim, col] += V^T[dim, key] . P^T[key, col]  B operand: P^T straight from the S^T accumulators (a lane
+//                                                   holds 4+4 keys of its own column: no transpose);
+//                                                   A operand: V^T, which is why value pages are stored
+//                                                   transposed, [page][kv head][dim][page_size]: a lane reads
+//                                                   8 contiguous bytes (4 keys) of one dim from each page.
+//
+// No LDS and no block-wide barrier: every wave is independent.  The next block's keys and values are
+// loaded while the current block is multiplied.  Keys beyond a column's own position are masked, values
+// beyond the last visible key are zeroed before use, and pages past the context are never dereferenced,
+// so what a reused page still holds cannot reach the result.
+//
+// Two launch shapes: general (any mix of portions and single tokens; grid = column tiles x kv heads x
+// requests, surplus tiles leave at once) and decode (every request has one token; the keys are split over
+// several waves which write unnormalised partial results, and a second kernel combines them).
+#include "common.h"
+#include "api.h"
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+template <int D>
+struct KVBlock {           // one block of 32 keys as this lane sees it
+  bf16x8 k[2][D / 32];     // [16-key subtile][32-dim step]
+  bf16x4 v[D / 16][2];     // [16-dim tile][subtile]: 4 keys of one dim
+};
+
+template <int D>
+__device__ __forceinline__ void load_block(KVBlock<D>& b, const bf16* __restrict__ k_pages,
+                                           const bf16* __restrict__ vt_pages, const int* __restrict__ table,
+                                           int base, int key_hi, int g, int nkv, int page_size, int lane) {
+  const int col = lane & 15, kq = lane >> 4;
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int kb = base + u * 16;
+    const int page = kb <= key_hi ? table[kb / page_size] : 0;  // past the context: the null page
+    const int off = kb % page_size;
+    const bf16* kp = k_pages + (((size_t)page * nkv + g) * page_size + off + col) * D + kq * 8;
+#pragma unroll
+    for (int s = 0; s < D / 32; ++s) b.k[u][s] = *reinterpret_cast<const bf16x8*>(kp + s * 32);
+    const bf16* vp = vt_pages + (((size_t)page * nkv + g) * D + col) * page_size + off + kq * 4;
+#pragma unroll
+    for (int c = 0; c < D / 16; ++c) b.v[c][u] = *reinterpret_cast<const bf16x4*>(vp + (size_t)c * 16 * page_size);
+  }
+}
+
+template <int D, int NT, bool SPLIT>
+__global__ void __launch_bounds__(MS_WAVE)
+attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* __restrict__ k_pages,
+                      const bf16* __restrict__ vt_pages, const int* __restrict__ block_table, int table_stride,
+                      const int* __restrict__ q_start, const int* __restrict__ context_lens,
+                      bf16* __restrict__ out, size_t out_stride, float* __restrict__ part_o,
+                      float* __restrict__ part_ml, int nh, int nkv, int page_size, float scale_log2e, int window,
+                      int keys_per_split, int n_splits) {
+  const int lane = threadIdx.x, col16 = lane & 15, kq = lane >> 4;
+  const int r = blockIdx.z, g = blockIdx.y;
+  const int rep = nh / nkv;
+  const int q0 = q_start[r];
+  const int qlen = q_start[r + 1] - q0;
+  const int start_pos = context_lens[r] - qlen;
+  const int ncols = qlen * rep;
+  const int c0 = SPLIT ? 0 : blockIdx.x * 16 * NT;
+  if (c0 >= ncols) return;
+  const int* table = block_table + (size_t)r * table_stride;
+
+  // key range of the tile: from the first column's window start to the last column's own position
+  const int last_col = min(ncols, c0 + 16 * NT) - 1;
+  int key_hi = start_pos + last_col / rep;
+  int key_lo = 0;
+  if (window > 0) key_lo = max(0, start_pos + c0 / rep - window + 1);
+  int blk_begin = key_lo / 32, blk_end = key_hi / 32 + 1;
+  if (SPLIT) {
+    const int per = keys_per_split / 32;
+    blk_begin += blockIdx.x * per;
+    blk_end = min(blk_end, blk_begin + per);
+    if (blk_begin >= blk_end) return;
+  }
+
+  // this lane's columns
+  int pos[NT], tok[NT], head[NT];
+  bool valid[NT];
+  bf16x8 qv[NT][D / 32];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const int c = c0 + t * 16 + col16;
+    valid[t] = c < ncols;
+    const int cc = min(c, ncols - 1);
+    tok[t] = q0 + cc / rep;
+    head[t] = g * rep + cc % rep;
+    pos[t] = valid[t] ? start_pos + cc / rep : -1;
+    const bf16* qp = q + (size_t)tok[t] * q_stride + (size_t)head[t] * D + kq * 8;
+#pragma unroll
+    for (int s = 0; s < D / 32; ++s) qv[t][s] = *reinterpret_cast<const bf16x8*>(qp + s * 32);
+  }
+
+  float m[NT], l[NT];
+  f32x4 o[D / 16][NT];
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    m[t] = -INFINITY;
+    l[t] = 0.f;
+#pragma unroll
+    for (int c = 0; c < D / 16; ++c) o[c][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  KVBlock<D> cur, nxt;
+  load_block<D>(cur, k_pages, vt_pages, table, blk_begin * 32, key_hi, g, nkv, page_size, lane);
+  for (int blk = blk_begin; blk < blk_end; ++blk) {
+    const int base = blk * 32;
+    if (blk + 1 < blk_end) load_block<D>(nxt, k_pages, vt_pages, table, base + 32, key_hi, g, nkv, page_size, lane);
+
+    // scores: s[u][t] holds keys base + u*16 + kq*4 + (0..3) of column t*16 + col16
+    f32x4 s[2][NT];
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < D / 32; ++ks) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.k[u][ks], qv[t][ks], acc, 0, 0, 0);
+        s[u][t] = acc;
+      }
+
+    // values past the last visible key may be anything a reused page still holds: make them zero
+    if (base + 31 > key_hi) {
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (base + u * 16 + kq * 4 + i > key_hi) {
+#pragma unroll
+            for (int c = 0; c < D / 16; ++c) cur.v[c][u][i] = (__bf16)0.0f;
+          }
+    }
+
+    bf16x8 p[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      float bm = -INFINITY;
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = base + u * 16 + kq * 4 + i;
+          const bool see = key <= pos[t] && (window <= 0 || key > pos[t] - window);
+          const float v = see ? s[u][t][i] * scale_log2e : -INFINITY;
+          s[u][t][i] = v;
+          bm = fmaxf(bm, v);
+        }
+      bm = fmaxf(bm, __shfl_xor(bm, 16, MS_WAVE));
+      bm = fmaxf(bm, __shfl_xor(bm, 32, MS_WAVE));
+      const float m_new = fmaxf(m[t], bm);
+      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
+      const float corr = fast_exp2(m[t] - m_safe);
+      m[t] = m_new;
+      float ls = 0.f;
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float e = fast_exp2(s[u][t][i] - m_safe);
+          ls += e;
+          p[t][u * 4 + i] = (__bf16)e;
+        }
+      l[t] = l[t] * corr + ls;
+#pragma unroll
+      for (int c = 0; c < D / 16; ++c) o[c][t] *= corr;
+    }
+
+#pragma unroll
+    for (int c = 0; c < D / 16; ++c) {
+      bf16x8 vv;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { vv[i] = cur.v[c][0][i]; vv[4 + i] = cur.v[c][1][i]; }
+#pragma unroll
+      for (int t = 0; t < NT; ++t) o[c][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, p[t], o[c][t], 0, 0, 0);
+    }
+    if (blk + 1 < blk_end) cur = nxt;
+  }
+
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    float lt = l[t];
+    lt += __shfl_xor(lt, 16, MS_WAVE);
+    lt += __shfl_xor(lt, 32, MS_WAVE);
+    if (!valid[t]) continue;
+    if (SPLIT) {
+      // unnormalised: O, the running maximum (log2 units) and the sum; the combine kernel weighs the splits
+      const size_t slot = ((size_t)r * nh + head[t]) * n_splits + blockIdx.x;
+      float* po = part_o + slot * D + kq * 4;
+#pragma unroll
+      for (int c = 0; c < D / 16; ++c) *reinterpret_cast<f32x4*>(po + c * 16) = o[c][t];
+      if (kq == 0) { part_ml[slot * 2] = m[t]; part_ml[slot * 2 + 1] = lt; }
+    } else {
+      const float inv = 1.0f / lt;
+      bf16* op = out + (size_t)tok[t] * out_stride + (size_t)head[t] * D + kq * 4;
+#pragma unroll
+      for (int c = 0; c < D / 16; ++c) {
+        bf16x4 w;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[i] = (__bf16)(o[c][t][i] * inv);
+        *reinterpret_cast<bf16x4*>(op + c * 16) = w;
+      }
+    }
+  }
+}
+
+// out[r, h, :] = sum_s 2^(m_s - M) O_s / sum_s 2^(m_s - M) l_s over the splits that request r used
+template <int D>
+__global__ void attention_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                         const int* __restrict__ q_start, const int* __restrict__ context_lens,
+                                         bf16* __restrict__ out, size_t out_stride, int nh, int window,
+                                         int keys_per_split, int n_splits) {
+  const int r = blockIdx.x / nh, h = blockIdx.x % nh;
+  const int key_hi = context_lens[r] - 1;
+  const int key_lo = window > 0 ? max(0, key_hi - window + 1) : 0;
+  const int blocks = key_hi / 32 + 1 - key_lo / 32;
+  const int used = min(n_splits, (blocks * 32 + keys_per_split - 1) / keys_per_split);
+  const size_t slot0 = ((size_t)r * nh + h) * n_splits;
+  float big = -INFINITY;
+  for (int s = 0; s < used; ++s) big = fmaxf(big, part_ml[(slot0 + s) * 2]);
+  float den = 0.f;
+  for (int s = 0; s < used; ++s) den += fast_exp2(part_ml[(slot0 + s) * 2] - big) * part_ml[(slot0 + s) * 2 + 1];
+  const float inv = 1.0f / den;
+  bf16* op = out + (size_t)q_start[r] * out_stride + (size_t)h * D;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+    float acc = 0.f;
+    for (int s = 0; s < used; ++s) acc += fast_exp2(part_ml[(slot0 + s) * 2] - big) * part_o[(slot0 + s) * D + d];
+    op[d] = __float2bfloat16(acc * inv);
+  }
+}
+
+template <int D, int NT>
+int launch_general(const bf16* q, size_t q_stride, const bf16* k, const bf16* vt, const int* table, int table_stride,
+                   const int* q_start, const int* ctx, bf16* out, size_t out_stride, int n_requests, int max_q_len,
+                   int nh, int nkv, int page_size, float scale, int window, hipStream_t stream) {
+  const int rep = nh / nkv;
+  const int tiles = (max_q_len * rep + 16 * NT - 1) / (16 * NT);
+  dim3 grid(tiles, nkv, n_requests), block(MS_WAVE);
+  attention_mfma_kernel<D, NT, false><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, q_start, ctx, out, out_stride, nullptr, nullptr, nh, nkv, page_size, scale * 1.4426950408889634f, window, 0, 0);
+  return ms_launch_status();
+}
+
+template <int D>
+int launch_decode(const bf16* q, size_t q_stride, const bf16* k, const bf16* vt, const int* table, int table_stride,
+                  const int* q_start, const int* ctx, bf16* out, size_t out_stride, float* part_o, float* part_ml,
+                  int n_requests, int nh, int nkv, int page_size, float scale, int window, int keys_per_split,
+                  int n_splits, hipStream_t stream) {
+  dim3 grid(n_splits, nkv, n_requests), block(MS_WAVE);
+  attention_mfma_kernel<D, 1, true><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, q_start, ctx, out, out_stride, part_o, part_ml, nh, nkv, page_size, scale * 1.4426950408889634f, window, keys_per_split, n_splits);
+  attention_combine_kernel<D><<<dim3(n_requests * nh), dim3(D < 64 ? 64 : D), 0, stream>>>(part_o, part_ml, q_start, ctx, out, out_stride, nh, window, keys_per_split, n_splits);
+  return ms_launch_status();
+}
+
+}  // namespace
+
+// Whether the matrix-core kernels take this geometry (else the caller uses the generic kernel).
+extern "C" int ms_attention_mfma_supported(int head_dim, int page_size) {
+  return (head_dim == 32 || head_dim == 64 || head_dim == 128) && page_size > 0 && page_size % 16 == 0;
+}
+
+// General shape.  q [N, >= nh*d] bfloat16 (row stride q_stride), k_pages [P, nkv, page_size, d],
+// vt_pages [P, nkv, d, page_size], block_table int32 [R, table_stride], q_start int32 [R + 1],
+// context_lens int32 [R] (keys held after this step), out [N, nh*d] (row stride out_stride).
+extern "C" int ms_paged_attention_mfma(const void* q, long long q_stride, const void* k_pages, const void* vt_pages,
+                                       const int* block_table, int table_stride, const int* q_start,
+                                       const int* context_lens, void* out, long long out_stride, int n_requests,
+                                       int max_q_len, int num_heads, int num_kv_heads, int head_dim, int page_size,
+                                       float scale, int window, hipStream_t stream) {
+  if (n_requests <= 0 || max_q_len <= 0) return MS_OK;
+  if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads || table_stride <= 0) return MS_BAD_ARG;
+  if (!ms_attention_mfma_supported(head_dim, page_size)) return MS_UNSUPPORTED;
+  if (q_stride % 8 || out_stride % 4 || ((uintptr_t)q % 16) || ((uintptr_t)out % 8)) return MS_UNSUPPORTED;
+  if (n_requests > 65535 || num_kv_heads > 65535) return MS_UNSUPPORTED;
+#define GO(D, NT) return launch_general<D, NT>((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)vt_pages, block_table, table_stride, q_start, context_lens, (bf16*)out, out_stride, n_requests, max_q_len, num_heads, num_kv_heads, page_size, scale, window, stream)
+  const int cols = max_q_len * (num_heads / num_kv_heads);
+  if (head_dim == 32) { if (cols > 32) GO(32, 4); else GO(32, 1); }
+  if (head_dim == 64) { if (cols > 32) GO(64, 4); else GO(64, 1); }
+  if (cols > 16) GO(128, 2); else GO(128, 1);
+#undef GO
+}
+
+// Decode shape: every request has exactly one token and the group (num_heads / num_kv_heads) is at most 16.
+// part_o: float [R, nh, n_splits, d], part_ml: float [R, nh, n_splits, 2]; keys_per_split a multiple of 32.
+extern "C" int ms_paged_attention_mfma_decode(const void* q, long long q_stride, const void* k_pages,
+                                              const void* vt_pages, const int* block_table, int table_stride,
+                                              const int* q_start, const int* context_lens, void* out,
+                                              long long out_stride, void* part_o, void* part_ml, int n_requests,
+                                              int num_heads, int num_kv_heads, int head_dim, int page_size,
+                                              float scale, int window, int keys_per_split, int n_splits,
+                                              hipStream_t stream) {
+  if (n_requests <= 0) return MS_OK;
+  if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads || table_stride <= 0) return MS_BAD_ARG;
+  if (num_heads / num_kv_heads > 16) return MS_UNSUPPORTED;
+  if (!ms_attention_mfma_supported(head_dim, page_size)) return MS_UNSUPPORTED;
+  if (keys_per_split <= 0 || keys_per_split % 32 || n_splits <= 0 || n_splits > 65535) return MS_BAD_ARG;
+  if (q_stride % 8 || out_stride % 4 || ((uintptr_t)q % 16) || ((uintptr_t)out % 8) || ((uintptr_t)part_o % 16)) return MS_UNSUPPORTED;
+  if (n_requests > 65535 || num_kv_heads > 65535) return MS_UNSUPPORTED;
+#define GO(D) return launch_decode<D>((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)vt_pages, block_table, table_stride, q_start, context_lens, (bf16*)out, out_stride, (float*)part_o, (float*)part_ml, n_requests, num_heads, num_kv_heads, page_size, scale, window, keys_per_split, n_splits, stream)
+  if (head_dim == 32) GO(32);
+  if (head_dim == 64) GO(64);
+  GO(128);
+#undef GO
+}

@@ -149,13 +149,14 @@ extern "C" int ms_silu_mul(const void* gate_up, void* out, int n_tokens, int int
 // The first rot_dim values of every q and k head are rotated with half-split pairing (j, j + rot_dim/2):
 //   x1' = x1 cos - x2 sin,  x2' = x2 cos + x1 sin,  angle = float(position) * inv_freq[j]
 // q is rotated in place.  With pages given, the rotated k and v go to
-// pages[slot / page_size][kv head][slot % page_size][:] for slot = slot_mapping[n] (slot < 0: not stored);
+// pages[slot / page_size][kv head][slot % page_size][:] for slot = slot_mapping[n] (slot < 0: not stored;
+// with v_transposed the value goes to v_pages[page][kv head][:][slot % page_size]);
 // k is also rotated in place so that a caller without pages sees it.
 template <typename T>
 __global__ void rope_store_kernel(T* __restrict__ qkv, const int* __restrict__ positions,
                                   const float* __restrict__ inv_freq, const int* __restrict__ slot_mapping,
                                   T* __restrict__ k_pages, T* __restrict__ v_pages, int nh, int nkv, int d,
-                                  int rot_dim, int page_size) {
+                                  int rot_dim, int page_size, int v_transposed) {
   const int n = blockIdx.x;
   T* row = qkv + (size_t)n * (nh + 2 * nkv) * d;
   const float pos = (float)positions[n];
@@ -185,13 +186,15 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const int* __restrict__ p
     const int h = w / d, i = w - h * d;
     const size_t dst = (((size_t)page * nkv + h) * page_size + off) * d + i;
     k_pages[dst] = k[w];
-    v_pages[dst] = v[w];
+    // value pages may be stored transposed, [page][kv head][dim][page_size], for the matrix-core attention
+    v_pages[v_transposed ? (((size_t)page * nkv + h) * d + i) * page_size + off : dst] = v[w];
   }
 }
 
 extern "C" int ms_rope_store(void* qkv, const int* positions, const float* inv_freq, const int* slot_mapping,
                              void* k_pages, void* v_pages, int n_tokens, int num_heads, int num_kv_heads,
-                             int head_dim, int rot_dim, int page_size, int dtype, hipStream_t stream) {
+                             int head_dim, int rot_dim, int page_size, int v_transposed, int dtype,
+                             hipStream_t stream) {
   if (n_tokens <= 0) return MS_OK;
   if (num_heads < 0 || num_kv_heads < 0 || head_dim <= 0 || rot_dim < 0 || rot_dim > head_dim || (rot_dim & 1))
     return MS_BAD_ARG;
@@ -199,7 +202,7 @@ extern "C" int ms_rope_store(void* qkv, const int* positions, const float* inv_f
   if (k_pages && (page_size <= 0 || slot_mapping == nullptr)) return MS_BAD_ARG;
   if (rot_dim > 0 && (positions == nullptr || inv_freq == nullptr)) return MS_BAD_ARG;
   dim3 grid(n_tokens), block(256);
-#define LAUNCH(T) rope_store_kernel<T><<<grid, block, 0, stream>>>((T*)qkv, positions, inv_freq, slot_mapping, (T*)k_pages, (T*)v_pages, num_heads, num_kv_heads, head_dim, rot_dim, page_size)
+#define LAUNCH(T) rope_store_kernel<T><<<grid, block, 0, stream>>>((T*)qkv, positions, inv_freq, slot_mapping, (T*)k_pages, (T*)v_pages, num_heads, num_kv_heads, head_dim, rot_dim, page_size, v_transposed)
   if (dtype == MS_F32) LAUNCH(float);
   else if (dtype == MS_BF16) LAUNCH(bf16);
   else return MS_BAD_ARG;

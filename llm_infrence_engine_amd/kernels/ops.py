@@ -29,11 +29,18 @@ _SIGNATURES = {
     "ms_residual_add": [_c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr],
     "ms_silu_mul": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "ms_rope_store": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int,
-                      _c_int, _c_int, _c_ptr],
+                      _c_int, _c_int, _c_int, _c_ptr],
     "ms_gemm_generic": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ll, _c_ll, _c_ll, _c_int,
                         _c_int, _c_int, _c_ptr],
     "ms_paged_attention_generic": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ll,
-                                   _c_int, _c_int, _c_int, _c_int, _c_int, _c_ll, _c_float, _c_int, _c_int, _c_ptr],
+                                   _c_int, _c_int, _c_int, _c_int, _c_int, _c_ll, _c_float, _c_int, _c_int, _c_int,
+                                   _c_ptr],
+    "ms_attention_mfma_supported": [_c_int, _c_int],
+    "ms_paged_attention_mfma": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int,
+                                _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
+    "ms_paged_attention_mfma_decode": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ll,
+                                       _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int,
+                                       _c_int, _c_int, _c_ptr],
     "ms_sample": [_c_ptr, _c_ll, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
 }
 
@@ -155,12 +162,18 @@ def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def _v_shape(k_pages: torch.Tensor, v_transposed: bool):
+    P, nkv, page_size, d = k_pages.shape
+    return (P, nkv, d, page_size) if v_transposed else (P, nkv, page_size, d)
+
+
 def rope_store(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, rot_dim: int = 0,
                positions: Optional[torch.Tensor] = None, inv_freq: Optional[torch.Tensor] = None,
                slot_mapping: Optional[torch.Tensor] = None, k_pages: Optional[torch.Tensor] = None,
-               v_pages: Optional[torch.Tensor] = None) -> torch.Tensor:
+               v_pages: Optional[torch.Tensor] = None, v_transposed: bool = False) -> torch.Tensor:
     """Rotate q and k of ``qkv`` [N, (nh + 2 nkv) d] in place and store k, v into pages
-    [pages, nkv, page_size, d] at ``slot_mapping`` (page * page_size + offset)."""
+    [pages, nkv, page_size, d] at ``slot_mapping`` (page * page_size + offset); with ``v_transposed`` the
+    value pages are [pages, nkv, d, page_size]."""
     _check(qkv, "qkv", None, (None, (num_heads + 2 * num_kv_heads) * head_dim))
     N = qkv.shape[0]
     page_size = 0
@@ -171,11 +184,12 @@ def rope_store(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: i
         _check(inv_freq, "inv_freq", torch.float32, (rot_dim // 2,))
     if k_pages is not None:
         _check(k_pages, "k_pages", qkv.dtype, (None, num_kv_heads, None, head_dim))
-        _check(v_pages, "v_pages", qkv.dtype, tuple(k_pages.shape))
-        _check(slot_mapping, "slot_mapping", torch.int32, (N,))
         page_size = k_pages.shape[2]
+        _check(v_pages, "v_pages", qkv.dtype, _v_shape(k_pages, v_transposed))
+        _check(slot_mapping, "slot_mapping", torch.int32, (N,))
     _call("ms_rope_store", qkv.data_ptr(), _ptr(positions), _ptr(inv_freq), _ptr(slot_mapping), _ptr(k_pages),
-          _ptr(v_pages), N, num_heads, num_kv_heads, head_dim, rot_dim, page_size, _code(qkv.dtype), _stream())
+          _ptr(v_pages), N, num_heads, num_kv_heads, head_dim, rot_dim, page_size, int(v_transposed),
+          _code(qkv.dtype), _stream())
     return qkv
 
 
@@ -247,15 +261,16 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] =
 
 def paged_attention_generic(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
                             token_req: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, num_heads: int,
-                            scale: float, window: Optional[int] = None) -> torch.Tensor:
+                            scale: float, window: Optional[int] = None, v_transposed: bool = False) -> torch.Tensor:
     """out[n, h] = softmax(scale * q[n, h] . K[keys visible to n]) V, keys read in place from pages.
 
     q: [N, >= nh * d] (a row slice of the fused projection is fine), out [N, nh * d],
-    pages [P, nkv, page_size, d], block_table int32 [R, max_pages], token_req / positions int32 [N].
+    pages [P, nkv, page_size, d] (values [P, nkv, d, page_size] with ``v_transposed``), block_table int32
+    [R, max_pages], token_req / positions int32 [N].
     Token n sees keys 0..positions[n] of request token_req[n] (the last ``window`` of them if given)."""
     _check(k_pages, "k_pages")
     P, nkv, page_size, d = k_pages.shape
-    _check(v_pages, "v_pages", k_pages.dtype, tuple(k_pages.shape))
+    _check(v_pages, "v_pages", k_pages.dtype, _v_shape(k_pages, v_transposed))
     _check(q, "q", k_pages.dtype, contiguous=False)
     N = q.shape[0]
     if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < num_heads * d:
@@ -271,7 +286,57 @@ def paged_attention_generic(q: torch.Tensor, k_pages: torch.Tensor, v_pages: tor
     _call("ms_paged_attention_generic", q.data_ptr(), q.stride(0) if N > 1 else q.shape[1], k_pages.data_ptr(),
           v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], token_req.data_ptr(), positions.data_ptr(),
           out.data_ptr(), num_heads * d, N, num_heads, nkv, d, page_size, P, float(scale), int(window or 0),
-          _code(q.dtype), _stream())
+          int(v_transposed), _code(q.dtype), _stream())
+    return out
+
+
+def attention_mfma_supported(head_dim: int, page_size: int) -> bool:
+    return bool(_get("ms_attention_mfma_supported")(head_dim, page_size))
+
+
+DECODE_WAVES = 1024      # waves a decode step's attention aims to put on the chip
+MIN_BLOCKS_PER_SPLIT = 2  # of 32 keys
+
+
+def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, vt_pages: torch.Tensor, block_table: torch.Tensor,
+                         q_start: torch.Tensor, context_lens: torch.Tensor, out: torch.Tensor, num_heads: int,
+                         scale: float, max_q_len: int, max_context_len: int, window: Optional[int] = None) -> torch.Tensor:
+    """Matrix-core attention, bfloat16.  k_pages [P, nkv, page_size, d], vt_pages [P, nkv, d, page_size];
+    request r owns tokens q_start[r]..q_start[r+1]-1 and holds context_lens[r] keys after this step.  With
+    one token per request (``max_q_len`` 1) the keys are split over several waves and combined."""
+    _check(k_pages, "k_pages", torch.bfloat16)
+    P, nkv, page_size, d = k_pages.shape
+    _check(vt_pages, "vt_pages", torch.bfloat16, (P, nkv, d, page_size))
+    _check(q, "q", torch.bfloat16, contiguous=False)
+    N = q.shape[0]
+    if q.dim() != 2 or q.stride(1) != 1 or q.shape[1] < num_heads * d:
+        raise ValueError(f"q must be [N, >= {num_heads * d}] with unit stride along rows, got {list(q.shape)}")
+    _check(out, "out", torch.bfloat16, (N, num_heads * d))
+    _check(block_table, "block_table", torch.int32)
+    R = block_table.shape[0]
+    _check(q_start, "q_start", torch.int32, (R + 1,))
+    _check(context_lens, "context_lens", torch.int32, (R,))
+    if num_heads % nkv:
+        raise ValueError(f"{num_heads} query heads cannot share {nkv} key/value heads")
+    if max_q_len < 1 or max_context_len < max_q_len or max_context_len > block_table.shape[1] * page_size:
+        raise ValueError(f"max_q_len {max_q_len} / max_context_len {max_context_len} do not fit a table of "
+                         f"{block_table.shape[1]} pages of {page_size}")
+    q_stride = q.stride(0) if N > 1 else q.shape[1]
+    if max_q_len == 1 and num_heads // nkv <= 16:
+        blocks = (max_context_len - 1) // 32 + 1
+        want = max(1, min(blocks // MIN_BLOCKS_PER_SPLIT, DECODE_WAVES // max(1, R * nkv)))
+        per = -(-blocks // want)
+        n_splits = -(-blocks // per)
+        part_o = torch.empty((R, num_heads, n_splits, d), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((R, num_heads, n_splits, 2), dtype=torch.float32, device=q.device)
+        _call("ms_paged_attention_mfma_decode", q.data_ptr(), q_stride, k_pages.data_ptr(), vt_pages.data_ptr(),
+              block_table.data_ptr(), block_table.shape[1], q_start.data_ptr(), context_lens.data_ptr(), out.data_ptr(),
+              num_heads * d, part_o.data_ptr(), part_ml.data_ptr(), R, num_heads, nkv, d, page_size, float(scale),
+              int(window or 0), per * 32, n_splits, _stream())
+    else:
+        _call("ms_paged_attention_mfma", q.data_ptr(), q_stride, k_pages.data_ptr(), vt_pages.data_ptr(),
+              block_table.data_ptr(), block_table.shape[1], q_start.data_ptr(), context_lens.data_ptr(), out.data_ptr(),
+              num_heads * d, R, max_q_len, num_heads, nkv, d, page_size, float(scale), int(window or 0), _stream())
     return out
 
 
@@ -293,8 +358,15 @@ def sample(logits: torch.Tensor, out: torch.Tensor, temperature: Optional[torch.
     return out
 
 
-def paged_attention(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor, ctx,
-                    out: torch.Tensor, num_heads: int, scale: float, window: Optional[int] = None) -> torch.Tensor:
-    """Attention of a step's tokens (``ctx`` is its StepContext) over the pages; picks the kernel."""
-    return paged_attention_generic(q, k_pages, v_pages, block_table, ctx.token_req, ctx.positions, out, num_heads,
-                                   scale, window)
+def paged_attention(q: torch.Tensor, kv, ctx, out: torch.Tensor, num_heads: int, scale: float,
+                    window: Optional[int] = None) -> torch.Tensor:
+    """Attention of a step's tokens (``ctx``: its StepContext) over a run's pages (``kv``: its KVView).
+    bfloat16 with transposed value pages and a head size the matrix-core kernel has goes there; everything
+    else (float32, other head sizes, small pages) goes to the generic kernel."""
+    d, page_size = kv.k_pages.shape[3], kv.k_pages.shape[2]
+    if (q.dtype == torch.bfloat16 and kv.v_transposed and attention_mfma_supported(d, page_size)
+            and q.data_ptr() % 16 == 0 and (q.shape[0] == 1 or q.stride(0) % 8 == 0)):
+        return paged_attention_mfma(q, kv.k_pages, kv.v_pages, kv.block_table, ctx.q_start, ctx.context_lens, out,
+                                    num_heads, scale, ctx.max_q_len, ctx.max_context_len, window)
+    return paged_attention_generic(q, kv.k_pages, kv.v_pages, kv.block_table, ctx.token_req, ctx.positions, out,
+                                   num_heads, scale, window, kv.v_transposed)

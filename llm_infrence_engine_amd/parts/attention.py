@@ -70,9 +70,9 @@ class GQAttention(Mixer):
         if self.position is not None:
             self.position.encode_and_store(qkv, nh, nkv, d, ctx, kv)
         elif kv.store:
-            ops.rope_store(qkv, nh, nkv, d, 0, None, None, kv.slot_mapping, kv.k_pages, kv.v_pages)
+            ops.rope_store(qkv, nh, nkv, d, 0, None, None, kv.slot_mapping, kv.k_pages, kv.v_pages, kv.v_transposed)
         out = self.rt.empty(ctx.num_tokens, nh * d)
-        ops.paged_attention(qkv, kv.k_pages, kv.v_pages, kv.block_table, ctx, out, nh, self.scale, self.window)
+        ops.paged_attention(qkv, kv, ctx, out, nh, self.scale, self.window)
         return linear.linear_residual(out, self.w_o, bias=self.b_o)
 
 

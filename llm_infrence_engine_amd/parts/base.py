@@ -58,11 +58,12 @@ class KVView:
     """One run's pages of its cache group, with the group's tables for the step's requests."""
 
     k_pages: torch.Tensor      # [pages, nkv, page_size, d]
-    v_pages: torch.Tensor
+    v_pages: torch.Tensor      # the same, or [pages, nkv, d, page_size] if v_transposed
     block_table: torch.Tensor  # int32 [R, max pages]
     slot_mapping: torch.Tensor  # int32 [N]: page * page_size + offset of each token
     store: bool = True         # False: the run reads another run's cache and writes nothing
     window: Optional[int] = None
+    v_transposed: bool = False
 
 
 @dataclass

@@ -28,7 +28,7 @@ class RotaryHalf(PositionEncoding):
         store = kv is not None and kv.store
         ops.rope_store(qkv, num_heads, num_kv_heads, head_dim, self.rotary_dim, ctx.positions, self.inv_freq,
                        kv.slot_mapping if store else None, kv.k_pages if store else None,
-                       kv.v_pages if store else None)
+                       kv.v_pages if store else None, store and kv.v_transposed)
 
 
 class NoPosition(PositionEncoding):
@@ -40,7 +40,7 @@ class NoPosition(PositionEncoding):
     def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, ctx, kv):
         if kv is not None and kv.store:
             ops.rope_store(qkv, num_heads, num_kv_heads, head_dim, 0, None, None, kv.slot_mapping, kv.k_pages,
-                           kv.v_pages)
+                           kv.v_pages, kv.v_transposed)
 
 
 register_part("position", "rotary_half", RotaryHalf)

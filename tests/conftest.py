@@ -35,7 +35,14 @@ TINY_C = {
     "head_dim": 48, "intermediate_size": 200, "vocab_size": 331, "rope_theta": 50000.0,
     "rms_norm_eps": 3e-6, "tie_word_embeddings": False,
 }
-TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+# head size 64 and 7 query heads per key/value head, as the 0.5B model has: the sizes the matrix-core kernels serve
+TINY_D = {
+    "architectures": ["Qwen2ForCausalLM"],
+    "num_hidden_layers": 2, "hidden_size": 448, "num_attention_heads": 7, "num_key_value_heads": 1,
+    "intermediate_size": 264, "vocab_size": 509, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
+    "tie_word_embeddings": True,
+}
+TINY = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D}
 
 
 def plain_random_weights(cfg: dict, seed: int, std: float = 0.02, dtype=torch.float32) -> dict:

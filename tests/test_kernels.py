@@ -2,6 +2,8 @@
 engine's (odd widths, head sizes in steps of 16, vocabularies that are no power of two)."""
 import math
 
+import numpy as np
+
 import pytest
 import torch
 
@@ -331,3 +333,67 @@ def test_linear_picks_a_kernel_for_every_shape(ops):
             got = linear.linear_swiglu(a, linear.interleave_rows(gate, up))
             want = torch.nn.functional.silu(a.double() @ gate.double().T) * (a.double() @ up.double().T)
             torch.testing.assert_close(got.double(), want, **tol(dtype))
+
+
+def _paged_case(g, dtype, nh, nkv, d, page_size, ctx, qlen, fill):
+    """Random requests laid out in shuffled pages (values transposed); returns what the kernels take and
+    the plain answer.  Unused slots, the tails of last pages and the null page hold ``fill``."""
+    R = len(ctx)
+    pages_per = [-(-c // page_size) for c in ctx]
+    P = sum(pages_per) + 4
+    order = torch.randperm(P - 1, generator=g) + 1
+    kp = torch.full((P, nkv, page_size, d), fill, dtype=dtype)
+    vt = torch.full((P, nkv, d, page_size), fill, dtype=dtype)
+    table = torch.zeros(R, max(pages_per), dtype=torch.int32)
+    qs, ks, vs, q_rows, req, pos = [], [], [], [], [], []
+    used = 0
+    for r in range(R):
+        k = torch.randn(nkv, ctx[r], d, generator=g).to(dtype)
+        v = torch.randn(nkv, ctx[r], d, generator=g).to(dtype)
+        q = (torch.randn(nh, qlen[r], d, generator=g) * 2).to(dtype)
+        k[:, min(3, ctx[r] - 1)] = (q[::nh // nkv, -1].float() * 1.5).to(dtype)   # one far key stands out
+        pages = order[used:used + pages_per[r]]
+        used += pages_per[r]
+        table[r, :pages_per[r]] = pages.to(torch.int32)
+        for j in range(ctx[r]):
+            kp[pages[j // page_size], :, j % page_size] = k[:, j]
+            vt[pages[j // page_size], :, :, j % page_size] = v[:, j]
+        qs.append(q); ks.append(k); vs.append(v)
+        q_rows.append(q.transpose(0, 1).reshape(qlen[r], nh * d))
+        req += [r] * qlen[r]
+        pos += list(range(ctx[r] - qlen[r], ctx[r]))
+    return dict(kp=kp, vt=vt, table=table, q=torch.cat(q_rows), req=req, pos=pos, qs=qs, ks=ks, vs=vs)
+
+
+@pytest.mark.parametrize("nh,nkv,d,page_size,window", [(14, 2, 64, 16, None), (6, 2, 32, 16, None), (8, 8, 128, 32, None),
+                                                        (4, 1, 64, 16, 40), (28, 4, 128, 16, None), (5, 5, 32, 64, 100)])
+@pytest.mark.parametrize("shape", ["mixed", "decode"])
+def test_paged_attention_mfma(ops, nh, nkv, d, page_size, window, shape):
+    g = torch.Generator().manual_seed(nh * 100 + d)
+    if shape == "mixed":
+        ctx, qlen = [70, 133, 201, 300], [70, 9, 1, 150]
+    else:
+        ctx, qlen = [1, 31, 32, 33, 600, 1500, 64, 17], [1] * 8
+    c = _paged_case(g, torch.bfloat16, nh, nkv, d, page_size, ctx, qlen, float("nan"))
+    scale = 1.0 / math.sqrt(d)
+    want = torch.cat([attention_reference(q.double(), k.double(), v.double(), scale, window).transpose(0, 1).reshape(-1, nh * d)
+                      for q, k, v in zip(c["qs"], c["ks"], c["vs"])])
+    N = c["q"].shape[0]
+    wide = torch.zeros(N, (nh + 2 * nkv) * d, dtype=torch.bfloat16, device=DEV)
+    wide[:, :nh * d] = c["q"].to(DEV)
+    out = torch.full((N, nh * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    q_start = torch.tensor([0] + list(np.cumsum(qlen)), dtype=torch.int32, device=DEV)
+    ops.paged_attention_mfma(wide, c["kp"].to(DEV), c["vt"].to(DEV), c["table"].to(DEV), q_start,
+                             torch.tensor(ctx, dtype=torch.int32, device=DEV), out, nh, scale, max(qlen), max(ctx), window)
+    torch.testing.assert_close(out.double().cpu(), want, **tol(torch.bfloat16))
+    # the generic kernel reads the same transposed pages
+    out2 = torch.empty_like(out)
+    ops.paged_attention_generic(wide, c["kp"].to(DEV), c["vt"].to(DEV), c["table"].to(DEV),
+                                torch.tensor(c["req"], dtype=torch.int32, device=DEV),
+                                torch.tensor(c["pos"], dtype=torch.int32, device=DEV), out2, nh, scale, window, v_transposed=True)
+    torch.testing.assert_close(out2.double().cpu(), want, **tol(torch.bfloat16))
+
+
+def test_attention_mfma_support_matrix(ops):
+    assert ops.attention_mfma_supported(64, 16) and ops.attention_mfma_supported(128, 32)
+    assert not ops.attention_mfma_supported(48, 16) and not ops.attention_mfma_supported(64, 8)

@@ -210,7 +210,7 @@ def register_toys(fw):
             v = qkv.view(qkv.shape[0], nh + 2 * nkv, d)
             v[:, :nh + nkv] += self.table[(ctx.positions.long() % self.period)][:, None, :]
             if kv is not None and kv.store:
-                ops.rope_store(qkv, nh, nkv, d, 0, None, None, kv.slot_mapping, kv.k_pages, kv.v_pages)
+                ops.rope_store(qkv, nh, nkv, d, 0, None, None, kv.slot_mapping, kv.k_pages, kv.v_pages, kv.v_transposed)
 
     @dataclass(frozen=True)
     class ToyConfig:

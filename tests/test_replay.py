@@ -75,23 +75,27 @@ def compare(got, want, dtype, requests):
     return worst
 
 
-LENGTHS = {"A": [5, 11, 17, 70, 129, 40, 200], "B": [1, 9, 23, 40, 150, 77, 64], "C": [33, 2, 96, 180, 50, 65, 31]}
-PAGE = {"A": 4, "B": 8, "C": 16}
+LENGTHS = {"A": [5, 11, 17, 70, 129, 40, 200], "B": [1, 9, 23, 40, 150, 77, 64], "C": [33, 2, 96, 180, 50, 65, 31],
+           "D": [70, 3, 160, 33, 97, 240, 64]}
+# pages of 4 and 8 tokens go to the generic kernels in both types; with pages of 16 and 32, B (head size 32)
+# and D (head size 64, 7 query heads per key/value head) run the matrix-core attention in bfloat16
+SETUPS = {"A": ("A", 4), "B": ("B", 8), "C": ("C", 16), "B16": ("B", 16), "D": ("D", 16), "D32": ("D", 32)}
+STD = {"A": 0.15, "B": 0.15, "C": 0.15, "D": 0.08}
 
 
-@pytest.fixture(scope="module", params=["A", "B", "C"])
+@pytest.fixture(scope="module", params=list(SETUPS))
 def setup(request, tmp_path_factory):
-    name = request.param
-    # std 0.15: attention scores of order one, so that a wrong key, position or page changes the logits
-    model_dir = make_model(tmp_path_factory, name, std=0.15, seed={"A": 0, "B": 1, "C": 2}[name])
+    name, page = SETUPS[request.param]
+    # weights large enough for attention scores of order one, so that a wrong key, position or page changes the logits
+    model_dir = make_model(tmp_path_factory, name, std=STD[name], seed={"A": 0, "B": 1, "C": 2, "D": 3}[name])
     reqs = make_requests(TINY[name]["vocab_size"], LENGTHS[name], seed=ord(name))
-    return name, model_dir, reqs, oracle(model_dir, reqs)
+    return (name, page), model_dir, reqs, oracle(model_dir, reqs)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("mode", ["whole", "bulk_then_single", "changing_portions", "mixed"])
 def test_replay_modes(setup, tmp_path, dtype, mode):
-    name, model_dir, reqs, want = setup
+    (name, page), model_dir, reqs, want = setup
     up = lambda n: -(-n // 64) * 64
     if mode == "mixed":
         # room for the longest request and a little more: requests wait for pages, and freed pages are used again
@@ -100,12 +104,12 @@ def test_replay_modes(setup, tmp_path, dtype, mode):
     else:
         max_tokens = up(max(len(t) for t in reqs.values()))
         steps = getattr(traces, mode)(reqs)
-    run_replay(model_dir, dtype, steps, tmp_path, max_tokens, page_size=PAGE[name])
+    run_replay(model_dir, dtype, steps, tmp_path, max_tokens, page_size=page)
     got = traces.collect(steps, tmp_path, TINY[name]["vocab_size"])
     if mode != "mixed":
         assert len(got) == sum(len(t) for t in reqs.values())
     worst = compare(got, want, dtype, reqs)
-    print(f"tiny {name} {dtype} {mode}: worst error is {worst:.3f} of its bound over {len(got)} places")
+    print(f"tiny {name} page {page} {dtype} {mode}: worst error is {worst:.3f} of its bound over {len(got)} places")
 
 
 def test_baseline_distribution_weights_too(tmp_path_factory, tmp_path):
