@@ -47,8 +47,11 @@ int ms_paged_attention_mfma_decode(const void* q, long long q_stride, const void
                                    const int* block_table, int table_stride, const int* q_start,
                                    const int* context_lens, void* out, long long out_stride, void* part_o,
                                    void* part_ml, int n_requests, int num_heads, int num_kv_heads, int head_dim,
-                                   int page_size, float scale, int window, int keys_per_split, int n_splits,
+                                   int page_size, float scale, int window, int min_blocks, int n_splits,
                                    hipStream_t stream);
+
+int ms_argmax(const float* logits, long long ld, int n_rows, int vocab, float* scratch_val, int* scratch_idx,
+              int n_chunks, int* out, hipStream_t stream);
 
 int ms_sample(const float* logits, long long ld, int n_rows, int vocab, const float* temperature, const int* top_k,
               const float* top_p, const unsigned long long* seeds, const int* draw_index, int* out,

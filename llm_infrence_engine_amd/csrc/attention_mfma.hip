@@ -65,7 +65,7 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
                       const int* __restrict__ q_start, const int* __restrict__ context_lens,
                       bf16* __restrict__ out, size_t out_stride, float* __restrict__ part_o,
                       float* __restrict__ part_ml, int nh, int nkv, int page_size, float scale_log2e, int window,
-                      int keys_per_split, int n_splits) {
+                      int min_blocks, int n_splits) {
   const int lane = threadIdx.x, col16 = lane & 15, kq = lane >> 4;
   const int r = blockIdx.z, g = blockIdx.y;
   const int rep = nh / nkv;
@@ -84,7 +84,8 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
   if (window > 0) key_lo = max(0, start_pos + c0 / rep - window + 1);
   int blk_begin = key_lo / 32, blk_end = key_hi / 32 + 1;
   if (SPLIT) {
-    const int per = keys_per_split / 32;
+    // every request spreads its own key blocks evenly over the splits (at least min_blocks each)
+    const int per = max(min_blocks, (blk_end - blk_begin + n_splits - 1) / n_splits);
     blk_begin += blockIdx.x * per;
     blk_end = min(blk_end, blk_begin + per);
     if (blk_begin >= blk_end) return;
@@ -224,12 +225,13 @@ template <int D>
 __global__ void attention_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                          const int* __restrict__ q_start, const int* __restrict__ context_lens,
                                          bf16* __restrict__ out, size_t out_stride, int nh, int window,
-                                         int keys_per_split, int n_splits) {
+                                         int min_blocks, int n_splits) {
   const int r = blockIdx.x / nh, h = blockIdx.x % nh;
   const int key_hi = context_lens[r] - 1;
   const int key_lo = window > 0 ? max(0, key_hi - window + 1) : 0;
   const int blocks = key_hi / 32 + 1 - key_lo / 32;
-  const int used = min(n_splits, (blocks * 32 + keys_per_split - 1) / keys_per_split);
+  const int per = max(min_blocks, (blocks + n_splits - 1) / n_splits);
+  const int used = (blocks + per - 1) / per;
   const size_t slot0 = ((size_t)r * nh + h) * n_splits;
   float big = -INFINITY;
   for (int s = 0; s < used; ++s) big = fmaxf(big, part_ml[(slot0 + s) * 2]);
@@ -258,11 +260,11 @@ int launch_general(const bf16* q, size_t q_stride, const bf16* k, const bf16* vt
 template <int D>
 int launch_decode(const bf16* q, size_t q_stride, const bf16* k, const bf16* vt, const int* table, int table_stride,
                   const int* q_start, const int* ctx, bf16* out, size_t out_stride, float* part_o, float* part_ml,
-                  int n_requests, int nh, int nkv, int page_size, float scale, int window, int keys_per_split,
+                  int n_requests, int nh, int nkv, int page_size, float scale, int window, int min_blocks,
                   int n_splits, hipStream_t stream) {
   dim3 grid(n_splits, nkv, n_requests), block(MS_WAVE);
-  attention_mfma_kernel<D, 1, true><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, q_start, ctx, out, out_stride, part_o, part_ml, nh, nkv, page_size, scale * 1.4426950408889634f, window, keys_per_split, n_splits);
-  attention_combine_kernel<D><<<dim3(n_requests * nh), dim3(D < 64 ? 64 : D), 0, stream>>>(part_o, part_ml, q_start, ctx, out, out_stride, nh, window, keys_per_split, n_splits);
+  attention_mfma_kernel<D, 1, true><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, q_start, ctx, out, out_stride, part_o, part_ml, nh, nkv, page_size, scale * 1.4426950408889634f, window, min_blocks, n_splits);
+  attention_combine_kernel<D><<<dim3(n_requests * nh), dim3(D < 64 ? 64 : D), 0, stream>>>(part_o, part_ml, q_start, ctx, out, out_stride, nh, window, min_blocks, n_splits);
   return ms_launch_status();
 }
 
@@ -295,22 +297,24 @@ extern "C" int ms_paged_attention_mfma(const void* q, long long q_stride, const 
 }
 
 // Decode shape: every request has exactly one token and the group (num_heads / num_kv_heads) is at most 16.
-// part_o: float [R, nh, n_splits, d], part_ml: float [R, nh, n_splits, 2]; keys_per_split a multiple of 32.
+// part_o: float [R, nh, n_splits, d], part_ml: float [R, nh, n_splits, 2].  Each request spreads its blocks of
+// 32 keys evenly over the n_splits waves, at least min_blocks to a wave, so the launch does not depend on
+// how long the contexts are.
 extern "C" int ms_paged_attention_mfma_decode(const void* q, long long q_stride, const void* k_pages,
                                               const void* vt_pages, const int* block_table, int table_stride,
                                               const int* q_start, const int* context_lens, void* out,
                                               long long out_stride, void* part_o, void* part_ml, int n_requests,
                                               int num_heads, int num_kv_heads, int head_dim, int page_size,
-                                              float scale, int window, int keys_per_split, int n_splits,
+                                              float scale, int window, int min_blocks, int n_splits,
                                               hipStream_t stream) {
   if (n_requests <= 0) return MS_OK;
   if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads || table_stride <= 0) return MS_BAD_ARG;
   if (num_heads / num_kv_heads > 16) return MS_UNSUPPORTED;
   if (!ms_attention_mfma_supported(head_dim, page_size)) return MS_UNSUPPORTED;
-  if (keys_per_split <= 0 || keys_per_split % 32 || n_splits <= 0 || n_splits > 65535) return MS_BAD_ARG;
+  if (min_blocks <= 0 || n_splits <= 0 || n_splits > 65535) return MS_BAD_ARG;
   if (q_stride % 8 || out_stride % 4 || ((uintptr_t)q % 16) || ((uintptr_t)out % 8) || ((uintptr_t)part_o % 16)) return MS_UNSUPPORTED;
   if (n_requests > 65535 || num_kv_heads > 65535) return MS_UNSUPPORTED;
-#define GO(D) return launch_decode<D>((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)vt_pages, block_table, table_stride, q_start, context_lens, (bf16*)out, out_stride, (float*)part_o, (float*)part_ml, n_requests, num_heads, num_kv_heads, page_size, scale, window, keys_per_split, n_splits, stream)
+#define GO(D) return launch_decode<D>((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)vt_pages, block_table, table_stride, q_start, context_lens, (bf16*)out, out_stride, (float*)part_o, (float*)part_ml, n_requests, num_heads, num_kv_heads, page_size, scale, window, min_blocks, n_splits, stream)
   if (head_dim == 32) GO(32);
   if (head_dim == 64) GO(64);
   GO(128);

@@ -1,13 +1,15 @@
 // out[M,N] = A[M,K] . W[N,K]^T for few rows (M <= 64, a decode step's tokens), bfloat16 in, float accumulation
 // on the matrix cores (v_mfma_f32_16x16x32_bf16).  The product is bound by reading W once from HBM, so
-// the kernel is shaped for memory parallelism: a block owns 16 output features and a slice of K; its four
-// waves take interleaved 32-wide k-steps, each lane streaming 16 bytes of one weight row per step, and add
-// their accumulators through LDS in a fixed order.  The weight tile is the MFMA's A operand and the
+// the kernel is shaped for memory parallelism: a block owns 16 output features and a slice of K; its
+// waves (4, 8 or 16 of them, more when there are few features so that the chip still fills) take
+// interleaved 32-wide k-steps, each lane streaming 16 bytes of one weight row per step, and add their
+// accumulators through LDS in a fixed order.  The weight tile is the MFMA's A operand and the
 // activation tile its B operand, so a lane ends up with 4 consecutive output features of one token.
 //
 // Epilogues: plain (+ bias) to bfloat16 or float; gated activation over interleaved rows (2j: gate j,
 // 2j+1: up j) writing silu(gate) * up; float partial sums [splits, M, N] when K is split over blocks
-// (whoever consumes them adds them up in order, so results do not depend on timing).
+// (whoever consumes them adds them up in order, so results do not depend on timing); and the residual
+// sum, out[m, n] += product (+ bias) on a float matrix, each element owned by one lane: no atomics.
 #include "common.h"
 #include "api.h"
 
@@ -16,14 +18,14 @@ namespace {
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
-enum { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_PARTIAL = 2 };
+enum { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_PARTIAL = 2, EPI_RESIDUAL = 3 };
 
-template <int MT, int EPI, typename TO>
-__global__ void __launch_bounds__(256)
+template <int MT, int EPI, typename TO, int WAVES>
+__global__ void __launch_bounds__(WAVES * MS_WAVE)
 gemm_skinny_kernel(const bf16* __restrict__ A, size_t lda, const bf16* __restrict__ W, size_t ldw,
                    const float* __restrict__ bias, TO* __restrict__ out, size_t ldo, int M, int N, int K,
                    int steps_per_split) {
-  __shared__ f32x4 red[3][MT][MS_WAVE];
+  __shared__ f32x4 red[WAVES - 1][MT][MS_WAVE];
   const int lane = threadIdx.x & (MS_WAVE - 1), wave = threadIdx.x / MS_WAVE;
   const int col = lane & 15, kq = lane >> 4;
   const int n0 = blockIdx.x * 16;
@@ -42,7 +44,7 @@ gemm_skinny_kernel(const bf16* __restrict__ A, size_t lda, const bf16* __restric
   for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
 #pragma unroll 4
-  for (int s = step_begin + wave; s < step_end; s += 4) {
+  for (int s = step_begin + wave; s < step_end; s += WAVES) {
     const int k = s * 32;
     bf16x8 wv = {0, 0, 0, 0, 0, 0, 0, 0};
     const bool in = k + kq * 8 < K;  // K is a multiple of 8: a lane's 8 values are all inside or all outside
@@ -64,7 +66,7 @@ gemm_skinny_kernel(const bf16* __restrict__ A, size_t lda, const bf16* __restric
 #pragma unroll
   for (int t = 0; t < MT; ++t)
 #pragma unroll
-    for (int w = 0; w < 3; ++w) acc[t] += red[w][t][lane];
+    for (int w = 0; w < WAVES - 1; ++w) acc[t] += red[w][t][lane];
 
   // lane holds out[m = t*16 + col][n = n0 + kq*4 + r], r = 0..3
   const int nb = n0 + kq * 4;
@@ -86,7 +88,11 @@ gemm_skinny_kernel(const bf16* __restrict__ A, size_t lda, const bf16* __restric
       const bool add_bias = bias != nullptr && (EPI != EPI_PARTIAL || blockIdx.y == 0);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        if (nb + r < N) o[r] = from_float<TO>(acc[t][r] + (add_bias ? bias[nb + r] : 0.f));
+        if (nb + r < N) {
+          float v = acc[t][r] + (add_bias ? bias[nb + r] : 0.f);
+          if (EPI == EPI_RESIDUAL) v += to_float(o[r]);
+          o[r] = from_float<TO>(v);
+        }
       }
     }
   }
@@ -97,13 +103,19 @@ int launch_mt(const bf16* A, size_t lda, const bf16* W, size_t ldw, const float*
               int N, int K, int splits, hipStream_t stream) {
   const int total_steps = (K + 31) / 32;
   const int per = (total_steps + splits - 1) / splits;
-  dim3 grid((N + 15) / 16, (total_steps + per - 1) / per), block(256);
-#define GO(MT) gemm_skinny_kernel<MT, EPI, TO><<<grid, block, 0, stream>>>(A, lda, W, ldw, bias, out, ldo, M, N, K, per)
+  const int tiles = (N + 15) / 16;
+  dim3 grid(tiles, (total_steps + per - 1) / per);
+  // enough waves to fill 256 CUs even when there are few features, but at least two k-steps per wave
+  int waves = 4;
+  while (waves < 16 && (long long)tiles * grid.y * waves < 1024 && per >= waves * 4) waves *= 2;
+#define GO2(MT, WV) gemm_skinny_kernel<MT, EPI, TO, WV><<<grid, dim3(WV * MS_WAVE), 0, stream>>>(A, lda, W, ldw, bias, out, ldo, M, N, K, per)
+#define GO(MT) do { if (waves == 4) GO2(MT, 4); else if (waves == 8) GO2(MT, 8); else GO2(MT, 16); } while (0)
   if (M <= 16) GO(1);
   else if (M <= 32) GO(2);
   else if (M <= 48) GO(3);
   else GO(4);
 #undef GO
+#undef GO2
   return ms_launch_status();
 }
 
@@ -120,6 +132,7 @@ extern "C" int ms_gemm_skinny_splits(int K, int splits) {
 // epilogue 0: out[M,N] (out_dtype float or bfloat16) = product + bias
 // epilogue 1: out[M,N/2] bfloat16 = silu(gate) * up over interleaved rows of W (no bias)
 // epilogue 2: out[splits,M,N] float partial sums (bias goes into split 0); `splits` as ms_gemm_skinny_splits gives
+// epilogue 3: out[M,N] float += product + bias
 extern "C" int ms_gemm_skinny(const void* A, long long lda, const void* W, long long ldw, const float* bias, void* out,
                               long long ldo, int M, int N, int K, int epilogue, int splits, int out_dtype,
                               hipStream_t stream) {
@@ -138,6 +151,10 @@ extern "C" int ms_gemm_skinny(const void* A, long long lda, const void* W, long 
   if (epilogue == EPI_SWIGLU) {
     if (N % 2 || ldo < N / 2 || out_dtype != MS_BF16 || bias) return MS_BAD_ARG;
     return launch_mt<EPI_SWIGLU, bf16>(a, lda, w, ldw, nullptr, (bf16*)out, ldo, M, N, K, 1, stream);
+  }
+  if (epilogue == EPI_RESIDUAL) {
+    if (ldo < N || out_dtype != MS_F32) return MS_BAD_ARG;
+    return launch_mt<EPI_RESIDUAL, float>(a, lda, w, ldw, bias, (float*)out, ldo, M, N, K, 1, stream);
   }
   if (epilogue == EPI_PARTIAL) {
     if (ldo < N || out_dtype != MS_F32 || splits < 1) return MS_BAD_ARG;

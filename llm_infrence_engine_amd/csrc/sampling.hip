@@ -152,7 +152,56 @@ sample_kernel(const float* __restrict__ logits, size_t ld, int V, const float* _
   if (threadIdx.x == 0) out[r] = chosen >= 0 ? chosen : top.i;  // rounding left no owner: the maximum is always kept
 }
 
+// First maximum of a row in two stages, so that a few rows still use the whole chip: stage 1 finds the best
+// of each of n_chunks slices of the row, stage 2 the best of those (larger value, then smaller index).
+__global__ void __launch_bounds__(256)
+argmax_chunks_kernel(const float* __restrict__ logits, size_t ld, int V, int n_chunks, float* __restrict__ val,
+                     int* __restrict__ idx) {
+  __shared__ MaxIdx red[4];
+  const int r = blockIdx.y, c = blockIdx.x;
+  const int len = (V + n_chunks - 1) / n_chunks;
+  const int begin = c * len, end = min(V, begin + len);
+  const float* row = logits + (size_t)r * ld;
+  MaxIdx best = {-INFINITY, 0x7fffffff};
+  for (int i = begin + threadIdx.x; i < end; i += blockDim.x) best = better(best, MaxIdx{row[i], i});
+  for (int o = MS_WAVE / 2; o > 0; o >>= 1) {
+    MaxIdx other = {__shfl_xor(best.v, o, MS_WAVE), __shfl_xor(best.i, o, MS_WAVE)};
+    best = better(best, other);
+  }
+  if ((threadIdx.x & (MS_WAVE - 1)) == 0) red[threadIdx.x / MS_WAVE] = best;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 4; ++w) best = better(best, red[w]);
+    val[(size_t)r * n_chunks + c] = best.v;
+    idx[(size_t)r * n_chunks + c] = best.i;
+  }
+}
+
+__global__ void __launch_bounds__(MS_WAVE)
+argmax_final_kernel(const float* __restrict__ val, const int* __restrict__ idx, int n_chunks, int* __restrict__ out) {
+  const int r = blockIdx.x;
+  MaxIdx best = {-INFINITY, 0x7fffffff};
+  for (int c = threadIdx.x; c < n_chunks; c += MS_WAVE)
+    best = better(best, MaxIdx{val[(size_t)r * n_chunks + c], idx[(size_t)r * n_chunks + c]});
+  for (int o = MS_WAVE / 2; o > 0; o >>= 1) {
+    MaxIdx other = {__shfl_xor(best.v, o, MS_WAVE), __shfl_xor(best.i, o, MS_WAVE)};
+    best = better(best, other);
+  }
+  if (threadIdx.x == 0) out[r] = best.i == 0x7fffffff ? 0 : best.i;
+}
+
 }  // namespace
+
+// out[r] = first index of the maximum of logits[r, :].  scratch_val / scratch_idx: [n_rows, n_chunks].
+extern "C" int ms_argmax(const float* logits, long long ld, int n_rows, int vocab, float* scratch_val,
+                         int* scratch_idx, int n_chunks, int* out, hipStream_t stream) {
+  if (n_rows <= 0) return MS_OK;
+  if (vocab <= 0 || ld < vocab || n_chunks <= 0 || n_rows > 65535) return MS_BAD_ARG;
+  argmax_chunks_kernel<<<dim3(n_chunks, n_rows), dim3(256), 0, stream>>>(logits, (size_t)ld, vocab, n_chunks,
+                                                                          scratch_val, scratch_idx);
+  argmax_final_kernel<<<dim3(n_rows), dim3(MS_WAVE), 0, stream>>>(scratch_val, scratch_idx, n_chunks, out);
+  return ms_launch_status();
+}
 
 extern "C" int ms_sample(const float* logits, long long ld, int n_rows, int vocab, const float* temperature,
                          const int* top_k, const float* top_p, const unsigned long long* seeds,

@@ -57,15 +57,14 @@ def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None
     return ops.gemm_generic(a, w, out, bias=bias)
 
 
-def linear_residual(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """A product that is about to be added to the residual stream: [M, N], or float partial sums [S, M, N]
-    over slices of K that the next norm adds up in order (few rows: more blocks to pull the weights)."""
-    if a.dtype == torch.bfloat16 and ops.skinny_ok(a, w):
-        n_tiles = -(-w.shape[0] // 16)
-        steps = -(-a.shape[1] // 32)
-        splits = max(1, min(-(-512 // n_tiles), steps // 4))
-        if splits > 1:
-            return ops.gemm_skinny(a, w, bias, ops.EPI_PARTIAL, splits=splits)
+def linear_residual(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                    residual: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """A product that is to be added to the float residual stream.  With few rows the kernel adds it into
+    ``residual`` itself (each element by one lane, no atomics) and None is returned; otherwise the product
+    [M, N] is returned for the next norm to add."""
+    if residual is not None and a.dtype == torch.bfloat16 and ops.skinny_ok(a, w):
+        ops.gemm_skinny(a, w, bias, ops.EPI_RESIDUAL, residual=residual)
+        return None
     return linear(a, w, bias)
 
 

@@ -41,6 +41,7 @@ _SIGNATURES = {
     "ms_paged_attention_mfma_decode": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ll,
                                        _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int,
                                        _c_int, _c_int, _c_ptr],
+    "ms_argmax": [_c_ptr, _c_ll, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr],
     "ms_sample": [_c_ptr, _c_ll, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
 }
 
@@ -216,7 +217,7 @@ def gemm_generic(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Opti
 
 
 SKINNY_MAX_ROWS = 64
-EPI_STORE, EPI_SWIGLU, EPI_PARTIAL = 0, 1, 2
+EPI_STORE, EPI_SWIGLU, EPI_PARTIAL, EPI_RESIDUAL = 0, 1, 2, 3
 
 
 def skinny_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
@@ -227,10 +228,12 @@ def skinny_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
 
 
 def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, epilogue: int = EPI_STORE,
-                splits: int = 1, out_dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+                splits: int = 1, out_dtype: torch.dtype = torch.bfloat16,
+                residual: Optional[torch.Tensor] = None) -> torch.Tensor:
     """a [M <= 64, K] @ w [N, K].T on the matrix cores, bfloat16 in.  Epilogues: EPI_STORE -> [M, N] (+ bias);
     EPI_SWIGLU -> [M, N / 2] = silu(even rows' products) * odd rows' products; EPI_PARTIAL -> float [S, M, N]
-    partial sums over slices of K (bias in the first), to be added in order by the consumer."""
+    partial sums over slices of K (bias in the first), to be added in order by the consumer; EPI_RESIDUAL ->
+    ``residual`` (float [M, N]) += product + bias, in place."""
     _check(a, "a", torch.bfloat16, contiguous=False)
     _check(w, "w", torch.bfloat16)
     if a.dim() != 2 or w.dim() != 2 or a.shape[1] != w.shape[1]:
@@ -249,6 +252,9 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] =
         if N % 2 or bias is not None:
             raise ValueError("the gated epilogue needs an even number of weight rows and no bias")
         out, ldo, out_dtype = torch.empty((M, N // 2), dtype=torch.bfloat16, device=a.device), N // 2, torch.bfloat16
+    elif epilogue == EPI_RESIDUAL:
+        _check(residual, "residual", torch.float32, (M, N))
+        out, ldo, out_dtype = residual, N, torch.float32
     elif epilogue == EPI_PARTIAL:
         splits = _get("ms_gemm_skinny_splits")(K, splits)
         out, ldo, out_dtype = torch.empty((splits, M, N), dtype=torch.float32, device=a.device), N, torch.float32
@@ -295,6 +301,7 @@ def attention_mfma_supported(head_dim: int, page_size: int) -> bool:
 
 
 DECODE_WAVES = 1024      # waves a decode step's attention aims to put on the chip
+MAX_SPLITS = 32
 MIN_BLOCKS_PER_SPLIT = 2  # of 32 keys
 
 
@@ -323,16 +330,15 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, vt_pages: torch
                          f"{block_table.shape[1]} pages of {page_size}")
     q_stride = q.stride(0) if N > 1 else q.shape[1]
     if max_q_len == 1 and num_heads // nkv <= 16:
-        blocks = (max_context_len - 1) // 32 + 1
-        want = max(1, min(blocks // MIN_BLOCKS_PER_SPLIT, DECODE_WAVES // max(1, R * nkv)))
-        per = -(-blocks // want)
-        n_splits = -(-blocks // per)
+        # a launch constant of the batch size alone (so that a captured graph stays valid as contexts grow):
+        # every request spreads its own key blocks over the splits inside the kernel
+        n_splits = max(1, min(MAX_SPLITS, DECODE_WAVES // max(1, R * nkv)))
         part_o = torch.empty((R, num_heads, n_splits, d), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((R, num_heads, n_splits, 2), dtype=torch.float32, device=q.device)
         _call("ms_paged_attention_mfma_decode", q.data_ptr(), q_stride, k_pages.data_ptr(), vt_pages.data_ptr(),
               block_table.data_ptr(), block_table.shape[1], q_start.data_ptr(), context_lens.data_ptr(), out.data_ptr(),
               num_heads * d, part_o.data_ptr(), part_ml.data_ptr(), R, num_heads, nkv, d, page_size, float(scale),
-              int(window or 0), per * 32, n_splits, _stream())
+              int(window or 0), MIN_BLOCKS_PER_SPLIT, n_splits, _stream())
     else:
         _call("ms_paged_attention_mfma", q.data_ptr(), q_stride, k_pages.data_ptr(), vt_pages.data_ptr(),
               block_table.data_ptr(), block_table.shape[1], q_start.data_ptr(), context_lens.data_ptr(), out.data_ptr(),
@@ -348,6 +354,12 @@ def sample(logits: torch.Tensor, out: torch.Tensor, temperature: Optional[torch.
     _check(logits, "logits", torch.float32)
     M, V = logits.shape
     _check(out, "out", torch.int32, (M,))
+    if temperature is None and M <= 65535:
+        n_chunks = max(1, min(128, V // 1024))
+        val = torch.empty((M, n_chunks), dtype=torch.float32, device=logits.device)
+        idx = torch.empty((M, n_chunks), dtype=torch.int32, device=logits.device)
+        _call("ms_argmax", logits.data_ptr(), V, M, V, val.data_ptr(), idx.data_ptr(), n_chunks, out.data_ptr(), _stream())
+        return out
     for t, name, dt in ((temperature, "temperature", torch.float32), (top_k, "top_k", torch.int32),
                         (top_p, "top_p", torch.float32), (seeds, "seeds", torch.int64),
                         (draw_index, "draw_index", torch.int32)):

@@ -63,6 +63,9 @@ class GQAttention(Mixer):
 
     # ---- step
     def forward(self, h, ctx, kv, state):
+        return self.forward_residual(h, ctx, kv, state, None)
+
+    def forward_residual(self, h, ctx, kv, state, x):
         if kv is None:
             raise RuntimeError("attention needs a key/value cache view")
         nh, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
@@ -73,7 +76,7 @@ class GQAttention(Mixer):
             ops.rope_store(qkv, nh, nkv, d, 0, None, None, kv.slot_mapping, kv.k_pages, kv.v_pages, kv.v_transposed)
         out = self.rt.empty(ctx.num_tokens, nh * d)
         ops.paged_attention(qkv, kv, ctx, out, nh, self.scale, self.window)
-        return linear.linear_residual(out, self.w_o, bias=self.b_o)
+        return linear.linear_residual(out, self.w_o, self.b_o, x)
 
 
 register_part("mixer", "gqa_attention", GQAttention)

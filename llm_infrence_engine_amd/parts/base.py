@@ -6,7 +6,9 @@ it is in.  Five kinds are chosen layer by layer:
 ``Norm``              forward(x, delta, rows, write_back) -> activations         (x: the float residual stream)
 ``PositionEncoding``  encode_and_store(qkv, nh, nkv, d, ctx, kv)                 (belongs to a mixer)
 ``Mixer``             forward(h, ctx, kv, state) -> [N, hidden]                  (attention here)
-``FeedForward``       forward(h, ctx) -> [N, hidden]    (both may return float partial sums [S, N, hidden])
+``FeedForward``       forward(h, ctx) -> [N, hidden]
+                      (both also forward_residual(..., x): add into the residual stream x and return None,
+                      or return the addend; the default returns forward's result)
 ``Block``             forward(x, pending, ctx, kv, state) -> pending             (the arrangement of the four)
 
 plus ``Embedding`` and ``Head`` at the model's ends.  Every part lists the checkpoint tensors it wants
@@ -141,10 +143,20 @@ class Mixer(Part):
                 state: Optional[StateView]) -> torch.Tensor:
         raise NotImplementedError
 
+    def forward_residual(self, h: torch.Tensor, ctx: StepContext, kv: Optional[KVView], state: Optional[StateView],
+                         x: torch.Tensor) -> Optional[torch.Tensor]:
+        """What the block calls.  A part whose last kernel can add into the float residual stream ``x`` does so
+        and returns None; the default returns ``forward``'s result for the next norm to add."""
+        return self.forward(h, ctx, kv, state)
+
 
 class FeedForward(Part):
     def forward(self, h: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         raise NotImplementedError
+
+    def forward_residual(self, h: torch.Tensor, ctx: StepContext, x: torch.Tensor) -> Optional[torch.Tensor]:
+        """As ``Mixer.forward_residual``."""
+        return self.forward(h, ctx)
 
 
 class Block(Part):

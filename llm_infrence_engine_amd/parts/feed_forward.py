@@ -24,7 +24,10 @@ class SwiGLU(FeedForward):
         self.w_down = linear.prepare_weight(d)
 
     def forward(self, h, ctx):
-        return linear.linear_residual(linear.linear_swiglu(h, self.w_gate_up), self.w_down)
+        return self.forward_residual(h, ctx, None)
+
+    def forward_residual(self, h, ctx, x):
+        return linear.linear_residual(linear.linear_swiglu(h, self.w_gate_up), self.w_down, None, x)
 
 
 register_part("feed_forward", "swiglu", SwiGLU)

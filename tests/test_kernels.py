@@ -289,6 +289,10 @@ def test_gemm_skinny(ops, M, N, K):
         parts = ops.gemm_skinny(a, w, bias, ops.EPI_PARTIAL, splits=splits)
         assert parts.dim() == 3 and parts.shape[1:] == (M, N) and parts.shape[0] <= splits
         torch.testing.assert_close(parts.double().sum(0), want + bias.double(), atol=2e-5, rtol=2e-5)
+    x = torch.randn(M, N, generator=g).to(DEV)
+    x0 = x.clone()
+    ops.gemm_skinny(a, w, bias, ops.EPI_RESIDUAL, residual=x)
+    torch.testing.assert_close(x.double(), x0.double() + want + bias.double(), atol=2e-5, rtol=2e-5)
     if N % 2 == 0:
         act = ops.gemm_skinny(a, w, None, ops.EPI_SWIGLU)
         wantact = torch.nn.functional.silu(want[:, 0::2]) * want[:, 1::2]
@@ -323,9 +327,12 @@ def test_linear_picks_a_kernel_for_every_shape(ops):
             lg = linear.linear(a, w, b, out_dtype=torch.float32)
             assert lg.dtype == torch.float32
             torch.testing.assert_close(lg.double(), want, **(tol(torch.float32) if dtype == torch.float32 or M <= 64 else tol(dtype)))
-            r = linear.linear_residual(a, w, b)
-            r = r.double().sum(0) if r.dim() == 3 else r.double()
-            torch.testing.assert_close(r, want, **tol(dtype))
+            x = torch.randn(M, N, generator=g).to(DEV)
+            x0 = x.clone()
+            r = linear.linear_residual(a, w, b, x)
+            got = x.double() - x0.double() if r is None else r.double()
+            assert (r is None) == (dtype == torch.bfloat16 and M <= 64 and K % 8 == 0)
+            torch.testing.assert_close(got, want, **tol(dtype))
         for M in (4, 90):
             a = torch.randn(M, 72, generator=g).to(dtype).to(DEV)
             gate = (torch.randn(50, 72, generator=g) / 8).to(dtype).to(DEV)
