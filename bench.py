@@ -68,7 +68,7 @@ def run_decode(eng_mod, model, batch, steps, warmup, vocab, seed):
     need = PROMPT_LEN + warmup + steps + extra
     pages = batch * (-(-need // BLOCK_SIZE) + 1)
     e = eng_mod.Engine(model, num_blocks=pages, block_size=BLOCK_SIZE, max_seqs=batch, max_len=CONTEXT_LIMIT,
-                       max_num_batched_tokens=budget)
+                       max_num_batched_tokens=budget, hip_graphs=True)
     for _ in range(batch):
         e.add_request(eng_mod.Request([int(t) for t in rng.integers(0, vocab, PROMPT_LEN)],
                                       max_new_tokens=warmup + steps + extra))

@@ -34,7 +34,8 @@ class Engine:
                                    max_prefill_chunk=max_prefill_chunk, hip_graphs=hip_graphs,
                                    device=str(model.rt.device))
         self.model = model
-        self.runner = ModelRunner(model, block_size, self.config.resolved_num_blocks(), max_seqs, max_len)
+        self.runner = ModelRunner(model, block_size, self.config.resolved_num_blocks(), max_seqs, max_len,
+                                  hip_graphs=hip_graphs)
         self.scheduler = Scheduler(self.runner.manager, self.config, clock, on_token, on_finish)
         self.sampler = Sampler(model.rt.device)
         self.clock = clock
@@ -87,7 +88,12 @@ class Engine:
                 if s.sample:
                     rows.append(s.request)
             logits = self.runner.step(entries)
-            useful = self.scheduler.commit(sched, self.sampler.sample(logits, rows))
+            greedy = self.runner.greedy_tokens
+            if greedy is not None and len(rows) == len(entries) and all(r.temperature <= 0.0 for r in rows):
+                sampled = greedy.tolist()       # the captured graph has already taken the argmax
+            else:
+                sampled = self.sampler.sample(logits, rows)
+            useful = self.scheduler.commit(sched, sampled)
         n_decode = sum(1 for s in sched if s.count == 1 and s.start > 0)
         n_prefill = sum(s.count for s in sched) - n_decode
         self.prefill_tokens_computed += n_prefill

@@ -1,0 +1,163 @@
+"""Decode-only steps replayed from captured HIP graphs, one graph per batch-size bucket.
+
+A decode step of a small model is bound by kernel launches, not by the GPU (the reference measured the
+same on its hardware and answered with CUDA graphs, src/miniserve/graph_decode.py:33-86).  The whole
+forward of a batch of single tokens is captured once per bucket {1, 2, 4, ..., max} (graph_decode.py:23-30)
+over static input buffers; a step then fills a pinned host copy of those buffers, sends it in one copy and
+replays.  Nothing in the captured kernels depends on how long the contexts are (block tables have their
+full width, the attention kernel spreads each request's keys over its waves itself), so a graph stays valid
+for the life of the engine.  Rows that pad a batch up to its bucket read the null page and store nothing.
+The greedy choice (argmax) of every row is part of the graph.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..kernels import ops
+from ..parts.base import StepContext
+from ..parts.model import RunCache
+from .batch import StepEntry
+
+
+def default_batch_sizes(max_batch: int) -> List[int]:
+    """1, 2, 4, 8, ... up to ``max_batch``, always including it (graph_decode.py:23-30)."""
+    sizes, b = [], 1
+    while b < max_batch:
+        sizes.append(b)
+        b *= 2
+    sizes.append(max_batch)
+    return sizes
+
+
+class _Bucket:
+    def __init__(self, B: int, width: int, n_groups: int, device):
+        self.B, self.width = B, width
+        # layout of the static int32 buffer
+        self.off: Dict[str, slice] = {}
+        o = 0
+        for name, n in (("token_ids", B), ("positions", B), ("token_req", B), ("q_start", B + 1),
+                        ("context_lens", B), ("state_slots", B), ("logit_rows", B)):
+            self.off[name] = slice(o, o + n)
+            o += n
+        self.tables, self.slots = [], []
+        for g in range(n_groups):
+            self.tables.append(slice(o, o + B * width)); o += B * width
+            self.slots.append(slice(o, o + B)); o += B
+        self.size = o
+        self.host = torch.zeros(o, dtype=torch.int32).pin_memory()
+        self.np = self.host.numpy()
+        self.dev = torch.zeros(o, dtype=torch.int32, device=device)
+        self.reset_host()
+        self.dev.copy_(self.host)
+        self.last_rows = 0
+        self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self.logits: Optional[torch.Tensor] = None
+        self.tokens: Optional[torch.Tensor] = None
+
+    def reset_host(self) -> None:
+        """Every row a padding row: token 0 at position 0, one visible key on the null page, nothing stored."""
+        a, B = self.np, self.B
+        a[:] = 0
+        a[self.off["token_req"]] = np.arange(B)
+        a[self.off["q_start"]] = np.arange(B + 1)
+        a[self.off["context_lens"]] = 1
+        a[self.off["logit_rows"]] = np.arange(B)
+        for s in self.slots:
+            a[s] = -1
+
+    def context(self) -> StepContext:
+        d, o = self.dev, self.off
+        return StepContext(
+            num_tokens=self.B, num_requests=self.B, token_ids=d[o["token_ids"]], positions=d[o["positions"]],
+            token_req=d[o["token_req"]], q_start=d[o["q_start"]], context_lens=d[o["context_lens"]],
+            state_slots=d[o["state_slots"]], logit_rows=d[o["logit_rows"]], max_q_len=1,
+            max_context_len=self.width, q_lens_host=[1] * self.B, start_pos_host=[0] * self.B,
+            state_slots_host=[0] * self.B)
+
+
+class DecodeGraphs:
+    def __init__(self, runner, batch_sizes: Optional[Sequence[int]] = None):
+        m = runner.manager
+        if runner.layout.state_runs:
+            raise ValueError("HIP graphs are not used for models whose mixers keep per-request state on the host side")
+        self.runner, self.manager = runner, m
+        self.sizes = sorted(set(batch_sizes or default_batch_sizes(m.max_requests)))
+        self.width = m.max_pages_per_request
+        self.buckets: Dict[int, _Bucket] = {}
+
+    @property
+    def max_batch(self) -> int:
+        return self.sizes[-1]
+
+    def _bucket(self, n: int) -> _Bucket:
+        B = next(b for b in self.sizes if b >= n)
+        bk = self.buckets.get(B)
+        if bk is None:
+            bk = self.buckets[B] = _Bucket(B, self.width, len(self.manager.groups), self.runner.rt.device)
+            self._capture(bk)
+        return bk
+
+    def _caches(self, bk: _Bucket) -> List[RunCache]:
+        r = self.runner
+        caches = []
+        for i in range(len(r.model.spec.order)):
+            g = r.layout.run_group[i]
+            kv = None
+            if g is not None:
+                kv = r.pools.kv_view(i, bk.dev[bk.tables[g]].view(bk.B, bk.width), bk.dev[bk.slots[g]])
+            caches.append(RunCache(kv, None))
+        return caches
+
+    def _capture(self, bk: _Bucket) -> None:
+        ctx, caches = bk.context(), self._caches(bk)
+        ctx.max_context_len = self.width * self.manager.page_size
+        model = self.runner.model
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):            # load kernels and settle allocations before capturing
+                model.forward(ctx, caches)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        bk.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(bk.graph):
+            bk.logits = model.forward(ctx, caches)
+            bk.tokens = torch.empty(bk.B, dtype=torch.int32, device=bk.logits.device)
+            ops.sample(bk.logits, bk.tokens)
+        torch.cuda.synchronize()
+
+    def run(self, entries: List[StepEntry]):
+        """One decode step for ``entries`` (one token each, pages already grown).  Returns (logits [R, V],
+        greedy tokens int32 [R]); both are views of static buffers that the next replay overwrites."""
+        m = self.manager
+        R = len(entries)
+        bk = self._bucket(R)
+        a, o, ps = bk.np, bk.off, m.page_size
+        rows = np.fromiter((m.row(e.req_id) for e in entries), dtype=np.int32, count=R)
+        pos = np.fromiter((m.computed(e.req_id) for e in entries), dtype=np.int32, count=R)
+        toks = np.fromiter((e.tokens[0] for e in entries), dtype=np.int64, count=R)
+        if toks.min() < 0 or toks.max() >= self.runner.model.spec.vocab_size:
+            raise ValueError("a token id is outside the vocabulary")
+        if int(pos.max()) + 1 > m.max_len:
+            raise ValueError(f"a request would hold {int(pos.max()) + 1} tokens; the cache is made for {m.max_len}")
+        if R < bk.last_rows:
+            bk.reset_host()
+        bk.last_rows = R
+        a[o["token_ids"]][:R] = toks
+        a[o["positions"]][:R] = pos
+        a[o["context_lens"]][:R] = pos + 1
+        a[o["state_slots"]][:R] = rows
+        used = int(pos.max()) // ps + 1
+        for g, grp in enumerate(m.groups):
+            t = a[bk.tables[g]].reshape(bk.B, bk.width)
+            t[:R, :used] = grp.tables[rows, :used]
+            page = t[np.arange(R), pos // ps]
+            if (page == 0).any():
+                raise RuntimeError("a token of this step has no page; grow the request before the step")
+            a[bk.slots[g]][:R] = page * ps + pos % ps
+        bk.dev.copy_(bk.host, non_blocking=True)
+        bk.graph.replay()
+        return bk.logits[:R], bk.tokens[:R]

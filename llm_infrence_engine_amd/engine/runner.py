@@ -18,7 +18,8 @@ from .batch import BatchBuilder, StepEntry
 
 
 class ModelRunner:
-    def __init__(self, model: Model, page_size: int, num_pages: int, max_requests: int, max_len: int):
+    def __init__(self, model: Model, page_size: int, num_pages: int, max_requests: int, max_len: int,
+                 hip_graphs: bool = False):
         if model.rt is None:
             raise RuntimeError("the model has no weights yet; load it first")
         self.model, self.rt = model, model.rt
@@ -26,6 +27,12 @@ class ModelRunner:
         self.manager = CacheManager(self.layout, page_size, num_pages, max_requests, max_len)
         self.pools = CachePools(self.layout, page_size, num_pages, max_requests, self.rt)
         self.builder = BatchBuilder(self.manager, model.spec.vocab_size, self.rt.device)
+        self.graphs = None
+        if hip_graphs and not self.layout.state_runs:
+            from .graph import DecodeGraphs
+
+            self.graphs = DecodeGraphs(self)
+        self.greedy_tokens: Optional[torch.Tensor] = None   # argmax of the last step's rows, if a graph computed it
 
     # ------------------------------------------------------------------ requests
     def add_request(self, req_id: Hashable) -> None:
@@ -48,6 +55,13 @@ class ModelRunner:
                 m.add(e.req_id)
         for e in entries:
             m.grow(e.req_id, m.computed(e.req_id) + len(e.tokens))
+        self.greedy_tokens = None
+        if (self.graphs is not None and len(entries) <= self.graphs.max_batch
+                and all(len(e.tokens) == 1 and len(e.want) == 1 for e in entries)):
+            logits, self.greedy_tokens = self.graphs.run(entries)
+            for e in entries:
+                m.advance(e.req_id, m.computed(e.req_id) + 1)
+            return logits
         ctx, tables, slots = self.builder.build(entries)
         if self.layout.state_runs:
             self.pools.zero_state([r for r, s in zip(ctx.state_slots_host, ctx.start_pos_host) if s == 0])
@@ -64,11 +78,12 @@ class ModelRunner:
 
 
 def load_runner(model_dir, dtype: str = "bfloat16", device: str = "cuda:0", page_size: int = 16,
-                num_pages: Optional[int] = None, max_requests: int = 32, max_len: int = 1024) -> ModelRunner:
+                num_pages: Optional[int] = None, max_requests: int = 32, max_len: int = 1024,
+                hip_graphs: bool = False) -> ModelRunner:
     """Model folder -> a runner with an empty cache."""
     from ..loading import load_model
 
     model = load_model(model_dir, dtype, device)
     if num_pages is None:
         num_pages = max_requests * (-(-max_len // page_size))
-    return ModelRunner(model, page_size, num_pages, max_requests, max_len)
+    return ModelRunner(model, page_size, num_pages, max_requests, max_len, hip_graphs)

@@ -171,3 +171,50 @@ def test_engine_refuses_the_cpu(tiny, eng):
     name, d, cfg, w = tiny
     with pytest.raises(RuntimeError, match="no CPU path"):
         eng.load_model(d, "float32", device="cpu")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_hip_graph_decode_equals_eager(tiny, eng, dtype):
+    """Decode steps replayed from captured graphs, with eager prompt portions, joins and finishes between the
+    replays: every replay's logits equal the eager step's, and so do the generated tokens."""
+    from llm_infrence_engine_amd.engine import StepEntry, load_runner
+
+    name, d, cfg, w = tiny
+    rng = np.random.default_rng(21)
+    seqs = {i: [int(t) for t in rng.integers(0, cfg["vocab_size"], n)] for i, n in enumerate((40, 29, 37))}
+    runs = {}
+    for graphs in (False, True):
+        r = load_runner(d, dtype=dtype, page_size=16, num_pages=12, max_requests=4, max_len=64, hip_graphs=graphs)
+        out = []
+        out.append(r.step([StepEntry(0, seqs[0][:20], [19])]).cpu())                       # eager: a prompt
+        for p in range(20, 26):
+            out.append(r.step([StepEntry(0, [seqs[0][p]], [0])]).cpu())                      # bucket of 1
+        out.append(r.step([StepEntry(1, seqs[1][:17], [16]), StepEntry(0, [seqs[0][26]], [0])]).cpu())   # eager: mixed
+        for p in range(6):
+            out.append(r.step([StepEntry(0, [seqs[0][27 + p]], [0]), StepEntry(1, [seqs[1][17 + p]], [0])]).cpu())
+        out.append(r.step([StepEntry(2, seqs[2][:30], [29])]).cpu())
+        for p in range(4):                                                                   # bucket of 4, one row padding
+            out.append(r.step([StepEntry(2, [seqs[2][30 + p]], [0]), StepEntry(0, [seqs[0][33 + p]], [0]),
+                               StepEntry(1, [seqs[1][23 + p]], [0])]).cpu())
+            if graphs:
+                assert r.greedy_tokens.tolist() == out[-1].argmax(-1).tolist()
+        r.free_request(1)
+        for p in range(3):                                                                   # back to a bucket of 2
+            out.append(r.step([StepEntry(2, [seqs[2][34 + p]], [0]), StepEntry(0, [seqs[0][37 + p]], [0])]).cpu())
+        runs[graphs] = out
+        if graphs:
+            assert sorted(r.graphs.buckets) == [1, 2, 4]
+    for a, b in zip(runs[False], runs[True]):
+        assert torch.equal(a, b)
+    exact = P.forward(w, cfg, seqs[2]).numpy()
+    assert np.abs(runs[True][-1][0].numpy() - exact[36]).max() < (1e-3 if dtype == "float32" else 0.5)
+
+
+def test_generation_with_hip_graphs(tiny, eng):
+    name, d, cfg, w = tiny
+    prompts = prompts_for(name, cfg["vocab_size"])
+    want = [P.greedy_generate(w, cfg, p, 10) for p in prompts]
+    llm = eng.LLM(d, dtype="float32", block_size=16, max_len=64, max_seqs=4, hip_graphs=True)
+    got = llm.generate(prompts, eng.SamplingParams(max_new_tokens=10))
+    assert [o.token_ids for o in got] == want
+    assert llm.engine.runner.graphs.buckets
