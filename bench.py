@@ -119,6 +119,7 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=MODEL["num_hidden_layers"],
                     help="fewer layers than the configuration has, if memory or time needs it (both numbers are reported)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points and the prefill")
+    ap.add_argument("--only", choices=["prefill"], help="run one part alone (for profiles): the 2,048-token prefill")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(f"bench.py measures one GPU; --gpus {a.gpus} is not supported by this single-GPU engine")
@@ -136,6 +137,11 @@ def main() -> int:
         eng.write_random_model(folder, cfg, seed=0, dtype="bfloat16")
         model = eng.load_model(folder, "bfloat16", "cuda:0")
     vocab = cfg.vocab_size
+    if a.only == "prefill":
+        pt = run_prefill(eng, model, vocab, seed=2, repeats=3)
+        print(json.dumps({"prefill": {"value": round(PREFILL_TOKENS / pt, 1), "tokens": PREFILL_TOKENS,
+                                      "ms": round(pt * 1e3, 3)}}), flush=True)
+        return 0
 
     dt, ctx = run_decode(eng, model, a.batch, a.steps, a.warmup, vocab, seed=1)
     value = a.batch / dt
