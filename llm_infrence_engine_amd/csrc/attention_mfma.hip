@@ -14,14 +14,18 @@
 //                                                   transposed, [page][kv head][dim][page_size]: a lane reads
 //                                                   8 contiguous bytes (4 keys) of one dim from each page.
 //
-// No LDS and no block-wide barrier: every wave is independent.  The next block's keys and values are
-// loaded while the current block is multiplied.  Keys beyond a column's own position are masked, values
-// beyond the last visible key are zeroed before use, and pages past the context are never dereferenced,
-// so what a reused page still holds cannot reach the result.
+// The WAVES waves of a block share a column tile and take its key blocks in turn (wave w: blocks w, w + WAVES,
+// ...), each with its own running maximum, sum and accumulators; at the end they are merged through LDS by
+// wave 0 in a fixed order.  That shortens the chain of dependent key blocks (a late prompt tile, a long
+// context) by WAVES and puts several waves on every SIMD to hide the latency of the page reads.  The next
+// block's keys and values are loaded while the current one is multiplied.  Keys beyond a column's own
+// position are masked, values beyond the last visible key are zeroed before use, and pages past the
+// context are never dereferenced, so what a reused page still holds cannot reach the result.
 //
 // Two launch shapes: general (any mix of portions and single tokens; grid = column tiles x kv heads x
-// requests, surplus tiles leave at once) and decode (every request has one token; the keys are split over
-// several waves which write unnormalised partial results, and a second kernel combines them).
+// requests, surplus tiles leave at once; a decode-only batch is the case of one tile per request) and
+// split (every request has one token and a long context: the keys are also split over several blocks which
+// write unnormalised partial results, and a second kernel combines them).
 #include "common.h"
 #include "api.h"
 
@@ -58,15 +62,18 @@ __device__ __forceinline__ void load_block(KVBlock<D>& b, const bf16* __restrict
   }
 }
 
-template <int D, int NT, bool SPLIT>
-__global__ void __launch_bounds__(MS_WAVE)
+template <int D, int NT, int WAVES, bool SPLIT>
+__global__ void __launch_bounds__(WAVES * MS_WAVE)
 attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* __restrict__ k_pages,
                       const bf16* __restrict__ vt_pages, const int* __restrict__ block_table, int table_stride,
                       const int* __restrict__ q_start, const int* __restrict__ context_lens,
                       bf16* __restrict__ out, size_t out_stride, float* __restrict__ part_o,
                       float* __restrict__ part_ml, int nh, int nkv, int page_size, float scale_log2e, int window,
                       int min_blocks, int n_splits) {
-  const int lane = threadIdx.x, col16 = lane & 15, kq = lane >> 4;
+  __shared__ float sm_m[WAVES][NT][16], sm_l[WAVES][NT][16];
+  __shared__ f32x4 sm_o[WAVES > 1 ? WAVES - 1 : 1][D / 16][NT][MS_WAVE];
+  const int lane = threadIdx.x & (MS_WAVE - 1), wave = threadIdx.x / MS_WAVE;
+  const int col16 = lane & 15, kq = lane >> 4;
   const int r = blockIdx.z, g = blockIdx.y;
   const int rep = nh / nkv;
   const int q0 = q_start[r];
@@ -119,10 +126,12 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
   }
 
   KVBlock<D> cur, nxt;
-  load_block<D>(cur, k_pages, vt_pages, table, blk_begin * 32, key_hi, g, nkv, page_size, lane);
-  for (int blk = blk_begin; blk < blk_end; ++blk) {
+  if (blk_begin + wave < blk_end)
+    load_block<D>(cur, k_pages, vt_pages, table, (blk_begin + wave) * 32, key_hi, g, nkv, page_size, lane);
+  for (int blk = blk_begin + wave; blk < blk_end; blk += WAVES) {
     const int base = blk * 32;
-    if (blk + 1 < blk_end) load_block<D>(nxt, k_pages, vt_pages, table, base + 32, key_hi, g, nkv, page_size, lane);
+    if (blk + WAVES < blk_end)
+      load_block<D>(nxt, k_pages, vt_pages, table, base + WAVES * 32, key_hi, g, nkv, page_size, lane);
 
     // scores: s[u][t] holds keys base + u*16 + kq*4 + (0..3) of column t*16 + col16
     f32x4 s[2][NT];
@@ -190,14 +199,49 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
 #pragma unroll
       for (int t = 0; t < NT; ++t) o[c][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, p[t], o[c][t], 0, 0, 0);
     }
-    if (blk + 1 < blk_end) cur = nxt;
+    if (blk + WAVES < blk_end) cur = nxt;
+  }
+
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {  // a column's sum is spread over the four lane groups
+    l[t] += __shfl_xor(l[t], 16, MS_WAVE);
+    l[t] += __shfl_xor(l[t], 32, MS_WAVE);
+  }
+  if (WAVES > 1) {
+    // merge the waves' partial results (each relative to its own maximum) in wave order
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      if (kq == 0) { sm_m[wave][t][col16] = m[t]; sm_l[wave][t][col16] = l[t]; }
+      if (wave > 0) {
+#pragma unroll
+        for (int c = 0; c < D / 16; ++c) sm_o[wave - 1][c][t][lane] = o[c][t];
+      }
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      float big = m[t];
+      for (int w = 1; w < WAVES; ++w) big = fmaxf(big, sm_m[w][t][col16]);
+      const float safe = big == -INFINITY ? 0.f : big;
+      const float f0 = fast_exp2(m[t] - safe);
+      float lsum = l[t] * f0;
+#pragma unroll
+      for (int c = 0; c < D / 16; ++c) o[c][t] *= f0;
+      for (int w = 1; w < WAVES; ++w) {
+        const float f = fast_exp2(sm_m[w][t][col16] - safe);
+        lsum += f * sm_l[w][t][col16];
+#pragma unroll
+        for (int c = 0; c < D / 16; ++c) o[c][t] += sm_o[w - 1][c][t][lane] * f;
+      }
+      m[t] = big;
+      l[t] = lsum;
+    }
   }
 
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
-    float lt = l[t];
-    lt += __shfl_xor(lt, 16, MS_WAVE);
-    lt += __shfl_xor(lt, 32, MS_WAVE);
+    const float lt = l[t];
     if (!valid[t]) continue;
     if (SPLIT) {
       // unnormalised: O, the running maximum (log2 units) and the sum; the combine kernel weighs the splits
@@ -246,24 +290,24 @@ __global__ void attention_combine_kernel(const float* __restrict__ part_o, const
   }
 }
 
-template <int D, int NT>
+template <int D, int NT, int WAVES>
 int launch_general(const bf16* q, size_t q_stride, const bf16* k, const bf16* vt, const int* table, int table_stride,
                    const int* q_start, const int* ctx, bf16* out, size_t out_stride, int n_requests, int max_q_len,
                    int nh, int nkv, int page_size, float scale, int window, hipStream_t stream) {
   const int rep = nh / nkv;
   const int tiles = (max_q_len * rep + 16 * NT - 1) / (16 * NT);
-  dim3 grid(tiles, nkv, n_requests), block(MS_WAVE);
-  attention_mfma_kernel<D, NT, false><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, q_start, ctx, out, out_stride, nullptr, nullptr, nh, nkv, page_size, scale * 1.4426950408889634f, window, 0, 0);
+  dim3 grid(tiles, nkv, n_requests), block(WAVES * MS_WAVE);
+  attention_mfma_kernel<D, NT, WAVES, false><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, q_start, ctx, out, out_stride, nullptr, nullptr, nh, nkv, page_size, scale * 1.4426950408889634f, window, 0, 0);
   return ms_launch_status();
 }
 
 template <int D>
-int launch_decode(const bf16* q, size_t q_stride, const bf16* k, const bf16* vt, const int* table, int table_stride,
-                  const int* q_start, const int* ctx, bf16* out, size_t out_stride, float* part_o, float* part_ml,
-                  int n_requests, int nh, int nkv, int page_size, float scale, int window, int min_blocks,
-                  int n_splits, hipStream_t stream) {
-  dim3 grid(n_splits, nkv, n_requests), block(MS_WAVE);
-  attention_mfma_kernel<D, 1, true><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, q_start, ctx, out, out_stride, part_o, part_ml, nh, nkv, page_size, scale * 1.4426950408889634f, window, min_blocks, n_splits);
+int launch_split(const bf16* q, size_t q_stride, const bf16* k, const bf16* vt, const int* table, int table_stride,
+                 const int* q_start, const int* ctx, bf16* out, size_t out_stride, float* part_o, float* part_ml,
+                 int n_requests, int nh, int nkv, int page_size, float scale, int window, int min_blocks,
+                 int n_splits, hipStream_t stream) {
+  dim3 grid(n_splits, nkv, n_requests), block(4 * MS_WAVE);
+  attention_mfma_kernel<D, 1, 4, true><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, q_start, ctx, out, out_stride, part_o, part_ml, nh, nkv, page_size, scale * 1.4426950408889634f, window, min_blocks, n_splits);
   attention_combine_kernel<D><<<dim3(n_requests * nh), dim3(D < 64 ? 64 : D), 0, stream>>>(part_o, part_ml, q_start, ctx, out, out_stride, nh, window, min_blocks, n_splits);
   return ms_launch_status();
 }
@@ -288,15 +332,17 @@ extern "C" int ms_paged_attention_mfma(const void* q, long long q_stride, const 
   if (!ms_attention_mfma_supported(head_dim, page_size)) return MS_UNSUPPORTED;
   if (q_stride % 8 || out_stride % 4 || ((uintptr_t)q % 16) || ((uintptr_t)out % 8)) return MS_UNSUPPORTED;
   if (n_requests > 65535 || num_kv_heads > 65535) return MS_UNSUPPORTED;
-#define GO(D, NT) return launch_general<D, NT>((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)vt_pages, block_table, table_stride, q_start, context_lens, (bf16*)out, out_stride, n_requests, max_q_len, num_heads, num_kv_heads, page_size, scale, window, stream)
+#define GO(D, NT, WV) return launch_general<D, NT, WV>((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)vt_pages, block_table, table_stride, q_start, context_lens, (bf16*)out, out_stride, n_requests, max_q_len, num_heads, num_kv_heads, page_size, scale, window, stream)
+  // few columns (a decode step): one narrow tile per request, more waves over its keys
   const int cols = max_q_len * (num_heads / num_kv_heads);
-  if (head_dim == 32) { if (cols > 32) GO(32, 4); else GO(32, 1); }
-  if (head_dim == 64) { if (cols > 32) GO(64, 4); else GO(64, 1); }
-  if (cols > 16) GO(128, 2); else GO(128, 1);
+  if (head_dim == 32) { if (cols > 16) GO(32, 4, 4); else GO(32, 1, 8); }
+  if (head_dim == 64) { if (cols > 16) GO(64, 4, 4); else GO(64, 1, 8); }
+  if (cols > 16) GO(128, 2, 4); else GO(128, 1, 8);
 #undef GO
 }
 
-// Decode shape: every request has exactly one token and the group (num_heads / num_kv_heads) is at most 16.
+// Split shape, for long contexts in small batches: every request has exactly one token and the group
+// (num_heads / num_kv_heads) is at most 16; the keys are spread over n_splits blocks and combined.
 // part_o: float [R, nh, n_splits, d], part_ml: float [R, nh, n_splits, 2].  Each request spreads its blocks of
 // 32 keys evenly over the n_splits waves, at least min_blocks to a wave, so the launch does not depend on
 // how long the contexts are.
@@ -314,7 +360,7 @@ extern "C" int ms_paged_attention_mfma_decode(const void* q, long long q_stride,
   if (min_blocks <= 0 || n_splits <= 0 || n_splits > 65535) return MS_BAD_ARG;
   if (q_stride % 8 || out_stride % 4 || ((uintptr_t)q % 16) || ((uintptr_t)out % 8) || ((uintptr_t)part_o % 16)) return MS_UNSUPPORTED;
   if (n_requests > 65535 || num_kv_heads > 65535) return MS_UNSUPPORTED;
-#define GO(D) return launch_decode<D>((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)vt_pages, block_table, table_stride, q_start, context_lens, (bf16*)out, out_stride, (float*)part_o, (float*)part_ml, n_requests, num_heads, num_kv_heads, page_size, scale, window, min_blocks, n_splits, stream)
+#define GO(D) return launch_split<D>((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)vt_pages, block_table, table_stride, q_start, context_lens, (bf16*)out, out_stride, (float*)part_o, (float*)part_ml, n_requests, num_heads, num_kv_heads, page_size, scale, window, min_blocks, n_splits, stream)
   if (head_dim == 32) GO(32);
   if (head_dim == 64) GO(64);
   GO(128);

@@ -6,7 +6,8 @@ forward of a batch of single tokens is captured once per bucket {1, 2, 4, ..., m
 over static input buffers; a step then fills a pinned host copy of those buffers, sends it in one copy and
 replays.  Nothing in the captured kernels depends on how long the contexts are (block tables have their
 full width, the attention kernel spreads each request's keys over its waves itself), so a graph stays valid
-for the life of the engine.  Rows that pad a batch up to its bucket read the null page and store nothing.
+for the life of the engine; only the choice between the attention's two launch shapes (contexts up to
+``ops.LONG_CONTEXT`` or beyond) is made per step, and each has graphs of its own.  Rows that pad a batch up to its bucket read the null page and store nothing.
 The greedy choice (argmax) of every row is part of the graph.
 """
 from __future__ import annotations
@@ -92,12 +93,13 @@ class DecodeGraphs:
     def max_batch(self) -> int:
         return self.sizes[-1]
 
-    def _bucket(self, n: int) -> _Bucket:
+    def _bucket(self, n: int, long_context: bool) -> _Bucket:
         B = next(b for b in self.sizes if b >= n)
-        bk = self.buckets.get(B)
+        key = (B, long_context)
+        bk = self.buckets.get(key)
         if bk is None:
-            bk = self.buckets[B] = _Bucket(B, self.width, len(self.manager.groups), self.runner.rt.device)
-            self._capture(bk)
+            bk = self.buckets[key] = _Bucket(B, self.width, len(self.manager.groups), self.runner.rt.device)
+            self._capture(bk, long_context)
         return bk
 
     def _caches(self, bk: _Bucket) -> List[RunCache]:
@@ -111,9 +113,10 @@ class DecodeGraphs:
             caches.append(RunCache(kv, None))
         return caches
 
-    def _capture(self, bk: _Bucket) -> None:
+    def _capture(self, bk: _Bucket, long_context: bool) -> None:
         ctx, caches = bk.context(), self._caches(bk)
-        ctx.max_context_len = self.width * self.manager.page_size
+        cap = self.width * self.manager.page_size
+        ctx.max_context_len = cap if long_context else min(cap, ops.LONG_CONTEXT)
         model = self.runner.model
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
@@ -134,10 +137,10 @@ class DecodeGraphs:
         greedy tokens int32 [R]); both are views of static buffers that the next replay overwrites."""
         m = self.manager
         R = len(entries)
-        bk = self._bucket(R)
-        a, o, ps = bk.np, bk.off, m.page_size
         rows = np.fromiter((m.row(e.req_id) for e in entries), dtype=np.int32, count=R)
         pos = np.fromiter((m.computed(e.req_id) for e in entries), dtype=np.int32, count=R)
+        bk = self._bucket(R, int(pos.max()) + 1 > ops.LONG_CONTEXT)
+        a, o, ps = bk.np, bk.off, m.page_size
         toks = np.fromiter((e.tokens[0] for e in entries), dtype=np.int64, count=R)
         if toks.min() < 0 or toks.max() >= self.runner.model.spec.vocab_size:
             raise ValueError("a token id is outside the vocabulary")

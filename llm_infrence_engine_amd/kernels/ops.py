@@ -300,17 +300,25 @@ def attention_mfma_supported(head_dim: int, page_size: int) -> bool:
     return bool(_get("ms_attention_mfma_supported")(head_dim, page_size))
 
 
-DECODE_WAVES = 1024      # waves a decode step's attention aims to put on the chip
+DECODE_WAVES = 1024       # waves a decode step's attention aims to put on the chip
 MAX_SPLITS = 32
-MIN_BLOCKS_PER_SPLIT = 2  # of 32 keys
+MIN_BLOCKS_PER_SPLIT = 8   # of 32 keys
+LONG_CONTEXT = 2048        # beyond this a small decode batch also splits its keys over blocks
+SPLIT_BELOW = 128          # ... when it has fewer (request, kv head) pairs than this
+
+
+def attention_splits_keys(n_requests: int, num_kv_heads: int, group: int, max_q_len: int, max_context_len: int) -> bool:
+    """Whether a step's attention takes the split shape (keys over several blocks plus a combine kernel)."""
+    return (max_q_len == 1 and group <= 16 and max_context_len > LONG_CONTEXT
+            and n_requests * num_kv_heads < SPLIT_BELOW)
 
 
 def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, vt_pages: torch.Tensor, block_table: torch.Tensor,
                          q_start: torch.Tensor, context_lens: torch.Tensor, out: torch.Tensor, num_heads: int,
                          scale: float, max_q_len: int, max_context_len: int, window: Optional[int] = None) -> torch.Tensor:
     """Matrix-core attention, bfloat16.  k_pages [P, nkv, page_size, d], vt_pages [P, nkv, d, page_size];
-    request r owns tokens q_start[r]..q_start[r+1]-1 and holds context_lens[r] keys after this step.  With
-    one token per request (``max_q_len`` 1) the keys are split over several waves and combined."""
+    request r owns tokens q_start[r]..q_start[r+1]-1 and holds context_lens[r] keys after this step.  A
+    small batch of single tokens with long contexts also splits the keys over blocks (and combines)."""
     _check(k_pages, "k_pages", torch.bfloat16)
     P, nkv, page_size, d = k_pages.shape
     _check(vt_pages, "vt_pages", torch.bfloat16, (P, nkv, d, page_size))
@@ -329,10 +337,10 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, vt_pages: torch
         raise ValueError(f"max_q_len {max_q_len} / max_context_len {max_context_len} do not fit a table of "
                          f"{block_table.shape[1]} pages of {page_size}")
     q_stride = q.stride(0) if N > 1 else q.shape[1]
-    if max_q_len == 1 and num_heads // nkv <= 16:
+    if attention_splits_keys(R, nkv, num_heads // nkv, max_q_len, max_context_len):
         # a launch constant of the batch size alone (so that a captured graph stays valid as contexts grow):
         # every request spreads its own key blocks over the splits inside the kernel
-        n_splits = max(1, min(MAX_SPLITS, DECODE_WAVES // max(1, R * nkv)))
+        n_splits = max(1, min(MAX_SPLITS, DECODE_WAVES // max(1, 4 * R * nkv)))
         part_o = torch.empty((R, num_heads, n_splits, d), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((R, num_heads, n_splits, 2), dtype=torch.float32, device=q.device)
         _call("ms_paged_attention_mfma_decode", q.data_ptr(), q_stride, k_pages.data_ptr(), vt_pages.data_ptr(),

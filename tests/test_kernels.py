@@ -374,15 +374,18 @@ def _paged_case(g, dtype, nh, nkv, d, page_size, ctx, qlen, fill):
 
 @pytest.mark.parametrize("nh,nkv,d,page_size,window", [(14, 2, 64, 16, None), (6, 2, 32, 16, None), (8, 8, 128, 32, None),
                                                         (4, 1, 64, 16, 40), (28, 4, 128, 16, None), (5, 5, 32, 64, 100)])
-@pytest.mark.parametrize("shape", ["mixed", "decode"])
+@pytest.mark.parametrize("shape", ["mixed", "decode", "long"])
 def test_paged_attention_mfma(ops, nh, nkv, d, page_size, window, shape):
     g = torch.Generator().manual_seed(nh * 100 + d)
     if shape == "mixed":
         ctx, qlen = [70, 133, 201, 300], [70, 9, 1, 150]
-    else:
+    elif shape == "decode":
         ctx, qlen = [1, 31, 32, 33, 600, 1500, 64, 17], [1] * 8
+    else:   # few requests with long contexts: keys split over blocks and combined
+        ctx, qlen = [2500, 1, 300], [1] * 3
     c = _paged_case(g, torch.bfloat16, nh, nkv, d, page_size, ctx, qlen, float("nan"))
     scale = 1.0 / math.sqrt(d)
+    assert ops.attention_splits_keys(len(ctx), nkv, nh // nkv, max(qlen), max(ctx)) == (shape == "long")
     want = torch.cat([attention_reference(q.double(), k.double(), v.double(), scale, window).transpose(0, 1).reshape(-1, nh * d)
                       for q, k, v in zip(c["qs"], c["ks"], c["vs"])])
     N = c["q"].shape[0]
