@@ -30,6 +30,10 @@ int ms_gemm_skinny_splits(int K, int splits);
 int ms_gemm_skinny(const void* A, long long lda, const void* W, long long ldw, const float* bias, void* out,
                    long long ldo, int M, int N, int K, int epilogue, int splits, int out_dtype, hipStream_t stream);
 
+int ms_gemm_skinny_norm(const float* x, long long ldx, const int* rows, const float* norm_w, float eps, const void* W,
+                        long long ldw, const float* bias, void* out, long long ldo, int M, int N, int K, int epilogue,
+                        int out_dtype, hipStream_t stream);
+
 int ms_paged_attention_generic(const void* q, long long q_stride, const void* k_pages, const void* v_pages,
                                const int* block_table, int table_stride, const int* token_req, const int* positions,
                                void* out, long long out_stride, int n_tokens, int num_heads, int num_kv_heads,

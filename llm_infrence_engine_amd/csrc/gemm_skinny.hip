@@ -10,6 +10,11 @@
 // 2j+1: up j) writing silu(gate) * up; float partial sums [splits, M, N] when K is split over blocks
 // (whoever consumes them adds them up in order, so results do not depend on timing); and the residual
 // sum, out[m, n] += product (+ bias) on a float matrix, each element owned by one lane: no atomics.
+//
+// With NORM the activations are the float residual stream and the RMS norm before the product is folded
+// in: the operand is bfloat16(x[m,k] * norm_weight[k]), the sum of squares of every row is gathered on the
+// way (every block sees all of K), and the accumulators are scaled by rsqrt(mean(x^2) + eps) before the
+// epilogue: norm(x) . W^T = rsqrt(..) * ((x * w) . W^T).
 #include "common.h"
 #include "api.h"
 
@@ -20,12 +25,16 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 enum { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_PARTIAL = 2, EPI_RESIDUAL = 3 };
 
-template <int MT, int EPI, typename TO, int WAVES>
+template <int MT, int EPI, typename TO, int WAVES, bool NORM>
 __global__ void __launch_bounds__(WAVES * MS_WAVE)
-gemm_skinny_kernel(const bf16* __restrict__ A, size_t lda, const bf16* __restrict__ W, size_t ldw,
+gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restrict__ W, size_t ldw,
                    const float* __restrict__ bias, TO* __restrict__ out, size_t ldo, int M, int N, int K,
-                   int steps_per_split) {
+                   int steps_per_split, const float* __restrict__ norm_w, float eps,
+                   const int* __restrict__ rows) {
   __shared__ f32x4 red[WAVES - 1][MT][MS_WAVE];
+  __shared__ float red_ss[NORM ? WAVES : 1][MT][16];
+  const bf16* A = (const bf16*)Av;
+  const float* X = (const float*)Av;
   const int lane = threadIdx.x & (MS_WAVE - 1), wave = threadIdx.x / MS_WAVE;
   const int col = lane & 15, kq = lane >> 4;
   const int n0 = blockIdx.x * 16;
@@ -35,13 +44,17 @@ gemm_skinny_kernel(const bf16* __restrict__ A, size_t lda, const bf16* __restric
 
   const int wn = min(n0 + col, N - 1);  // rows past the end repeat the last one; their results are not stored
   const bf16* wrow = W + (size_t)wn * ldw + kq * 8;
-  const bf16* arow[MT];
+  size_t arow[MT];  // element offset of this lane's activation row and k slice
 #pragma unroll
-  for (int t = 0; t < MT; ++t) arow[t] = A + (size_t)min(t * 16 + col, M - 1) * lda + kq * 8;
+  for (int t = 0; t < MT; ++t) {
+    const int m = min(t * 16 + col, M - 1);
+    arow[t] = (size_t)(rows ? rows[m] : m) * lda + kq * 8;  // rows: the activations are gathered rows of A
+  }
 
   f32x4 acc[MT];
+  float ss[MT];
 #pragma unroll
-  for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < MT; ++t) { acc[t] = f32x4{0.f, 0.f, 0.f, 0.f}; ss[t] = 0.f; }
 
 #pragma unroll 4
   for (int s = step_begin + wave; s < step_end; s += WAVES) {
@@ -49,11 +62,39 @@ gemm_skinny_kernel(const bf16* __restrict__ A, size_t lda, const bf16* __restric
     bf16x8 wv = {0, 0, 0, 0, 0, 0, 0, 0};
     const bool in = k + kq * 8 < K;  // K is a multiple of 8: a lane's 8 values are all inside or all outside
     if (in) wv = *reinterpret_cast<const bf16x8*>(wrow + k);
+    f32x4 nw0 = {0.f, 0.f, 0.f, 0.f}, nw1 = {0.f, 0.f, 0.f, 0.f};
+    if (NORM && in) {
+      nw0 = *reinterpret_cast<const f32x4*>(norm_w + k + kq * 8);
+      nw1 = *reinterpret_cast<const f32x4*>(norm_w + k + kq * 8 + 4);
+    }
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
       bf16x8 av = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (in) av = *reinterpret_cast<const bf16x8*>(arow[t] + k);
+      if (NORM) {
+        if (in) {
+          const f32x4 x0 = *reinterpret_cast<const f32x4*>(X + arow[t] + k);
+          const f32x4 x1 = *reinterpret_cast<const f32x4*>(X + arow[t] + k + 4);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            ss[t] = fmaf(x0[i], x0[i], ss[t]);
+            ss[t] = fmaf(x1[i], x1[i], ss[t]);
+            av[i] = (__bf16)(x0[i] * nw0[i]);
+            av[4 + i] = (__bf16)(x1[i] * nw1[i]);
+          }
+        }
+      } else {
+        if (in) av = *reinterpret_cast<const bf16x8*>(A + arow[t] + k);
+      }
       acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, av, acc[t], 0, 0, 0);
+    }
+  }
+
+  if (NORM) {  // a row's squares are spread over the four lane groups and over the waves
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      ss[t] += __shfl_xor(ss[t], 16, MS_WAVE);
+      ss[t] += __shfl_xor(ss[t], 32, MS_WAVE);
+      if (kq == 0) red_ss[wave][t][col] = ss[t];
     }
   }
 
@@ -67,6 +108,15 @@ gemm_skinny_kernel(const bf16* __restrict__ A, size_t lda, const bf16* __restric
   for (int t = 0; t < MT; ++t)
 #pragma unroll
     for (int w = 0; w < WAVES - 1; ++w) acc[t] += red[w][t][lane];
+  if (NORM) {
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      float total = 0.f;
+#pragma unroll
+      for (int w = 0; w < WAVES; ++w) total += red_ss[w][t][col];
+      acc[t] *= 1.0f / sqrtf(total / (float)K + eps);
+    }
+  }
 
   // lane holds out[m = t*16 + col][n = n0 + kq*4 + r], r = 0..3
   const int nb = n0 + kq * 4;
@@ -98,9 +148,10 @@ gemm_skinny_kernel(const bf16* __restrict__ A, size_t lda, const bf16* __restric
   }
 }
 
-template <int EPI, typename TO>
-int launch_mt(const bf16* A, size_t lda, const bf16* W, size_t ldw, const float* bias, TO* out, size_t ldo, int M,
-              int N, int K, int splits, hipStream_t stream) {
+template <int EPI, typename TO, bool NORM = false>
+int launch_mt(const void* A, size_t lda, const bf16* W, size_t ldw, const float* bias, TO* out, size_t ldo, int M,
+              int N, int K, int splits, hipStream_t stream, const float* norm_w = nullptr, float eps = 0.f,
+              const int* rows = nullptr) {
   const int total_steps = (K + 31) / 32;
   const int per = (total_steps + splits - 1) / splits;
   const int tiles = (N + 15) / 16;
@@ -108,7 +159,7 @@ int launch_mt(const bf16* A, size_t lda, const bf16* W, size_t ldw, const float*
   // enough waves to fill 256 CUs even when there are few features, but at least two k-steps per wave
   int waves = 4;
   while (waves < 16 && (long long)tiles * grid.y * waves < 1024 && per >= waves * 4) waves *= 2;
-#define GO2(MT, WV) gemm_skinny_kernel<MT, EPI, TO, WV><<<grid, dim3(WV * MS_WAVE), 0, stream>>>(A, lda, W, ldw, bias, out, ldo, M, N, K, per)
+#define GO2(MT, WV) gemm_skinny_kernel<MT, EPI, TO, WV, NORM><<<grid, dim3(WV * MS_WAVE), 0, stream>>>(A, lda, W, ldw, bias, out, ldo, M, N, K, per, norm_w, eps, rows)
 #define GO(MT) do { if (waves == 4) GO2(MT, 4); else if (waves == 8) GO2(MT, 8); else GO2(MT, 16); } while (0)
   if (M <= 16) GO(1);
   else if (M <= 32) GO(2);
@@ -159,6 +210,30 @@ extern "C" int ms_gemm_skinny(const void* A, long long lda, const void* W, long 
   if (epilogue == EPI_PARTIAL) {
     if (ldo < N || out_dtype != MS_F32 || splits < 1) return MS_BAD_ARG;
     return launch_mt<EPI_PARTIAL, float>(a, lda, w, ldw, bias, (float*)out, ldo, M, N, K, splits, stream);
+  }
+  return MS_BAD_ARG;
+}
+
+// As ms_gemm_skinny with epilogue 0 or 1, but the activations are rows of the float residual stream x[M,K]
+// and the RMS norm (weight norm_w[K], eps) that precedes the product is folded into the kernel.  With `rows`
+// (int32 [M]) row m of the product comes from x[rows[m]].
+extern "C" int ms_gemm_skinny_norm(const float* x, long long ldx, const int* rows, const float* norm_w, float eps, const void* W,
+                                   long long ldw, const float* bias, void* out, long long ldo, int M, int N, int K,
+                                   int epilogue, int out_dtype, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return MS_OK;
+  if (M > 64) return MS_UNSUPPORTED;
+  if (K <= 0 || K % 8 || ldx % 4 || ldw % 8 || ldx < K || ldw < K) return MS_UNSUPPORTED;
+  if (((uintptr_t)x | (uintptr_t)W | (uintptr_t)norm_w) % 16) return MS_UNSUPPORTED;
+  const bf16* w = (const bf16*)W;
+  if (epilogue == EPI_STORE) {
+    if (ldo < N) return MS_BAD_ARG;
+    if (out_dtype == MS_BF16) return launch_mt<EPI_STORE, bf16, true>(x, ldx, w, ldw, bias, (bf16*)out, ldo, M, N, K, 1, stream, norm_w, eps, rows);
+    if (out_dtype == MS_F32) return launch_mt<EPI_STORE, float, true>(x, ldx, w, ldw, bias, (float*)out, ldo, M, N, K, 1, stream, norm_w, eps, rows);
+    return MS_BAD_ARG;
+  }
+  if (epilogue == EPI_SWIGLU) {
+    if (N % 2 || ldo < N / 2 || out_dtype != MS_BF16 || bias) return MS_BAD_ARG;
+    return launch_mt<EPI_SWIGLU, bf16, true>(x, ldx, w, ldw, nullptr, (bf16*)out, ldo, M, N, K, 1, stream, norm_w, eps, rows);
   }
   return MS_BAD_ARG;
 }

@@ -19,6 +19,23 @@ from . import ops
 _mm_out_dtype_ok = None  # whether torch.mm can write float from bfloat16 inputs (found out at first use)
 
 
+class LazyNorm:
+    """Rows of the float residual stream that are still to be RMS-normalised.  The product that consumes them
+    folds the norm in when it can (few rows, bfloat16 weights); otherwise ``materialize`` runs the norm kernel."""
+
+    def __init__(self, x: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
+                 rows: Optional[torch.Tensor] = None):
+        self.x, self.weight, self.eps, self.out_dtype, self.rows = x, weight, eps, out_dtype, rows
+
+    @property
+    def num_rows(self) -> int:
+        return self.x.shape[0] if self.rows is None else self.rows.numel()
+
+    def materialize(self) -> torch.Tensor:
+        out = torch.empty((self.num_rows, self.x.shape[1]), dtype=self.out_dtype, device=self.x.device)
+        return ops.rms_norm(self.x, self.weight, self.eps, out, rows=self.rows)
+
+
 def prepare_weight(w: torch.Tensor) -> torch.Tensor:
     """The layout the kernels read: [out features, in features], rows contiguous."""
     return w.contiguous()
@@ -44,7 +61,11 @@ def _library_mm(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> Opt
 
 def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
            out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-    """[M, K] x [N, K] -> [M, N] in ``out_dtype`` (default: a's type)."""
+    """[M, K] x [N, K] -> [M, N] in ``out_dtype`` (default: a's type).  ``a`` may be a ``LazyNorm``."""
+    if isinstance(a, LazyNorm):
+        if ops.skinny_norm_ok(a.x, w, a.num_rows):
+            return ops.gemm_skinny_norm(a.x, a.weight, a.eps, w, bias, ops.EPI_STORE, out_dtype or a.out_dtype, a.rows)
+        a = a.materialize()
     out_dtype = out_dtype or a.dtype
     if a.dtype == torch.bfloat16:
         if ops.skinny_ok(a, w):
@@ -69,7 +90,12 @@ def linear_residual(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tenso
 
 
 def linear_swiglu(a: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
-    """silu(a @ gate.T) * (a @ up.T) for ``w_gate_up`` = interleave_rows(gate, up): [M, I]."""
+    """silu(a @ gate.T) * (a @ up.T) for ``w_gate_up`` = interleave_rows(gate, up): [M, I].  ``a`` may be a
+    ``LazyNorm``."""
+    if isinstance(a, LazyNorm):
+        if ops.skinny_norm_ok(a.x, w_gate_up, a.num_rows):
+            return ops.gemm_skinny_norm(a.x, a.weight, a.eps, w_gate_up, None, ops.EPI_SWIGLU, rows=a.rows)
+        a = a.materialize()
     if a.dtype == torch.bfloat16 and ops.skinny_ok(a, w_gate_up):
         return ops.gemm_skinny(a, w_gate_up, None, ops.EPI_SWIGLU)
     gu = linear(a, w_gate_up)

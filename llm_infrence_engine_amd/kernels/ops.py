@@ -22,6 +22,8 @@ _SIGNATURES = {
     "ms_embed": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "ms_rms_norm": [_c_ptr, _c_ptr, _c_int, _c_int, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int,
                     _c_int, _c_ptr],
+    "ms_gemm_skinny_norm": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_int,
+                            _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "ms_bias_add": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "ms_gemm_skinny_splits": [_c_int, _c_int],
     "ms_gemm_skinny": [_c_ptr, _c_ll, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int,
@@ -262,6 +264,46 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] =
         raise ValueError(f"unknown epilogue {epilogue}")
     _call("ms_gemm_skinny", a.data_ptr(), a.stride(0) if M > 1 else K, w.data_ptr(), K, _ptr(bias), out.data_ptr(), ldo,
           M, N, K, epilogue, splits, _code(out_dtype), _stream())
+    return out
+
+
+def skinny_norm_ok(x: torch.Tensor, w: torch.Tensor, n_rows: int) -> bool:
+    """Whether the few-rows kernel with the RMS norm folded in takes float rows of ``x`` against ``w``."""
+    return (x.dtype == torch.float32 and w.dtype == torch.bfloat16 and n_rows <= SKINNY_MAX_ROWS and x.dim() == 2
+            and x.shape[1] % 8 == 0 and x.is_contiguous() and w.is_contiguous() and x.data_ptr() % 16 == 0
+            and w.data_ptr() % 16 == 0)
+
+
+def gemm_skinny_norm(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w: torch.Tensor,
+                     bias: Optional[torch.Tensor] = None, epilogue: int = EPI_STORE,
+                     out_dtype: torch.dtype = torch.bfloat16, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """rms_norm(x[rows]) @ w.T with the norm folded into the product: x float32 [N, K] is the residual stream,
+    ``norm_weight`` float32 [K].  Epilogues EPI_STORE (+ bias) and EPI_SWIGLU as in ``gemm_skinny``."""
+    _check(x, "x", torch.float32)
+    _check(w, "w", torch.bfloat16)
+    N_rows, K = x.shape
+    M = N_rows
+    if rows is not None:
+        _check(rows, "rows", torch.int32)
+        M = rows.numel()
+    if w.shape[1] != K:
+        raise ValueError(f"shapes do not fit: x {list(x.shape)}, w {list(w.shape)}")
+    if not skinny_norm_ok(x, w, M):
+        raise ValueError(f"the few-rows kernel takes at most {SKINNY_MAX_ROWS} float rows with K a multiple of 8")
+    _check(norm_weight, "norm_weight", torch.float32, (K,))
+    N = w.shape[0]
+    if bias is not None:
+        _check(bias, "bias", torch.float32, (N,))
+    if epilogue == EPI_STORE:
+        out, ldo = torch.empty((M, N), dtype=out_dtype, device=x.device), N
+    elif epilogue == EPI_SWIGLU:
+        if N % 2 or bias is not None:
+            raise ValueError("the gated epilogue needs an even number of weight rows and no bias")
+        out, ldo, out_dtype = torch.empty((M, N // 2), dtype=torch.bfloat16, device=x.device), N // 2, torch.bfloat16
+    else:
+        raise ValueError(f"epilogue {epilogue} is not available with the folded norm")
+    _call("ms_gemm_skinny_norm", x.data_ptr(), K, _ptr(rows), norm_weight.data_ptr(), float(eps), w.data_ptr(), K,
+          _ptr(bias), out.data_ptr(), ldo, M, N, K, epilogue, _code(out_dtype), _stream())
     return out
 
 

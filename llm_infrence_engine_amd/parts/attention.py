@@ -17,6 +17,8 @@ from .base import KVNeed, Mixer, register_part
 
 
 class GQAttention(Mixer):
+    accepts_lazy_norm = True
+
     def __init__(self, prefix: str, position, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  scale: float, qkv_bias: bool = True, out_bias: bool = False, window: Optional[int] = None):
         if num_heads % num_kv_heads:

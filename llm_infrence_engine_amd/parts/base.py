@@ -116,6 +116,12 @@ class Part:
 
 
 class Norm(Part):
+    def lazy(self, x: torch.Tensor, delta: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None,
+             write_back: bool = True):
+        """What a block calls for a consumer that declares ``accepts_lazy_norm``: may return an object that
+        the consumer's first product normalises on the fly (``kernels.linear.LazyNorm``).  Default: ``forward``."""
+        return self.forward(x, delta, rows, write_back)
+
     def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor] = None,
                 rows: Optional[torch.Tensor] = None, write_back: bool = True) -> torch.Tensor:
         """Normalised activations of the float residual stream ``x`` [N, H].  With ``delta`` the sum
@@ -133,6 +139,8 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
+    accepts_lazy_norm = False   # True: h may be a LazyNorm that the part hands to kernels.linear
+
     def cache_need(self) -> Optional[KVNeed]:
         return None
 
@@ -151,6 +159,8 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    accepts_lazy_norm = False
+
     def forward(self, h: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         raise NotImplementedError
 
@@ -190,6 +200,8 @@ class Embedding(Part):
 
 
 class Head(Part):
+    accepts_lazy_norm = False
+
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         """Float logits [M, V] of normalised rows h [M, H]."""
         raise NotImplementedError

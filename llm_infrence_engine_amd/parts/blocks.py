@@ -11,10 +11,10 @@ from .base import Block, register_part
 
 class PreNormResidual(Block):
     def forward(self, x, pending, ctx, kv, state):
-        h = self.mixer_norm.forward(x, delta=pending)
-        a = self.mixer.forward_residual(h, ctx, kv, state, x)
-        h = self.feed_forward_norm.forward(x, delta=a)
-        return self.feed_forward.forward_residual(h, ctx, x)
+        norm = self.mixer_norm.lazy if self.mixer.accepts_lazy_norm else self.mixer_norm.forward
+        a = self.mixer.forward_residual(norm(x, delta=pending), ctx, kv, state, x)
+        norm = self.feed_forward_norm.lazy if self.feed_forward.accepts_lazy_norm else self.feed_forward_norm.forward
+        return self.feed_forward.forward_residual(norm(x, delta=a), ctx, x)
 
 
 register_part("block", "pre_norm_residual", PreNormResidual)

@@ -27,6 +27,8 @@ class TokenEmbedding(Embedding):
 
 
 class LMHead(Head):
+    accepts_lazy_norm = True
+
     def __init__(self, prefix: str, hidden_size: int, vocab_size: int, tied_to=None):
         self.prefix, self.hidden_size, self.vocab_size, self.tied_to = prefix, hidden_size, vocab_size, tied_to
 

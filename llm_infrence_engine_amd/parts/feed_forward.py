@@ -9,6 +9,8 @@ from .base import FeedForward, register_part
 
 
 class SwiGLU(FeedForward):
+    accepts_lazy_norm = True
+
     def __init__(self, prefix: str, hidden_size: int, intermediate_size: int):
         self.prefix, self.hidden_size, self.intermediate_size = prefix, hidden_size, intermediate_size
 

@@ -92,5 +92,5 @@ class Model:
             pending = self.layers[run.layer].forward(x, pending, ctx, c.kv, c.state)
         if ctx.logit_rows.numel() == 0:
             return torch.empty(0, self.spec.vocab_size, dtype=torch.float32, device=x.device)
-        h = self.final_norm.forward(x, delta=pending, rows=ctx.logit_rows, write_back=False)
-        return self.head.forward(h)
+        norm = self.final_norm.lazy if self.head.accepts_lazy_norm else self.final_norm.forward
+        return self.head.forward(norm(x, delta=pending, rows=ctx.logit_rows, write_back=False))

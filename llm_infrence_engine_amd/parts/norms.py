@@ -5,7 +5,9 @@ type (src/miniserve/model.py:69-73); here the weight is applied in float too and
 """
 from __future__ import annotations
 
-from ..kernels import ops
+import torch
+
+from ..kernels import linear, ops
 from ..weights.spec import TensorSpec
 from .base import Norm, register_part
 
@@ -25,6 +27,17 @@ class RMSNorm(Norm):
         n = x.shape[0] if rows is None else rows.numel()
         out = self.rt.empty(n, self.size)
         return ops.rms_norm(x, self.weight, self.eps, out, delta=delta, rows=rows, write_back=write_back)
+
+
+    def lazy(self, x, delta=None, rows=None, write_back=True):
+        """As ``forward``, for a consumer that can fold the norm into its first product: with few rows in
+        bfloat16 the addend is summed into x now and the normalisation is left to that product."""
+        n = x.shape[0] if rows is None else rows.numel()
+        if self.rt.dtype != torch.bfloat16 or n > ops.SKINNY_MAX_ROWS or self.size % 8 or (delta is not None and not write_back):
+            return self.forward(x, delta, rows, write_back)
+        if delta is not None:
+            ops.residual_add(x, delta)
+        return linear.LazyNorm(x, self.weight, self.eps, self.rt.dtype, rows)
 
 
 register_part("norm", "rms_norm", RMSNorm)

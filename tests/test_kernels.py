@@ -407,3 +407,32 @@ def test_paged_attention_mfma(ops, nh, nkv, d, page_size, window, shape):
 def test_attention_mfma_support_matrix(ops):
     assert ops.attention_mfma_supported(64, 16) and ops.attention_mfma_supported(128, 32)
     assert not ops.attention_mfma_supported(48, 16) and not ops.attention_mfma_supported(64, 8)
+
+
+@pytest.mark.parametrize("M", [1, 8, 33, 64])
+@pytest.mark.parametrize("N,K", [(1152, 896), (330, 72), (50, 200)])
+def test_gemm_skinny_with_the_norm_folded_in(ops, M, N, K):
+    g = torch.Generator().manual_seed(M + N)
+    x = (torch.randn(M + 5, K, generator=g) * 3).to(DEV)
+    nw = (1 + 0.1 * torch.randn(K, generator=g)).to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16().to(DEV)
+    bias = torch.randn(N, generator=g).to(DEV)
+    rows = torch.randperm(M + 5, generator=g)[:M].to(torch.int32).to(DEV)
+    xd = x.double()
+    h = nw.double() * (xd * torch.rsqrt((xd ** 2).mean(-1, keepdim=True) + 1e-5))
+    want = h @ w.double().T + bias.double()
+    t = dict(atol=3e-2, rtol=2e-2)   # the operand x * weight is rounded to bfloat16 before the product
+    got = ops.gemm_skinny_norm(x[:M].contiguous(), nw, 1e-5, w, bias)
+    torch.testing.assert_close(got.double(), want[:M], **t)
+    got = ops.gemm_skinny_norm(x, nw, 1e-5, w, bias, out_dtype=torch.float32, rows=rows)
+    assert got.dtype == torch.float32
+    torch.testing.assert_close(got.double(), want[rows.long()], **t)
+    if N % 2 == 0:
+        act = ops.gemm_skinny_norm(x, nw, 1e-5, w, None, ops.EPI_SWIGLU, rows=rows)
+        p = (h @ w.double().T)[rows.long()]
+        torch.testing.assert_close(act.double(), torch.nn.functional.silu(p[:, 0::2]) * p[:, 1::2], **t)
+    # against the unfused pair of kernels: the same up to the rounding of the operand
+    hb = torch.empty(M, K, dtype=torch.bfloat16, device=DEV)
+    ops.rms_norm(x, nw, 1e-5, hb, rows=rows)
+    unfused = ops.gemm_skinny(hb, w, bias, out_dtype=torch.float32)
+    torch.testing.assert_close(got, unfused, atol=3e-2, rtol=2e-2)
