@@ -1,0 +1,185 @@
+// One kernel for the front of an attention layer on few rows (a decode step's tokens):
+//   RMS norm (folded in as in gemm_skinny.hip) -> q, k, v projection with bias -> rotary encoding of q and k
+//   (half-split pairing, float angles) -> q to its buffer, k and v straight into their cache pages.
+// A block owns two 16-row tiles of the packed [q heads | k heads | v heads] weight that lie half a head
+// apart, so a lane ends up holding both members (j, j + d/2) of four rotary pairs of one token and can
+// rotate them in registers.  Requires the rotary dimension to be the whole head and d/2 a multiple of 16.
+#include "common.h"
+#include "api.h"
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+template <int MT, int WAVES>
+__global__ void __launch_bounds__(WAVES * MS_WAVE)
+qkv_rope_store_kernel(const float* __restrict__ X, size_t ldx, const float* __restrict__ norm_w, float eps,
+                      const bf16* __restrict__ W, const float* __restrict__ bias, const int* __restrict__ positions,
+                      const float* __restrict__ inv_freq, const int* __restrict__ slot_mapping,
+                      bf16* __restrict__ q_out, bf16* __restrict__ k_pages, bf16* __restrict__ v_pages, int M, int K,
+                      int nh, int nkv, int d, int page_size, int v_transposed) {
+  __shared__ f32x4 red[WAVES - 1][2][MT][MS_WAVE];
+  __shared__ float red_ss[WAVES][MT][16];
+  const int lane = threadIdx.x & (MS_WAVE - 1), wave = threadIdx.x / MS_WAVE;
+  const int col = lane & 15, kq = lane >> 4;
+  const int pairs_per_head = d / 32;
+  const int head = blockIdx.x / pairs_per_head;          // 0..nh-1: q, then nkv k heads, then nkv v heads
+  const int j0 = (blockIdx.x % pairs_per_head) * 16;      // first feature of the low tile within the head
+  const int half = d / 2;
+  const int total_steps = (K + 31) / 32;
+
+  const bf16* w_lo = W + ((size_t)head * d + j0 + col) * K + kq * 8;
+  const bf16* w_hi = w_lo + (size_t)half * K;
+  size_t xrow[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) xrow[t] = (size_t)min(t * 16 + col, M - 1) * ldx + kq * 8;
+
+  f32x4 lo[MT], hi[MT];
+  float ss[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) { lo[t] = hi[t] = f32x4{0.f, 0.f, 0.f, 0.f}; ss[t] = 0.f; }
+
+#pragma unroll 2
+  for (int s = wave; s < total_steps; s += WAVES) {
+    const int k = s * 32;
+    const bool in = k + kq * 8 < K;
+    bf16x8 wl = {0, 0, 0, 0, 0, 0, 0, 0}, wh = {0, 0, 0, 0, 0, 0, 0, 0};
+    f32x4 nw0 = {0.f, 0.f, 0.f, 0.f}, nw1 = {0.f, 0.f, 0.f, 0.f};
+    if (in) {
+      wl = *reinterpret_cast<const bf16x8*>(w_lo + k);
+      wh = *reinterpret_cast<const bf16x8*>(w_hi + k);
+      nw0 = *reinterpret_cast<const f32x4*>(norm_w + k + kq * 8);
+      nw1 = *reinterpret_cast<const f32x4*>(norm_w + k + kq * 8 + 4);
+    }
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      bf16x8 av = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (in) {
+        const f32x4 x0 = *reinterpret_cast<const f32x4*>(X + xrow[t] + k);
+        const f32x4 x1 = *reinterpret_cast<const f32x4*>(X + xrow[t] + k + 4);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          ss[t] = fmaf(x0[i], x0[i], ss[t]);
+          ss[t] = fmaf(x1[i], x1[i], ss[t]);
+          av[i] = (__bf16)(x0[i] * nw0[i]);
+          av[4 + i] = (__bf16)(x1[i] * nw1[i]);
+        }
+      }
+      lo[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wl, av, lo[t], 0, 0, 0);
+      hi[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wh, av, hi[t], 0, 0, 0);
+    }
+  }
+
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    ss[t] += __shfl_xor(ss[t], 16, MS_WAVE);
+    ss[t] += __shfl_xor(ss[t], 32, MS_WAVE);
+    if (kq == 0) red_ss[wave][t][col] = ss[t];
+    if (wave > 0) { red[wave - 1][0][t][lane] = lo[t]; red[wave - 1][1][t][lane] = hi[t]; }
+  }
+  __syncthreads();
+  if (wave > 0) return;
+
+  // lane holds features j0 + kq*4 + r (lo) and the same + d/2 (hi) of token t*16 + col
+  const int j = j0 + kq * 4;
+  const int row_lo = head * d + j;
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int m = t * 16 + col;
+    if (m >= M) continue;
+    float total = 0.f;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) total += red_ss[w][t][col];
+    const float inv = 1.0f / sqrtf(total / (float)K + eps);
+    float a[4], b[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float va = lo[t][r], vb = hi[t][r];
+#pragma unroll
+      for (int w = 0; w < WAVES - 1; ++w) { va += red[w][0][t][lane][r]; vb += red[w][1][t][lane][r]; }
+      a[r] = va * inv + (bias ? bias[row_lo + r] : 0.f);
+      b[r] = vb * inv + (bias ? bias[row_lo + half + r] : 0.f);
+    }
+    if (head < nh + nkv) {  // q and k heads turn by position * inv_freq[j]
+      const float pos = (float)positions[m];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float sn, cs;
+        sincosf(pos * inv_freq[j + r], &sn, &cs);
+        const float x1 = a[r], x2 = b[r];
+        a[r] = x1 * cs - x2 * sn;
+        b[r] = x2 * cs + x1 * sn;
+      }
+    }
+    bf16x4 pa, pb;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) { pa[r] = (__bf16)a[r]; pb[r] = (__bf16)b[r]; }
+    if (head < nh) {
+      bf16* qp = q_out + (size_t)m * nh * d + row_lo;
+      *reinterpret_cast<bf16x4*>(qp) = pa;
+      *reinterpret_cast<bf16x4*>(qp + half) = pb;
+      continue;
+    }
+    const long long slot = slot_mapping[m];
+    if (slot < 0) continue;
+    const long long page = slot / page_size;
+    const int off = (int)(slot % page_size);
+    if (head < nh + nkv) {
+      bf16* kp = k_pages + (((size_t)page * nkv + (head - nh)) * page_size + off) * d + j;
+      *reinterpret_cast<bf16x4*>(kp) = pa;
+      *reinterpret_cast<bf16x4*>(kp + half) = pb;
+    } else if (v_transposed) {
+      bf16* vp = v_pages + (((size_t)page * nkv + (head - nh - nkv)) * d + j) * page_size + off;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        vp[(size_t)r * page_size] = __float2bfloat16(a[r]);
+        vp[(size_t)(half + r) * page_size] = __float2bfloat16(b[r]);
+      }
+    } else {
+      bf16* vp = v_pages + (((size_t)page * nkv + (head - nh - nkv)) * page_size + off) * d + j;
+      *reinterpret_cast<bf16x4*>(vp) = pa;
+      *reinterpret_cast<bf16x4*>(vp + half) = pb;
+    }
+  }
+}
+
+template <int MT>
+int launch(const float* X, size_t ldx, const float* norm_w, float eps, const bf16* W, const float* bias,
+           const int* positions, const float* inv_freq, const int* slot_mapping, bf16* q_out, bf16* k_pages,
+           bf16* v_pages, int M, int K, int nh, int nkv, int d, int page_size, int v_transposed, hipStream_t stream) {
+  const int blocks = (nh + 2 * nkv) * (d / 32);
+  const int steps = (K + 31) / 32;
+  int waves = 4;
+  while (waves < 16 && blocks * waves < 1024 && steps >= waves * 2) waves *= 2;
+#define GO(WV) qkv_rope_store_kernel<MT, WV><<<dim3(blocks), dim3(WV * MS_WAVE), 0, stream>>>(X, ldx, norm_w, eps, W, bias, positions, inv_freq, slot_mapping, q_out, k_pages, v_pages, M, K, nh, nkv, d, page_size, v_transposed)
+  if (waves == 4) GO(4); else if (waves == 8) GO(8); else GO(16);
+#undef GO
+  return ms_launch_status();
+}
+
+}  // namespace
+
+// x float [M, K] (M <= 64), W bfloat16 [(nh + 2 nkv) d, K] packed q | k | v, bias float or null,
+// q_out bfloat16 [M, nh d], pages bfloat16 as in ms_rope_store, inv_freq float [d / 2].
+extern "C" int ms_qkv_rope_store(const float* x, long long ldx, const float* norm_w, float eps, const void* W,
+                                 const float* bias, const int* positions, const float* inv_freq,
+                                 const int* slot_mapping, void* q_out, void* k_pages, void* v_pages, int M, int K,
+                                 int num_heads, int num_kv_heads, int head_dim, int page_size, int v_transposed,
+                                 hipStream_t stream) {
+  if (M <= 0) return MS_OK;
+  if (M > 64 || head_dim % 32 || head_dim <= 0) return MS_UNSUPPORTED;
+  if (K <= 0 || K % 8 || ldx % 4 || ldx < K) return MS_UNSUPPORTED;
+  if (((uintptr_t)x | (uintptr_t)W | (uintptr_t)norm_w | (uintptr_t)q_out | (uintptr_t)k_pages | (uintptr_t)v_pages) % 16)
+    return MS_UNSUPPORTED;
+  if (num_heads <= 0 || num_kv_heads <= 0 || page_size <= 0 || !positions || !inv_freq || !slot_mapping || !q_out ||
+      !k_pages || !v_pages)
+    return MS_BAD_ARG;
+#define GO(MT) return launch<MT>(x, ldx, norm_w, eps, (const bf16*)W, bias, positions, inv_freq, slot_mapping, (bf16*)q_out, (bf16*)k_pages, (bf16*)v_pages, M, K, num_heads, num_kv_heads, head_dim, page_size, v_transposed, stream)
+  if (M <= 16) GO(1);
+  if (M <= 32) GO(2);
+  if (M <= 48) GO(3);
+  GO(4);
+#undef GO
+}

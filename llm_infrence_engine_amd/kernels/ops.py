@@ -24,6 +24,8 @@ _SIGNATURES = {
                     _c_int, _c_ptr],
     "ms_gemm_skinny_norm": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_int,
                             _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "ms_qkv_rope_store": [_c_ptr, _c_ll, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                          _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "ms_bias_add": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "ms_gemm_skinny_splits": [_c_int, _c_int],
     "ms_gemm_skinny": [_c_ptr, _c_ll, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int,
@@ -305,6 +307,37 @@ def gemm_skinny_norm(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w: 
     _call("ms_gemm_skinny_norm", x.data_ptr(), K, _ptr(rows), norm_weight.data_ptr(), float(eps), w.data_ptr(), K,
           _ptr(bias), out.data_ptr(), ldo, M, N, K, epilogue, _code(out_dtype), _stream())
     return out
+
+
+def qkv_rope_store_ok(x: torch.Tensor, w: torch.Tensor, head_dim: int, rot_dim: int) -> bool:
+    """Whether norm + projection + rotary + cache store run as one kernel for these rows."""
+    return skinny_norm_ok(x, w, x.shape[0]) and head_dim % 32 == 0 and rot_dim == head_dim
+
+
+def qkv_rope_store(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w_qkv: torch.Tensor,
+                   bias: Optional[torch.Tensor], num_heads: int, num_kv_heads: int, head_dim: int,
+                   positions: torch.Tensor, inv_freq: torch.Tensor, slot_mapping: torch.Tensor,
+                   k_pages: torch.Tensor, v_pages: torch.Tensor, v_transposed: bool) -> torch.Tensor:
+    """rms_norm(x) @ w_qkv.T + bias, q and k rotated (whole head, half-split pairs), k and v stored into the
+    pages at ``slot_mapping``; returns q bfloat16 [M, nh * d].  x float32 [M <= 64, K]."""
+    _check(x, "x", torch.float32)
+    M, K = x.shape
+    _check(w_qkv, "w_qkv", torch.bfloat16, ((num_heads + 2 * num_kv_heads) * head_dim, K))
+    if not qkv_rope_store_ok(x, w_qkv, head_dim, head_dim):
+        raise ValueError("the fused projection takes at most 64 float rows, K a multiple of 8 and head sizes in steps of 32")
+    _check(norm_weight, "norm_weight", torch.float32, (K,))
+    if bias is not None:
+        _check(bias, "bias", torch.float32, (w_qkv.shape[0],))
+    _check(positions, "positions", torch.int32, (M,))
+    _check(inv_freq, "inv_freq", torch.float32, (head_dim // 2,))
+    _check(slot_mapping, "slot_mapping", torch.int32, (M,))
+    _check(k_pages, "k_pages", torch.bfloat16, (None, num_kv_heads, None, head_dim))
+    _check(v_pages, "v_pages", torch.bfloat16, _v_shape(k_pages, v_transposed))
+    q = torch.empty((M, num_heads * head_dim), dtype=torch.bfloat16, device=x.device)
+    _call("ms_qkv_rope_store", x.data_ptr(), K, norm_weight.data_ptr(), float(eps), w_qkv.data_ptr(), _ptr(bias),
+          positions.data_ptr(), inv_freq.data_ptr(), slot_mapping.data_ptr(), q.data_ptr(), k_pages.data_ptr(),
+          v_pages.data_ptr(), M, K, num_heads, num_kv_heads, head_dim, k_pages.shape[2], int(v_transposed), _stream())
+    return q
 
 
 def paged_attention_generic(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,

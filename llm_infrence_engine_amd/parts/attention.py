@@ -71,13 +71,17 @@ class GQAttention(Mixer):
         if kv is None:
             raise RuntimeError("attention needs a key/value cache view")
         nh, nkv, d = self.num_heads, self.num_kv_heads, self.head_dim
-        qkv = linear.linear(h, self.w_qkv, bias=self.b_qkv)
+        q = None
         if self.position is not None:
-            self.position.encode_and_store(qkv, nh, nkv, d, ctx, kv)
-        elif kv.store:
-            ops.rope_store(qkv, nh, nkv, d, 0, None, None, kv.slot_mapping, kv.k_pages, kv.v_pages, kv.v_transposed)
+            q = self.position.project_encode_store(h, self.w_qkv, self.b_qkv, nh, nkv, d, ctx, kv)
+        if q is None:
+            q = linear.linear(h, self.w_qkv, bias=self.b_qkv)   # [N, (nh + 2 nkv) d]: attention reads its q part
+            if self.position is not None:
+                self.position.encode_and_store(q, nh, nkv, d, ctx, kv)
+            elif kv.store:
+                ops.rope_store(q, nh, nkv, d, 0, None, None, kv.slot_mapping, kv.k_pages, kv.v_pages, kv.v_transposed)
         out = self.rt.empty(ctx.num_tokens, nh * d)
-        ops.paged_attention(qkv, kv, ctx, out, nh, self.scale, self.window)
+        ops.paged_attention(q, kv, ctx, out, nh, self.scale, self.window)
         return linear.linear_residual(out, self.w_o, self.b_o, x)
 
 

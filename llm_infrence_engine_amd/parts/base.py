@@ -131,6 +131,12 @@ class Norm(Part):
 
 
 class PositionEncoding(Part):
+    def project_encode_store(self, h, w_qkv: torch.Tensor, bias: Optional[torch.Tensor], num_heads: int,
+                             num_kv_heads: int, head_dim: int, ctx: StepContext, kv: Optional[KVView]):
+        """Optional shortcut: projection, encoding and cache store in one kernel; returns q [N, nh d], or None
+        when it cannot (then the mixer projects and calls ``encode_and_store``)."""
+        return None
+
     def encode_and_store(self, qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
                          ctx: StepContext, kv: Optional[KVView]) -> None:
         """Encode positions into the q and k parts of ``qkv`` [N, (nh + 2 nkv) d] in place and, if ``kv``

@@ -9,7 +9,7 @@ from __future__ import annotations
 
 import torch
 
-from ..kernels import ops
+from ..kernels import linear, ops
 from .base import PositionEncoding, register_part
 
 
@@ -23,6 +23,13 @@ class RotaryHalf(PositionEncoding):
         self.rt = rt
         j = torch.arange(0, self.rotary_dim, 2, dtype=torch.float64)
         self.inv_freq = (1.0 / (self.theta ** (j / self.rotary_dim))).to(torch.float32).to(rt.device)
+
+    def project_encode_store(self, h, w_qkv, bias, num_heads, num_kv_heads, head_dim, ctx, kv):
+        if not (isinstance(h, linear.LazyNorm) and h.rows is None and kv is not None and kv.store
+                and ops.qkv_rope_store_ok(h.x, w_qkv, head_dim, self.rotary_dim)):
+            return None
+        return ops.qkv_rope_store(h.x, h.weight, h.eps, w_qkv, bias, num_heads, num_kv_heads, head_dim, ctx.positions,
+                                  self.inv_freq, kv.slot_mapping, kv.k_pages, kv.v_pages, kv.v_transposed)
 
     def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, ctx, kv):
         store = kv is not None and kv.store

@@ -436,3 +436,40 @@ def test_gemm_skinny_with_the_norm_folded_in(ops, M, N, K):
     ops.rms_norm(x, nw, 1e-5, hb, rows=rows)
     unfused = ops.gemm_skinny(hb, w, bias, out_dtype=torch.float32)
     torch.testing.assert_close(got, unfused, atol=3e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("M", [1, 8, 40])
+@pytest.mark.parametrize("nh,nkv,d,K,v_transposed", [(14, 2, 64, 896, True), (6, 3, 32, 72, False), (4, 1, 128, 200, True)])
+def test_qkv_rope_store_fused_equals_the_separate_kernels(ops, M, nh, nkv, d, K, v_transposed):
+    g = torch.Generator().manual_seed(M + d)
+    page_size, pages = 16, 12
+    x = (torch.randn(M, K, generator=g) * 2).to(DEV)
+    nw = (1 + 0.1 * torch.randn(K, generator=g)).to(DEV)
+    w = (torch.randn((nh + 2 * nkv) * d, K, generator=g) / math.sqrt(K)).bfloat16().to(DEV)
+    bias = torch.randn((nh + 2 * nkv) * d, generator=g).to(DEV)
+    pos = torch.randint(0, 3000, (M,), generator=g).to(torch.int32).to(DEV)
+    slots = torch.randperm(pages * page_size, generator=g)[:M].to(torch.int32)
+    if M > 2:
+        slots[2] = -1
+    slots = slots.to(DEV)
+    inv_freq = (1.0 / (1e6 ** (torch.arange(0, d, 2, dtype=torch.float64) / d))).float().to(DEV)
+    vshape = (pages, nkv, d, page_size) if v_transposed else (pages, nkv, page_size, d)
+    kp1, vp1 = torch.zeros(pages, nkv, page_size, d, dtype=torch.bfloat16, device=DEV), torch.zeros(vshape, dtype=torch.bfloat16, device=DEV)
+    kp2, vp2 = torch.zeros_like(kp1), torch.zeros_like(vp1)
+    q = ops.qkv_rope_store(x, nw, 1e-6, w, bias, nh, nkv, d, pos, inv_freq, slots, kp1, vp1, v_transposed)
+    # the separate kernels, in float between them so that only the final rounding differs
+    qkv = ops.gemm_skinny_norm(x, nw, 1e-6, w, bias, out_dtype=torch.float32)
+    exact = qkv.double().view(M, nh + 2 * nkv, d).cpu()
+    rot = rope_reference(exact[:, :nh + nkv], pos.cpu(), d, inv_freq.double().cpu())
+    torch.testing.assert_close(q.double().cpu().view(M, nh, d), rot[:, :nh], atol=3e-2, rtol=1.6e-2)
+    for n in range(M):
+        s = int(slots[n])
+        if s < 0:
+            continue
+        p, o = divmod(s, page_size)
+        torch.testing.assert_close(kp1[p, :, o].double().cpu(), rot[n, nh:], atol=3e-2, rtol=1.6e-2)
+        v = vp1[p, :, :, o] if v_transposed else vp1[p, :, o]
+        torch.testing.assert_close(v.double().cpu(), exact[n, nh + nkv:], atol=3e-2, rtol=1.6e-2)
+    untouched = torch.ones(pages * page_size, dtype=torch.bool)
+    untouched[slots[slots >= 0].long().cpu()] = False
+    assert (kp1.permute(0, 2, 1, 3).reshape(pages * page_size, -1)[untouched.to(DEV)] == 0).all()
