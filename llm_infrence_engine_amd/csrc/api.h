@@ -25,10 +25,8 @@ int ms_rope_store(void* qkv, const int* positions, const float* inv_freq, const 
 int ms_gemm_generic(const void* A, const void* W, const float* bias, void* C, int M, int N, int K, long long lda,
                     long long ldw, long long ldc, int in_dtype, int out_dtype, int accumulate, hipStream_t stream);
 
-int ms_gemm_skinny_splits(int K, int splits);
-
 int ms_gemm_skinny(const void* A, long long lda, const void* W, long long ldw, const float* bias, void* out,
-                   long long ldo, int M, int N, int K, int epilogue, int splits, int out_dtype, hipStream_t stream);
+                   long long ldo, int M, int N, int K, int epilogue, int out_dtype, hipStream_t stream);
 
 int ms_gemm_skinny_norm(const float* x, long long ldx, const int* rows, const float* norm_w, float eps, const void* W,
                         long long ldw, const float* bias, void* out, long long ldo, int M, int N, int K, int epilogue,

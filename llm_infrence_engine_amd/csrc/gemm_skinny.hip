@@ -1,15 +1,16 @@
 // out[M,N] = A[M,K] . W[N,K]^T for few rows (M <= 64, a decode step's tokens), bfloat16 in, float accumulation
 // on the matrix cores (v_mfma_f32_16x16x32_bf16).  The product is bound by reading W once from HBM, so
-// the kernel is shaped for memory parallelism: a block owns 16 output features and a slice of K; its
-// waves (4, 8 or 16 of them, more when there are few features so that the chip still fills) take
-// interleaved 32-wide k-steps, each lane streaming 16 bytes of one weight row per step, and add their
-// accumulators through LDS in a fixed order.  The weight tile is the MFMA's A operand and the
-// activation tile its B operand, so a lane ends up with 4 consecutive output features of one token.
+// the kernel is shaped for memory parallelism: a block owns NTILE tiles of 16 output features; its WAVES
+// waves take interleaved 32-wide k-steps, each lane streaming 16 bytes of one weight row per tile and step,
+// and the waves' accumulators are added through LDS in a fixed order (so a result does not depend on what
+// else is in the batch).  The weight tile is the MFMA's A operand and the activation tile its B operand:
+// a lane ends up with 4 consecutive output features of one token.  One activation load serves the NTILE
+// weight tiles of the block, which matters as M grows and the activations are read once per block.
+// (tile, 16-token group) pairs are spread over the waves for the final sum and the epilogue.
 //
 // Epilogues: plain (+ bias) to bfloat16 or float; gated activation over interleaved rows (2j: gate j,
-// 2j+1: up j) writing silu(gate) * up; float partial sums [splits, M, N] when K is split over blocks
-// (whoever consumes them adds them up in order, so results do not depend on timing); and the residual
-// sum, out[m, n] += product (+ bias) on a float matrix, each element owned by one lane: no atomics.
+// 2j+1: up j) writing silu(gate) * up; the residual sum out[m, n] += product (+ bias) on a float matrix, each
+// element owned by one lane: no atomics.
 //
 // With NORM the activations are the float residual stream and the RMS norm before the product is folded
 // in: the operand is bfloat16(x[m,k] * norm_weight[k]), the sum of squares of every row is gathered on the
@@ -23,27 +24,27 @@ namespace {
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
-enum { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_PARTIAL = 2, EPI_RESIDUAL = 3 };
+enum { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_RESIDUAL = 3 };
 
-template <int MT, int EPI, typename TO, int WAVES, bool NORM>
+template <int MT, int NTILE, int WAVES, int EPI, typename TO, bool NORM>
 __global__ void __launch_bounds__(WAVES * MS_WAVE)
 gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restrict__ W, size_t ldw,
                    const float* __restrict__ bias, TO* __restrict__ out, size_t ldo, int M, int N, int K,
-                   int steps_per_split, const float* __restrict__ norm_w, float eps,
-                   const int* __restrict__ rows) {
-  __shared__ f32x4 red[WAVES - 1][MT][MS_WAVE];
+                   const float* __restrict__ norm_w, float eps, const int* __restrict__ rows) {
+  constexpr int ITEMS = NTILE * MT;
+  __shared__ f32x4 red[WAVES - 1][ITEMS][MS_WAVE];
   __shared__ float red_ss[NORM ? WAVES : 1][MT][16];
   const bf16* A = (const bf16*)Av;
   const float* X = (const float*)Av;
   const int lane = threadIdx.x & (MS_WAVE - 1), wave = threadIdx.x / MS_WAVE;
   const int col = lane & 15, kq = lane >> 4;
-  const int n0 = blockIdx.x * 16;
+  const int n0 = blockIdx.x * 16 * NTILE;
   const int total_steps = (K + 31) / 32;
-  const int step_begin = blockIdx.y * steps_per_split;
-  const int step_end = min(total_steps, step_begin + steps_per_split);
 
-  const int wn = min(n0 + col, N - 1);  // rows past the end repeat the last one; their results are not stored
-  const bf16* wrow = W + (size_t)wn * ldw + kq * 8;
+  const bf16* wrow[NTILE];
+#pragma unroll
+  for (int u = 0; u < NTILE; ++u)  // rows past the end repeat the last one; their results are not stored
+    wrow[u] = W + (size_t)min(n0 + u * 16 + col, N - 1) * ldw + kq * 8;
   size_t arow[MT];  // element offset of this lane's activation row and k slice
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
@@ -51,17 +52,25 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
     arow[t] = (size_t)(rows ? rows[m] : m) * lda + kq * 8;  // rows: the activations are gathered rows of A
   }
 
-  f32x4 acc[MT];
+  f32x4 acc[NTILE][MT];
   float ss[MT];
 #pragma unroll
-  for (int t = 0; t < MT; ++t) { acc[t] = f32x4{0.f, 0.f, 0.f, 0.f}; ss[t] = 0.f; }
+  for (int t = 0; t < MT; ++t) {
+    ss[t] = 0.f;
+#pragma unroll
+    for (int u = 0; u < NTILE; ++u) acc[u][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
 
-#pragma unroll 4
-  for (int s = step_begin + wave; s < step_end; s += WAVES) {
+#pragma unroll 2
+  for (int s = wave; s < total_steps; s += WAVES) {
     const int k = s * 32;
-    bf16x8 wv = {0, 0, 0, 0, 0, 0, 0, 0};
     const bool in = k + kq * 8 < K;  // K is a multiple of 8: a lane's 8 values are all inside or all outside
-    if (in) wv = *reinterpret_cast<const bf16x8*>(wrow + k);
+    bf16x8 wv[NTILE];
+#pragma unroll
+    for (int u = 0; u < NTILE; ++u) {
+      wv[u] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+      if (in) wv[u] = *reinterpret_cast<const bf16x8*>(wrow[u] + k);
+    }
     f32x4 nw0 = {0.f, 0.f, 0.f, 0.f}, nw1 = {0.f, 0.f, 0.f, 0.f};
     if (NORM && in) {
       nw0 = *reinterpret_cast<const f32x4*>(norm_w + k + kq * 8);
@@ -85,7 +94,8 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
       } else {
         if (in) av = *reinterpret_cast<const bf16x8*>(A + arow[t] + k);
       }
-      acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv, av, acc[t], 0, 0, 0);
+#pragma unroll
+      for (int u = 0; u < NTILE; ++u) acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[u], av, acc[u][t], 0, 0, 0);
     }
   }
 
@@ -97,119 +107,111 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
       if (kq == 0) red_ss[wave][t][col] = ss[t];
     }
   }
-
-  if (wave > 0) {
+  // item (u, t) is finished by wave (u * MT + t) % WAVES; every other wave leaves its share in LDS
 #pragma unroll
-    for (int t = 0; t < MT; ++t) red[wave - 1][t][lane] = acc[t];
-  }
-  __syncthreads();
-  if (wave > 0) return;
-#pragma unroll
-  for (int t = 0; t < MT; ++t)
-#pragma unroll
-    for (int w = 0; w < WAVES - 1; ++w) acc[t] += red[w][t][lane];
-  if (NORM) {
+  for (int u = 0; u < NTILE; ++u)
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
-      float total = 0.f;
-#pragma unroll
-      for (int w = 0; w < WAVES; ++w) total += red_ss[w][t][col];
-      acc[t] *= 1.0f / sqrtf(total / (float)K + eps);
+      const int item = u * MT + t, owner = item % WAVES;
+      if (wave != owner) red[wave < owner ? wave : wave - 1][item][lane] = acc[u][t];
     }
-  }
+  __syncthreads();
 
-  // lane holds out[m = t*16 + col][n = n0 + kq*4 + r], r = 0..3
-  const int nb = n0 + kq * 4;
 #pragma unroll
-  for (int t = 0; t < MT; ++t) {
-    const int m = t * 16 + col;
-    if (m >= M) continue;
-    if (EPI == EPI_SWIGLU) {
-      // rows nb, nb+1 are (gate, up) of feature nb/2; rows nb+2, nb+3 of feature nb/2 + 1
+  for (int u = 0; u < NTILE; ++u)
 #pragma unroll
-      for (int p = 0; p < 2; ++p) {
-        if (nb + 2 * p + 1 < N) {
-          const float g = acc[t][2 * p], u = acc[t][2 * p + 1];
-          out[(size_t)m * ldo + nb / 2 + p] = from_float<TO>(g / (1.0f + expf(-g)) * u);
-        }
+    for (int t = 0; t < MT; ++t) {
+      const int item = u * MT + t, owner = item % WAVES;
+      if (wave != owner) continue;
+      // sum in wave order: the waves below the owner, the owner itself, the waves above
+      f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+      for (int w = 0; w < WAVES; ++w) sum += w == owner ? acc[u][t] : red[w < owner ? w : w - 1][item][lane];
+      if (NORM) {
+        float total = 0.f;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) total += red_ss[w][t][col];
+        sum *= 1.0f / sqrtf(total / (float)K + eps);
       }
-    } else {
-      TO* o = out + (EPI == EPI_PARTIAL ? (size_t)blockIdx.y * M * ldo : 0) + (size_t)m * ldo + nb;
-      const bool add_bias = bias != nullptr && (EPI != EPI_PARTIAL || blockIdx.y == 0);
+      // lane holds out[m = t*16 + col][n = nb + r], r = 0..3
+      const int m = t * 16 + col;
+      const int nb = n0 + u * 16 + kq * 4;
+      if (m >= M) continue;
+      if (EPI == EPI_SWIGLU) {
+        // rows nb, nb+1 are (gate, up) of feature nb/2; rows nb+2, nb+3 of feature nb/2 + 1
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        if (nb + r < N) {
-          float v = acc[t][r] + (add_bias ? bias[nb + r] : 0.f);
-          if (EPI == EPI_RESIDUAL) v += to_float(o[r]);
-          o[r] = from_float<TO>(v);
+        for (int p = 0; p < 2; ++p) {
+          if (nb + 2 * p + 1 < N) {
+            const float g = sum[2 * p], up = sum[2 * p + 1];
+            out[(size_t)m * ldo + nb / 2 + p] = from_float<TO>(g / (1.0f + expf(-g)) * up);
+          }
+        }
+      } else {
+        TO* o = out + (size_t)m * ldo + nb;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          if (nb + r < N) {
+            float v = sum[r] + (bias ? bias[nb + r] : 0.f);
+            if (EPI == EPI_RESIDUAL) v += to_float(o[r]);
+            o[r] = from_float<TO>(v);
+          }
         }
       }
     }
-  }
 }
 
-template <int EPI, typename TO, bool NORM = false>
-int launch_mt(const void* A, size_t lda, const bf16* W, size_t ldw, const float* bias, TO* out, size_t ldo, int M,
-              int N, int K, int splits, hipStream_t stream, const float* norm_w = nullptr, float eps = 0.f,
-              const int* rows = nullptr) {
-  const int total_steps = (K + 31) / 32;
-  const int per = (total_steps + splits - 1) / splits;
+// The shapes of block on offer: (tiles per block, waves).  LDS holds (waves - 1) * tiles * MT KB.
+template <int MT, int EPI, typename TO, bool NORM>
+int launch_cfg(const void* A, size_t lda, const bf16* W, size_t ldw, const float* bias, TO* out, size_t ldo, int M,
+               int N, int K, hipStream_t stream, const float* norm_w, float eps, const int* rows) {
   const int tiles = (N + 15) / 16;
-  dim3 grid(tiles, (total_steps + per - 1) / per);
-  // enough waves to fill 256 CUs even when there are few features, but at least two k-steps per wave
-  int waves = 4;
-  while (waves < 16 && (long long)tiles * grid.y * waves < 1024 && per >= waves * 4) waves *= 2;
-#define GO2(MT, WV) gemm_skinny_kernel<MT, EPI, TO, WV, NORM><<<grid, dim3(WV * MS_WAVE), 0, stream>>>(A, lda, W, ldw, bias, out, ldo, M, N, K, per, norm_w, eps, rows)
-#define GO(MT) do { if (waves == 4) GO2(MT, 4); else if (waves == 8) GO2(MT, 8); else GO2(MT, 16); } while (0)
-  if (M <= 16) GO(1);
-  else if (M <= 32) GO(2);
-  else if (M <= 48) GO(3);
-  else GO(4);
+  const int steps = (K + 31) / 32;
+  // as many tiles per block as still leaves a block for every CU; narrow outputs keep one tile per block
+  // (two when there are several token groups, whose activations would otherwise be read once per tile)
+  int ntile = tiles >= 1024 ? 4 : (tiles >= 512 ? 2 : 1);
+  if (ntile == 1 && MT >= 2 && tiles >= 32) ntile = 2;
+#define GO(NT, WV) gemm_skinny_kernel<MT, NT, WV, EPI, TO, NORM><<<dim3((tiles + NT - 1) / NT), dim3(WV * MS_WAVE), 0, stream>>>(A, lda, W, ldw, bias, out, ldo, M, N, K, norm_w, eps, rows)
+  if (ntile == 4) GO(4, 4);
+  else if (ntile == 2) GO(2, 8);
+  else if (steps >= 32 || MT > 1) GO(1, 16);
+  else GO(1, 8);
 #undef GO
-#undef GO2
   return ms_launch_status();
+}
+
+template <int EPI, typename TO, bool NORM>
+int launch_mt(const void* A, size_t lda, const bf16* W, size_t ldw, const float* bias, TO* out, size_t ldo, int M,
+              int N, int K, hipStream_t stream, const float* norm_w = nullptr, float eps = 0.f,
+              const int* rows = nullptr) {
+  if (M <= 16) return launch_cfg<1, EPI, TO, NORM>(A, lda, W, ldw, bias, out, ldo, M, N, K, stream, norm_w, eps, rows);
+  if (M <= 32) return launch_cfg<2, EPI, TO, NORM>(A, lda, W, ldw, bias, out, ldo, M, N, K, stream, norm_w, eps, rows);
+  return launch_cfg<4, EPI, TO, NORM>(A, lda, W, ldw, bias, out, ldo, M, N, K, stream, norm_w, eps, rows);
 }
 
 }  // namespace
 
-// The number of partial sums that ms_gemm_skinny writes for `splits` asked for (a split never is empty).
-extern "C" int ms_gemm_skinny_splits(int K, int splits) {
-  const int total_steps = (K + 31) / 32;
-  if (splits < 1) splits = 1;
-  const int per = (total_steps + splits - 1) / splits;
-  return (total_steps + per - 1) / per;
-}
-
 // epilogue 0: out[M,N] (out_dtype float or bfloat16) = product + bias
 // epilogue 1: out[M,N/2] bfloat16 = silu(gate) * up over interleaved rows of W (no bias)
-// epilogue 2: out[splits,M,N] float partial sums (bias goes into split 0); `splits` as ms_gemm_skinny_splits gives
 // epilogue 3: out[M,N] float += product + bias
 extern "C" int ms_gemm_skinny(const void* A, long long lda, const void* W, long long ldw, const float* bias, void* out,
-                              long long ldo, int M, int N, int K, int epilogue, int splits, int out_dtype,
-                              hipStream_t stream) {
+                              long long ldo, int M, int N, int K, int epilogue, int out_dtype, hipStream_t stream) {
   if (M <= 0 || N <= 0) return MS_OK;
   if (M > 64) return MS_UNSUPPORTED;
   if (K <= 0 || K % 8 || lda % 8 || ldw % 8 || lda < K || ldw < K) return MS_UNSUPPORTED;
   if (((uintptr_t)A | (uintptr_t)W) % 16) return MS_UNSUPPORTED;
-  const bf16* a = (const bf16*)A;
   const bf16* w = (const bf16*)W;
   if (epilogue == EPI_STORE) {
     if (ldo < N) return MS_BAD_ARG;
-    if (out_dtype == MS_BF16) return launch_mt<EPI_STORE, bf16>(a, lda, w, ldw, bias, (bf16*)out, ldo, M, N, K, 1, stream);
-    if (out_dtype == MS_F32) return launch_mt<EPI_STORE, float>(a, lda, w, ldw, bias, (float*)out, ldo, M, N, K, 1, stream);
+    if (out_dtype == MS_BF16) return launch_mt<EPI_STORE, bf16, false>(A, lda, w, ldw, bias, (bf16*)out, ldo, M, N, K, stream);
+    if (out_dtype == MS_F32) return launch_mt<EPI_STORE, float, false>(A, lda, w, ldw, bias, (float*)out, ldo, M, N, K, stream);
     return MS_BAD_ARG;
   }
   if (epilogue == EPI_SWIGLU) {
     if (N % 2 || ldo < N / 2 || out_dtype != MS_BF16 || bias) return MS_BAD_ARG;
-    return launch_mt<EPI_SWIGLU, bf16>(a, lda, w, ldw, nullptr, (bf16*)out, ldo, M, N, K, 1, stream);
+    return launch_mt<EPI_SWIGLU, bf16, false>(A, lda, w, ldw, nullptr, (bf16*)out, ldo, M, N, K, stream);
   }
   if (epilogue == EPI_RESIDUAL) {
     if (ldo < N || out_dtype != MS_F32) return MS_BAD_ARG;
-    return launch_mt<EPI_RESIDUAL, float>(a, lda, w, ldw, bias, (float*)out, ldo, M, N, K, 1, stream);
-  }
-  if (epilogue == EPI_PARTIAL) {
-    if (ldo < N || out_dtype != MS_F32 || splits < 1) return MS_BAD_ARG;
-    return launch_mt<EPI_PARTIAL, float>(a, lda, w, ldw, bias, (float*)out, ldo, M, N, K, splits, stream);
+    return launch_mt<EPI_RESIDUAL, float, false>(A, lda, w, ldw, bias, (float*)out, ldo, M, N, K, stream);
   }
   return MS_BAD_ARG;
 }
@@ -217,9 +219,9 @@ extern "C" int ms_gemm_skinny(const void* A, long long lda, const void* W, long 
 // As ms_gemm_skinny with epilogue 0 or 1, but the activations are rows of the float residual stream x[M,K]
 // and the RMS norm (weight norm_w[K], eps) that precedes the product is folded into the kernel.  With `rows`
 // (int32 [M]) row m of the product comes from x[rows[m]].
-extern "C" int ms_gemm_skinny_norm(const float* x, long long ldx, const int* rows, const float* norm_w, float eps, const void* W,
-                                   long long ldw, const float* bias, void* out, long long ldo, int M, int N, int K,
-                                   int epilogue, int out_dtype, hipStream_t stream) {
+extern "C" int ms_gemm_skinny_norm(const float* x, long long ldx, const int* rows, const float* norm_w, float eps,
+                                   const void* W, long long ldw, const float* bias, void* out, long long ldo, int M,
+                                   int N, int K, int epilogue, int out_dtype, hipStream_t stream) {
   if (M <= 0 || N <= 0) return MS_OK;
   if (M > 64) return MS_UNSUPPORTED;
   if (K <= 0 || K % 8 || ldx % 4 || ldw % 8 || ldx < K || ldw < K) return MS_UNSUPPORTED;
@@ -227,13 +229,13 @@ extern "C" int ms_gemm_skinny_norm(const float* x, long long ldx, const int* row
   const bf16* w = (const bf16*)W;
   if (epilogue == EPI_STORE) {
     if (ldo < N) return MS_BAD_ARG;
-    if (out_dtype == MS_BF16) return launch_mt<EPI_STORE, bf16, true>(x, ldx, w, ldw, bias, (bf16*)out, ldo, M, N, K, 1, stream, norm_w, eps, rows);
-    if (out_dtype == MS_F32) return launch_mt<EPI_STORE, float, true>(x, ldx, w, ldw, bias, (float*)out, ldo, M, N, K, 1, stream, norm_w, eps, rows);
+    if (out_dtype == MS_BF16) return launch_mt<EPI_STORE, bf16, true>(x, ldx, w, ldw, bias, (bf16*)out, ldo, M, N, K, stream, norm_w, eps, rows);
+    if (out_dtype == MS_F32) return launch_mt<EPI_STORE, float, true>(x, ldx, w, ldw, bias, (float*)out, ldo, M, N, K, stream, norm_w, eps, rows);
     return MS_BAD_ARG;
   }
   if (epilogue == EPI_SWIGLU) {
     if (N % 2 || ldo < N / 2 || out_dtype != MS_BF16 || bias) return MS_BAD_ARG;
-    return launch_mt<EPI_SWIGLU, bf16, true>(x, ldx, w, ldw, nullptr, (bf16*)out, ldo, M, N, K, 1, stream, norm_w, eps, rows);
+    return launch_mt<EPI_SWIGLU, bf16, true>(x, ldx, w, ldw, nullptr, (bf16*)out, ldo, M, N, K, stream, norm_w, eps, rows);
   }
   return MS_BAD_ARG;
 }

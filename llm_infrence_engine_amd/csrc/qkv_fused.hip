@@ -13,6 +13,26 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
+// sin and cos of a rotation angle for bfloat16 results: three-part Cody-Waite reduction by pi/2 (the first
+// two parts have 11 bits, so n * part is exact for |x| < 2^13 * pi/2) and short polynomials on [-pi/4, pi/4];
+// absolute error ~2e-7.  Larger angles take the library routine.
+__device__ __forceinline__ void sincos_rot(float x, float* sn, float* cs) {
+  if (fabsf(x) > 12000.f) { sincosf(x, sn, cs); return; }
+  const float n = rintf(x * 0.636619772367581343f);
+  float r = fmaf(-n, 1.5703125f, x);
+  r = fmaf(-n, 4.837512969970703e-4f, r);
+  r = fmaf(-n, 7.549790126404332e-08f, r);
+  const float r2 = r * r;
+  const float sp = fmaf(r2, fmaf(r2, fmaf(r2, 2.7557314297e-6f, -1.9841270114e-4f), 8.3333337680e-3f), -1.6666667163e-1f);
+  const float s0 = fmaf(r * r2, sp, r);
+  const float cp = fmaf(r2, fmaf(r2, fmaf(r2, 2.4801587642e-5f, -1.3888889225e-3f), 4.1666667908e-2f), -0.5f);
+  const float c0 = fmaf(r2, cp, 1.0f);
+  const int q = (int)n & 3;
+  const float s1 = (q & 1) ? c0 : s0, c1 = (q & 1) ? s0 : c0;
+  *sn = (q & 2) ? -s1 : s1;
+  *cs = ((q + 1) & 2) ? -c1 : c1;
+}
+
 template <int MT, int WAVES>
 __global__ void __launch_bounds__(WAVES * MS_WAVE)
 qkv_rope_store_kernel(const float* __restrict__ X, size_t ldx, const float* __restrict__ norm_w, float eps,
@@ -77,10 +97,13 @@ qkv_rope_store_kernel(const float* __restrict__ X, size_t ldx, const float* __re
     ss[t] += __shfl_xor(ss[t], 16, MS_WAVE);
     ss[t] += __shfl_xor(ss[t], 32, MS_WAVE);
     if (kq == 0) red_ss[wave][t][col] = ss[t];
-    if (wave > 0) { red[wave - 1][0][t][lane] = lo[t]; red[wave - 1][1][t][lane] = hi[t]; }
+    const int owner = t % WAVES;  // token group t is finished by wave t; the others leave their share in LDS
+    if (wave != owner) {
+      red[wave < owner ? wave : wave - 1][0][t][lane] = lo[t];
+      red[wave < owner ? wave : wave - 1][1][t][lane] = hi[t];
+    }
   }
   __syncthreads();
-  if (wave > 0) return;
 
   // lane holds features j0 + kq*4 + r (lo) and the same + d/2 (hi) of token t*16 + col
   const int j = j0 + kq * 4;
@@ -88,7 +111,8 @@ qkv_rope_store_kernel(const float* __restrict__ X, size_t ldx, const float* __re
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     const int m = t * 16 + col;
-    if (m >= M) continue;
+    const int owner = t % WAVES;
+    if (wave != owner || m >= M) continue;
     float total = 0.f;
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) total += red_ss[w][t][col];
@@ -96,9 +120,11 @@ qkv_rope_store_kernel(const float* __restrict__ X, size_t ldx, const float* __re
     float a[4], b[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      float va = lo[t][r], vb = hi[t][r];
-#pragma unroll
-      for (int w = 0; w < WAVES - 1; ++w) { va += red[w][0][t][lane][r]; vb += red[w][1][t][lane][r]; }
+      float va = 0.f, vb = 0.f;
+      for (int w = 0; w < WAVES; ++w) {  // in wave order
+        va += w == owner ? lo[t][r] : red[w < owner ? w : w - 1][0][t][lane][r];
+        vb += w == owner ? hi[t][r] : red[w < owner ? w : w - 1][1][t][lane][r];
+      }
       a[r] = va * inv + (bias ? bias[row_lo + r] : 0.f);
       b[r] = vb * inv + (bias ? bias[row_lo + half + r] : 0.f);
     }
@@ -107,7 +133,7 @@ qkv_rope_store_kernel(const float* __restrict__ X, size_t ldx, const float* __re
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         float sn, cs;
-        sincosf(pos * inv_freq[j + r], &sn, &cs);
+        sincos_rot(pos * inv_freq[j + r], &sn, &cs);
         const float x1 = a[r], x2 = b[r];
         a[r] = x1 * cs - x2 * sn;
         b[r] = x2 * cs + x1 * sn;
@@ -151,10 +177,11 @@ int launch(const float* X, size_t ldx, const float* norm_w, float eps, const bf1
            bf16* v_pages, int M, int K, int nh, int nkv, int d, int page_size, int v_transposed, hipStream_t stream) {
   const int blocks = (nh + 2 * nkv) * (d / 32);
   const int steps = (K + 31) / 32;
+  // LDS holds (waves - 1) * 2 * MT KB
   int waves = 4;
-  while (waves < 16 && blocks * waves < 1024 && steps >= waves * 2) waves *= 2;
+  while (waves < (MT == 1 ? 16 : 8) && blocks * waves < 1024 && steps >= waves * 2) waves *= 2;
 #define GO(WV) qkv_rope_store_kernel<MT, WV><<<dim3(blocks), dim3(WV * MS_WAVE), 0, stream>>>(X, ldx, norm_w, eps, W, bias, positions, inv_freq, slot_mapping, q_out, k_pages, v_pages, M, K, nh, nkv, d, page_size, v_transposed)
-  if (waves == 4) GO(4); else if (waves == 8) GO(8); else GO(16);
+  if (waves == 4) GO(4); else if (waves == 8) GO(8); else { if constexpr (MT == 1) GO(16); }
 #undef GO
   return ms_launch_status();
 }
@@ -179,7 +206,6 @@ extern "C" int ms_qkv_rope_store(const float* x, long long ldx, const float* nor
 #define GO(MT) return launch<MT>(x, ldx, norm_w, eps, (const bf16*)W, bias, positions, inv_freq, slot_mapping, (bf16*)q_out, (bf16*)k_pages, (bf16*)v_pages, M, K, num_heads, num_kv_heads, head_dim, page_size, v_transposed, stream)
   if (M <= 16) GO(1);
   if (M <= 32) GO(2);
-  if (M <= 48) GO(3);
   GO(4);
 #undef GO
 }

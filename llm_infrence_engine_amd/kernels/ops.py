@@ -27,9 +27,8 @@ _SIGNATURES = {
     "ms_qkv_rope_store": [_c_ptr, _c_ll, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                           _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "ms_bias_add": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
-    "ms_gemm_skinny_splits": [_c_int, _c_int],
     "ms_gemm_skinny": [_c_ptr, _c_ll, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int,
-                       _c_int, _c_ptr],
+                       _c_ptr],
     "ms_residual_add": [_c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr],
     "ms_silu_mul": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "ms_rope_store": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int,
@@ -221,7 +220,7 @@ def gemm_generic(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, bias: Opti
 
 
 SKINNY_MAX_ROWS = 64
-EPI_STORE, EPI_SWIGLU, EPI_PARTIAL, EPI_RESIDUAL = 0, 1, 2, 3
+EPI_STORE, EPI_SWIGLU, EPI_RESIDUAL = 0, 1, 3
 
 
 def skinny_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
@@ -232,12 +231,10 @@ def skinny_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
 
 
 def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, epilogue: int = EPI_STORE,
-                splits: int = 1, out_dtype: torch.dtype = torch.bfloat16,
-                residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+                out_dtype: torch.dtype = torch.bfloat16, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
     """a [M <= 64, K] @ w [N, K].T on the matrix cores, bfloat16 in.  Epilogues: EPI_STORE -> [M, N] (+ bias);
-    EPI_SWIGLU -> [M, N / 2] = silu(even rows' products) * odd rows' products; EPI_PARTIAL -> float [S, M, N]
-    partial sums over slices of K (bias in the first), to be added in order by the consumer; EPI_RESIDUAL ->
-    ``residual`` (float [M, N]) += product + bias, in place."""
+    EPI_SWIGLU -> [M, N / 2] = silu(even rows' products) * odd rows' products; EPI_RESIDUAL -> ``residual``
+    (float [M, N]) += product + bias, in place."""
     _check(a, "a", torch.bfloat16, contiguous=False)
     _check(w, "w", torch.bfloat16)
     if a.dim() != 2 or w.dim() != 2 or a.shape[1] != w.shape[1]:
@@ -259,13 +256,10 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] =
     elif epilogue == EPI_RESIDUAL:
         _check(residual, "residual", torch.float32, (M, N))
         out, ldo, out_dtype = residual, N, torch.float32
-    elif epilogue == EPI_PARTIAL:
-        splits = _get("ms_gemm_skinny_splits")(K, splits)
-        out, ldo, out_dtype = torch.empty((splits, M, N), dtype=torch.float32, device=a.device), N, torch.float32
     else:
         raise ValueError(f"unknown epilogue {epilogue}")
     _call("ms_gemm_skinny", a.data_ptr(), a.stride(0) if M > 1 else K, w.data_ptr(), K, _ptr(bias), out.data_ptr(), ldo,
-          M, N, K, epilogue, splits, _code(out_dtype), _stream())
+          M, N, K, epilogue, _code(out_dtype), _stream())
     return out
 
 

@@ -273,7 +273,7 @@ def test_ops_refuse_cpu_tensors_and_wrong_shapes(ops):
 
 
 @pytest.mark.parametrize("M", [1, 8, 16, 17, 33, 64])
-@pytest.mark.parametrize("N,K", [(1152, 896), (331, 72), (896, 4864), (50, 200)])
+@pytest.mark.parametrize("N,K", [(1152, 896), (331, 72), (896, 4864), (50, 200), (9728, 104), (17000, 64)])
 def test_gemm_skinny(ops, M, N, K):
     g = torch.Generator().manual_seed(M * 1000 + N)
     a = torch.randn(M, K, generator=g).bfloat16().to(DEV)
@@ -285,10 +285,6 @@ def test_gemm_skinny(ops, M, N, K):
     f = ops.gemm_skinny(a, w, None, out_dtype=torch.float32)
     assert f.dtype == torch.float32
     torch.testing.assert_close(f.double(), want, atol=2e-5, rtol=2e-5)
-    for splits in (2, 5):
-        parts = ops.gemm_skinny(a, w, bias, ops.EPI_PARTIAL, splits=splits)
-        assert parts.dim() == 3 and parts.shape[1:] == (M, N) and parts.shape[0] <= splits
-        torch.testing.assert_close(parts.double().sum(0), want + bias.double(), atol=2e-5, rtol=2e-5)
     x = torch.randn(M, N, generator=g).to(DEV)
     x0 = x.clone()
     ops.gemm_skinny(a, w, bias, ops.EPI_RESIDUAL, residual=x)
