@@ -43,15 +43,25 @@ struct KVBlock {           // one block of 32 keys as this lane sees it
   bf16x4 v[D / 16][2];     // [16-dim tile][subtile]: 4 keys of one dim
 };
 
+// The pages of the two 16-key halves of the block at `base`; past the context: the null page.
+__device__ __forceinline__ void pages_of(const int* __restrict__ table, int base, int key_hi, int page_size,
+                                         int* pages) {
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int kb = base + u * 16;
+    pages[u] = kb <= key_hi ? table[kb / page_size] : 0;
+  }
+}
+
 template <int D>
 __device__ __forceinline__ void load_block(KVBlock<D>& b, const bf16* __restrict__ k_pages,
-                                           const bf16* __restrict__ vt_pages, const int* __restrict__ table,
-                                           int base, int key_hi, int g, int nkv, int page_size, int lane) {
+                                           const bf16* __restrict__ vt_pages, const int* pages,
+                                           int base, int g, int nkv, int page_size, int lane) {
   const int col = lane & 15, kq = lane >> 4;
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
     const int kb = base + u * 16;
-    const int page = kb <= key_hi ? table[kb / page_size] : 0;  // past the context: the null page
+    const int page = pages[u];
     const int off = kb % page_size;
     const bf16* kp = k_pages + (((size_t)page * nkv + g) * page_size + off + col) * D + kq * 8;
 #pragma unroll
@@ -76,13 +86,21 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
   const int col16 = lane & 15, kq = lane >> 4;
   const int r = blockIdx.z, g = blockIdx.y;
   const int rep = nh / nkv;
+  const int* table = block_table + (size_t)r * table_stride;
+  // Without a window a wave's first key block is known before the request's lengths are: ask for its page
+  // ids at once, so that they travel together with the lengths instead of after them.
+  int first_pages[2] = {0, 0};
+  const bool early = !SPLIT && window <= 0;
+  if (early) {
+#pragma unroll
+    for (int u = 0; u < 2; ++u) first_pages[u] = table[min((wave * 32 + u * 16) / page_size, table_stride - 1)];
+  }
   const int q0 = q_start[r];
   const int qlen = q_start[r + 1] - q0;
   const int start_pos = context_lens[r] - qlen;
   const int ncols = qlen * rep;
   const int c0 = SPLIT ? 0 : blockIdx.x * 16 * NT;
   if (c0 >= ncols) return;
-  const int* table = block_table + (size_t)r * table_stride;
 
   // key range of the tile: from the first column's window start to the last column's own position
   const int last_col = min(ncols, c0 + 16 * NT) - 1;
@@ -126,12 +144,24 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
   }
 
   KVBlock<D> cur, nxt;
-  if (blk_begin + wave < blk_end)
-    load_block<D>(cur, k_pages, vt_pages, table, (blk_begin + wave) * 32, key_hi, g, nkv, page_size, lane);
+  if (blk_begin + wave < blk_end) {
+    const int base = (blk_begin + wave) * 32;
+    int pages[2];
+    if (early) {  // blk_begin is 0 here; halves past the last key fall back to the null page
+#pragma unroll
+      for (int u = 0; u < 2; ++u) pages[u] = base + u * 16 <= key_hi ? first_pages[u] : 0;
+    } else {
+      pages_of(table, base, key_hi, page_size, pages);
+    }
+    load_block<D>(cur, k_pages, vt_pages, pages, base, g, nkv, page_size, lane);
+  }
   for (int blk = blk_begin + wave; blk < blk_end; blk += WAVES) {
     const int base = blk * 32;
-    if (blk + WAVES < blk_end)
-      load_block<D>(nxt, k_pages, vt_pages, table, base + WAVES * 32, key_hi, g, nkv, page_size, lane);
+    if (blk + WAVES < blk_end) {
+      int pages[2];
+      pages_of(table, base + WAVES * 32, key_hi, page_size, pages);
+      load_block<D>(nxt, k_pages, vt_pages, pages, base + WAVES * 32, g, nkv, page_size, lane);
+    }
 
     // scores: s[u][t] holds keys base + u*16 + kq*4 + (0..3) of column t*16 + col16
     f32x4 s[2][NT];
@@ -335,8 +365,8 @@ extern "C" int ms_paged_attention_mfma(const void* q, long long q_stride, const 
 #define GO(D, NT, WV) return launch_general<D, NT, WV>((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)vt_pages, block_table, table_stride, q_start, context_lens, (bf16*)out, out_stride, n_requests, max_q_len, num_heads, num_kv_heads, page_size, scale, window, stream)
   // few columns (a decode step): one narrow tile per request, more waves over its keys
   const int cols = max_q_len * (num_heads / num_kv_heads);
-  if (head_dim == 32) { if (cols > 16) GO(32, 4, 4); else GO(32, 1, 8); }
-  if (head_dim == 64) { if (cols > 16) GO(64, 4, 4); else GO(64, 1, 8); }
+  if (head_dim == 32) { if (cols > 16) GO(32, 4, 4); else GO(32, 1, 16); }
+  if (head_dim == 64) { if (cols > 16) GO(64, 4, 4); else GO(64, 1, 16); }
   if (cols > 16) GO(128, 2, 4); else GO(128, 1, 8);
 #undef GO
 }

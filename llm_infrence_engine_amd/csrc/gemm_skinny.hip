@@ -52,6 +52,28 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
     arow[t] = (size_t)(rows ? rows[m] : m) * lda + kq * 8;  // rows: the activations are gathered rows of A
   }
 
+  // what the epilogue will need from memory is asked for now, so that it arrives under the main loop
+  f32x4 pre[NTILE][MT];   // the residual values this wave will add to (EPI_RESIDUAL)
+  f32x4 bv[NTILE];        // bias of this lane's 4 features per tile
+#pragma unroll
+  for (int u = 0; u < NTILE; ++u) {
+    const int nb = n0 + u * 16 + kq * 4;
+    bv[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (bias && EPI != EPI_SWIGLU) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) if (nb + r < N) bv[u][r] = bias[nb + r];
+    }
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      pre[u][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (EPI == EPI_RESIDUAL && wave == (u * MT + t) % WAVES && t * 16 + col < M) {
+        const float* o = reinterpret_cast<const float*>(out) + (size_t)(t * 16 + col) * ldo + nb;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) if (nb + r < N) pre[u][t][r] = o[r];
+      }
+    }
+  }
+
   f32x4 acc[NTILE][MT];
   float ss[MT];
 #pragma unroll
@@ -61,7 +83,8 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
     for (int u = 0; u < NTILE; ++u) acc[u][t] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-#pragma unroll 2
+  // the loads of several steps are in flight together: the kernel lives on memory parallelism
+#pragma unroll (MT * NTILE <= 2 ? 8 : 4)
   for (int s = wave; s < total_steps; s += WAVES) {
     const int k = s * 32;
     const bool in = k + kq * 8 < K;  // K is a multiple of 8: a lane's 8 values are all inside or all outside
@@ -149,11 +172,7 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
         TO* o = out + (size_t)m * ldo + nb;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          if (nb + r < N) {
-            float v = sum[r] + (bias ? bias[nb + r] : 0.f);
-            if (EPI == EPI_RESIDUAL) v += to_float(o[r]);
-            o[r] = from_float<TO>(v);
-          }
+          if (nb + r < N) o[r] = from_float<TO>(sum[r] + bv[u][r] + pre[u][t][r]);
         }
       }
     }

@@ -56,12 +56,29 @@ qkv_rope_store_kernel(const float* __restrict__ X, size_t ldx, const float* __re
 #pragma unroll
   for (int t = 0; t < MT; ++t) xrow[t] = (size_t)min(t * 16 + col, M - 1) * ldx + kq * 8;
 
+  // what the epilogue will need from memory is asked for now, so that it arrives under the main loop
+  const int jl = j0 + kq * 4;
+  float b_lo[4], b_hi[4], freq[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    b_lo[r] = bias ? bias[head * d + jl + r] : 0.f;
+    b_hi[r] = bias ? bias[head * d + jl + half + r] : 0.f;
+    freq[r] = head < nh + nkv ? inv_freq[jl + r] : 0.f;
+  }
+  int pos_m[MT], slot_m[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int m = min(t * 16 + col, M - 1);
+    pos_m[t] = positions[m];
+    slot_m[t] = slot_mapping[m];
+  }
+
   f32x4 lo[MT], hi[MT];
   float ss[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) { lo[t] = hi[t] = f32x4{0.f, 0.f, 0.f, 0.f}; ss[t] = 0.f; }
 
-#pragma unroll 2
+#pragma unroll (MT == 1 ? 4 : 2)
   for (int s = wave; s < total_steps; s += WAVES) {
     const int k = s * 32;
     const bool in = k + kq * 8 < K;
@@ -125,15 +142,15 @@ qkv_rope_store_kernel(const float* __restrict__ X, size_t ldx, const float* __re
         va += w == owner ? lo[t][r] : red[w < owner ? w : w - 1][0][t][lane][r];
         vb += w == owner ? hi[t][r] : red[w < owner ? w : w - 1][1][t][lane][r];
       }
-      a[r] = va * inv + (bias ? bias[row_lo + r] : 0.f);
-      b[r] = vb * inv + (bias ? bias[row_lo + half + r] : 0.f);
+      a[r] = va * inv + b_lo[r];
+      b[r] = vb * inv + b_hi[r];
     }
     if (head < nh + nkv) {  // q and k heads turn by position * inv_freq[j]
-      const float pos = (float)positions[m];
+      const float pos = (float)pos_m[t];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         float sn, cs;
-        sincos_rot(pos * inv_freq[j + r], &sn, &cs);
+        sincos_rot(pos * freq[r], &sn, &cs);
         const float x1 = a[r], x2 = b[r];
         a[r] = x1 * cs - x2 * sn;
         b[r] = x2 * cs + x1 * sn;
@@ -148,7 +165,7 @@ qkv_rope_store_kernel(const float* __restrict__ X, size_t ldx, const float* __re
       *reinterpret_cast<bf16x4*>(qp + half) = pb;
       continue;
     }
-    const long long slot = slot_mapping[m];
+    const long long slot = slot_m[t];
     if (slot < 0) continue;
     const long long page = slot / page_size;
     const int off = (int)(slot % page_size);
