@@ -18,7 +18,7 @@ int ms_residual_add(float* x, const void* delta, long long total, int dtype, hip
 
 int ms_silu_mul(const void* gate_up, void* out, int n_tokens, int intermediate, int dtype, hipStream_t stream);
 
-int ms_rope_store(void* qkv, const int* positions, const float* inv_freq, const int* slot_mapping, void* k_pages,
+int ms_rope_store(void* qkv, const float* bias, const int* positions, const float* inv_freq, const int* slot_mapping, void* k_pages,
                   void* v_pages, int n_tokens, int num_heads, int num_kv_heads, int head_dim, int rot_dim,
                   int page_size, int v_transposed, int dtype, hipStream_t stream);
 

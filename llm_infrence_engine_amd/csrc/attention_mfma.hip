@@ -99,7 +99,8 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
   const int qlen = q_start[r + 1] - q0;
   const int start_pos = context_lens[r] - qlen;
   const int ncols = qlen * rep;
-  const int c0 = SPLIT ? 0 : blockIdx.x * 16 * NT;
+  // late tiles of a prompt see the most keys: they go first so that the long ones do not finish last
+  const int c0 = SPLIT ? 0 : (gridDim.x - 1 - blockIdx.x) * 16 * NT;
   if (c0 >= ncols) return;
 
   // key range of the tile: from the first column's window start to the last column's own position
@@ -108,6 +109,10 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
   int key_lo = 0;
   if (window > 0) key_lo = max(0, start_pos + c0 / rep - window + 1);
   int blk_begin = key_lo / 32, blk_end = key_hi / 32 + 1;
+  // a block whose keys every column of the tile sees needs no mask: all keys at or before the first column's
+  // position (and, with a window, after the last column's window start); tiles with idle columns always mask
+  const int first_pos = start_pos + c0 / rep;
+  const bool full_tile = c0 + 16 * NT <= ncols;
   if (SPLIT) {
     // every request spreads its own key blocks evenly over the splits (at least min_blocks each)
     const int per = max(min_blocks, (blk_end - blk_begin + n_splits - 1) / n_splits);
@@ -187,20 +192,32 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
           }
     }
 
+    const bool unmasked = full_tile && base + 31 <= first_pos && (window <= 0 || base > key_hi - window);
     bf16x8 p[NT];
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
       float bm = -INFINITY;
+      if (unmasked) {
 #pragma unroll
-      for (int u = 0; u < 2; ++u)
+        for (int u = 0; u < 2; ++u)
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int key = base + u * 16 + kq * 4 + i;
-          const bool see = key <= pos[t] && (window <= 0 || key > pos[t] - window);
-          const float v = see ? s[u][t][i] * scale_log2e : -INFINITY;
-          s[u][t][i] = v;
-          bm = fmaxf(bm, v);
-        }
+          for (int i = 0; i < 4; ++i) {
+            const float v = s[u][t][i] * scale_log2e;
+            s[u][t][i] = v;
+            bm = fmaxf(bm, v);
+          }
+      } else {
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int key = base + u * 16 + kq * 4 + i;
+            const bool see = key <= pos[t] && (window <= 0 || key > pos[t] - window);
+            const float v = see ? s[u][t][i] * scale_log2e : -INFINITY;
+            s[u][t][i] = v;
+            bm = fmaxf(bm, v);
+          }
+      }
       bm = fmaxf(bm, __shfl_xor(bm, 16, MS_WAVE));
       bm = fmaxf(bm, __shfl_xor(bm, 32, MS_WAVE));
       const float m_new = fmaxf(m[t], bm);

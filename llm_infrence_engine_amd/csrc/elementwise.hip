@@ -40,7 +40,31 @@ __global__ void rms_norm_kernel(float* __restrict__ x, const TD* __restrict__ de
   const int r = blockIdx.x;
   const int src = rows ? rows[r] : r;
   float* xr = x + (size_t)src * H;
+  T* o = out + (size_t)r * H;
   float ss = 0.f;
+  if (H % 4 == 0 && n_partials == 1) {  // four values at a time (rows start 16-byte aligned when H % 4 == 0)
+    const TD* dr = delta ? delta + (size_t)src * H : nullptr;
+    for (int i = threadIdx.x * 4; i < H; i += blockDim.x * 4) {
+      float4 v = *reinterpret_cast<const float4*>(xr + i);
+      if (dr) {
+        v.x += to_float(dr[i]); v.y += to_float(dr[i + 1]); v.z += to_float(dr[i + 2]); v.w += to_float(dr[i + 3]);
+        if (write_back) *reinterpret_cast<float4*>(xr + i) = v;
+      }
+      *reinterpret_cast<float4*>(buf + i) = v;
+      ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+    }
+    ss = block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+    for (int i = threadIdx.x * 4; i < H; i += blockDim.x * 4) {
+      const float4 v = *reinterpret_cast<const float4*>(buf + i);
+      const float4 g = *reinterpret_cast<const float4*>(w + i);
+      o[i] = from_float<T>(g.x * (v.x * inv));
+      o[i + 1] = from_float<T>(g.y * (v.y * inv));
+      o[i + 2] = from_float<T>(g.z * (v.z * inv));
+      o[i + 3] = from_float<T>(g.w * (v.w * inv));
+    }
+    return;
+  }
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
     float v = xr[i];
     if (delta) {
@@ -52,7 +76,6 @@ __global__ void rms_norm_kernel(float* __restrict__ x, const TD* __restrict__ de
   }
   ss = block_sum(ss, red);
   const float inv = 1.0f / sqrtf(ss / (float)H + eps);
-  T* o = out + (size_t)r * H;
   for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = from_float<T>(w[i] * (buf[i] * inv));
 }
 
@@ -123,11 +146,31 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, i
   size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   const size_t stride = (size_t)gridDim.x * blockDim.x;
   for (; idx < total; idx += stride) {
-    const size_t n = idx / I;
-    const int i = (int)(idx - n * I);
-    const float g = to_float(gu[n * 2 * I + 2 * i]);
-    const float u = to_float(gu[n * 2 * I + 2 * i + 1]);
+    // out[n, i] sits at idx and its (gate, up) pair at 2 * idx: rows are contiguous, so no division is needed
+    const float g = to_float(gu[2 * idx]);
+    const float u = to_float(gu[2 * idx + 1]);
     out[idx] = from_float<T>(g / (1.0f + expf(-g)) * u);
+  }
+}
+
+// bfloat16, eight outputs per thread: two 16-byte loads, one 16-byte store
+__global__ void silu_mul_bf16x8_kernel(const uint4* __restrict__ gu, uint4* __restrict__ out, size_t total8) {
+  size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; idx < total8; idx += stride) {
+    const uint4 a = gu[2 * idx], b = gu[2 * idx + 1];
+    const unsigned in[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};  // each word: gate (low half), up (high half)
+    unsigned short r[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float g = __uint_as_float(in[i] << 16), u = __uint_as_float(in[i] & 0xffff0000u);
+      const bf16 h = __float2bfloat16(g / (1.0f + expf(-g)) * u);
+      r[i] = *reinterpret_cast<const unsigned short*>(&h);
+    }
+    uint4 o;
+    o.x = r[0] | ((unsigned)r[1] << 16); o.y = r[2] | ((unsigned)r[3] << 16);
+    o.z = r[4] | ((unsigned)r[5] << 16); o.w = r[6] | ((unsigned)r[7] << 16);
+    out[idx] = o;
   }
 }
 
@@ -139,6 +182,11 @@ extern "C" int ms_silu_mul(const void* gate_up, void* out, int n_tokens, int int
   int blocks = (int)((total + 255) / 256);
   if (blocks > 8192) blocks = 8192;
   if (dtype == MS_F32) silu_mul_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gate_up, (float*)out, intermediate, total);
+  else if (dtype == MS_BF16 && total % 8 == 0 && (uintptr_t)gate_up % 16 == 0 && (uintptr_t)out % 16 == 0) {
+    int b8 = (int)((total / 8 + 255) / 256);
+    if (b8 > 16384) b8 = 16384;
+    silu_mul_bf16x8_kernel<<<b8, 256, 0, stream>>>((const uint4*)gate_up, (uint4*)out, total / 8);
+  }
   else if (dtype == MS_BF16) silu_mul_kernel<bf16><<<blocks, 256, 0, stream>>>((const bf16*)gate_up, (bf16*)out, intermediate, total);
   else return MS_BAD_ARG;
   return ms_launch_status();
@@ -148,12 +196,13 @@ extern "C" int ms_silu_mul(const void* gate_up, void* out, int n_tokens, int int
 // One block per token.  qkv[n] = [q heads | k heads | v heads], head_dim values each.
 // The first rot_dim values of every q and k head are rotated with half-split pairing (j, j + rot_dim/2):
 //   x1' = x1 cos - x2 sin,  x2' = x2 cos + x1 sin,  angle = float(position) * inv_freq[j]
+// With `bias` ([(nh + 2 nkv) d] float) it is added to q, k and v first, for a projection that came without it.
 // q is rotated in place.  With pages given, the rotated k and v go to
 // pages[slot / page_size][kv head][slot % page_size][:] for slot = slot_mapping[n] (slot < 0: not stored;
 // with v_transposed the value goes to v_pages[page][kv head][:][slot % page_size]);
 // k is also rotated in place so that a caller without pages sees it.
 template <typename T>
-__global__ void rope_store_kernel(T* __restrict__ qkv, const int* __restrict__ positions,
+__global__ void rope_store_kernel(T* __restrict__ qkv, const float* __restrict__ bias, const int* __restrict__ positions,
                                   const float* __restrict__ inv_freq, const int* __restrict__ slot_mapping,
                                   T* __restrict__ k_pages, T* __restrict__ v_pages, int nh, int nkv, int d,
                                   int rot_dim, int page_size, int v_transposed) {
@@ -173,9 +222,21 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const int* __restrict__ p
     T* x = row + (size_t)h * d;
     float s, c;
     sincosf(pos * inv_freq[j], &s, &c);
-    const float x1 = to_float(x[j]), x2 = to_float(x[j + half]);
+    float x1 = to_float(x[j]), x2 = to_float(x[j + half]);
+    if (bias) { x1 += bias[h * d + j]; x2 += bias[h * d + j + half]; }
     x[j] = from_float<T>(x1 * c - x2 * s);
     x[j + half] = from_float<T>(x2 * c + x1 * s);
+  }
+  if (bias) {  // what is not rotated still gets its bias: the tails of q and k heads beyond rot_dim, and v
+    const int tail = d - rot_dim;
+    for (int w = threadIdx.x; w < n_rot_heads * tail; w += blockDim.x) {
+      const int idx = (w / tail) * d + rot_dim + w % tail;
+      row[idx] = from_float<T>(to_float(row[idx]) + bias[idx]);
+    }
+    for (int w = threadIdx.x; w < nkv * d; w += blockDim.x) {
+      const int idx = (nh + nkv) * d + w;
+      row[idx] = from_float<T>(to_float(row[idx]) + bias[idx]);
+    }
   }
   if (slot < 0) return;
   __syncthreads();
@@ -191,7 +252,7 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const int* __restrict__ p
   }
 }
 
-extern "C" int ms_rope_store(void* qkv, const int* positions, const float* inv_freq, const int* slot_mapping,
+extern "C" int ms_rope_store(void* qkv, const float* bias, const int* positions, const float* inv_freq, const int* slot_mapping,
                              void* k_pages, void* v_pages, int n_tokens, int num_heads, int num_kv_heads,
                              int head_dim, int rot_dim, int page_size, int v_transposed, int dtype,
                              hipStream_t stream) {
@@ -202,7 +263,7 @@ extern "C" int ms_rope_store(void* qkv, const int* positions, const float* inv_f
   if (k_pages && (page_size <= 0 || slot_mapping == nullptr)) return MS_BAD_ARG;
   if (rot_dim > 0 && (positions == nullptr || inv_freq == nullptr)) return MS_BAD_ARG;
   dim3 grid(n_tokens), block(256);
-#define LAUNCH(T) rope_store_kernel<T><<<grid, block, 0, stream>>>((T*)qkv, positions, inv_freq, slot_mapping, (T*)k_pages, (T*)v_pages, num_heads, num_kv_heads, head_dim, rot_dim, page_size, v_transposed)
+#define LAUNCH(T) rope_store_kernel<T><<<grid, block, 0, stream>>>((T*)qkv, bias, positions, inv_freq, slot_mapping, (T*)k_pages, (T*)v_pages, num_heads, num_kv_heads, head_dim, rot_dim, page_size, v_transposed)
   if (dtype == MS_F32) LAUNCH(float);
   else if (dtype == MS_BF16) LAUNCH(bf16);
   else return MS_BAD_ARG;

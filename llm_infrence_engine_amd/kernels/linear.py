@@ -59,6 +59,12 @@ def _library_mm(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> Opt
     return torch.mm(a, w.t(), out_dtype=out_dtype) if _mm_out_dtype_ok else None
 
 
+def goes_to_library(a, w: torch.Tensor) -> bool:
+    """Whether ``linear(a, w)`` is the library's product (which comes without a bias epilogue)."""
+    return (isinstance(a, torch.Tensor) and a.dtype == torch.bfloat16 and not ops.skinny_ok(a, w)
+            and a.shape[0] > ops.SKINNY_MAX_ROWS and a.is_contiguous())
+
+
 def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
            out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """[M, K] x [N, K] -> [M, N] in ``out_dtype`` (default: a's type).  ``a`` may be a ``LazyNorm``."""

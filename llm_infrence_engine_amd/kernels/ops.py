@@ -31,7 +31,7 @@ _SIGNATURES = {
                        _c_ptr],
     "ms_residual_add": [_c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr],
     "ms_silu_mul": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
-    "ms_rope_store": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int,
+    "ms_rope_store": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int,
                       _c_int, _c_int, _c_int, _c_ptr],
     "ms_gemm_generic": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ll, _c_ll, _c_ll, _c_int,
                         _c_int, _c_int, _c_ptr],
@@ -174,8 +174,9 @@ def _v_shape(k_pages: torch.Tensor, v_transposed: bool):
 def rope_store(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, rot_dim: int = 0,
                positions: Optional[torch.Tensor] = None, inv_freq: Optional[torch.Tensor] = None,
                slot_mapping: Optional[torch.Tensor] = None, k_pages: Optional[torch.Tensor] = None,
-               v_pages: Optional[torch.Tensor] = None, v_transposed: bool = False) -> torch.Tensor:
-    """Rotate q and k of ``qkv`` [N, (nh + 2 nkv) d] in place and store k, v into pages
+               v_pages: Optional[torch.Tensor] = None, v_transposed: bool = False,
+               bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Add ``bias`` (if given), rotate q and k of ``qkv`` [N, (nh + 2 nkv) d] in place and store k, v into pages
     [pages, nkv, page_size, d] at ``slot_mapping`` (page * page_size + offset); with ``v_transposed`` the
     value pages are [pages, nkv, d, page_size]."""
     _check(qkv, "qkv", None, (None, (num_heads + 2 * num_kv_heads) * head_dim))
@@ -191,7 +192,9 @@ def rope_store(qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: i
         page_size = k_pages.shape[2]
         _check(v_pages, "v_pages", qkv.dtype, _v_shape(k_pages, v_transposed))
         _check(slot_mapping, "slot_mapping", torch.int32, (N,))
-    _call("ms_rope_store", qkv.data_ptr(), _ptr(positions), _ptr(inv_freq), _ptr(slot_mapping), _ptr(k_pages),
+    if bias is not None:
+        _check(bias, "bias", torch.float32, (qkv.shape[1],))
+    _call("ms_rope_store", qkv.data_ptr(), _ptr(bias), _ptr(positions), _ptr(inv_freq), _ptr(slot_mapping), _ptr(k_pages),
           _ptr(v_pages), N, num_heads, num_kv_heads, head_dim, rot_dim, page_size, int(v_transposed),
           _code(qkv.dtype), _stream())
     return qkv

@@ -75,8 +75,14 @@ class GQAttention(Mixer):
         if self.position is not None:
             q = self.position.project_encode_store(h, self.w_qkv, self.b_qkv, nh, nkv, d, ctx, kv)
         if q is None:
-            q = linear.linear(h, self.w_qkv, bias=self.b_qkv)   # [N, (nh + 2 nkv) d]: attention reads its q part
-            if self.position is not None:
+            # [N, (nh + 2 nkv) d]: attention reads its q part.  A library product has no bias epilogue; a position
+            # encoding that can add the bias on its way saves a pass over the projection.
+            late_bias = (self.b_qkv is not None and getattr(self.position, "adds_bias", False)
+                         and linear.goes_to_library(h, self.w_qkv))
+            q = linear.linear(h, self.w_qkv, bias=None if late_bias else self.b_qkv)
+            if late_bias:
+                self.position.encode_and_store(q, nh, nkv, d, ctx, kv, bias=self.b_qkv)
+            elif self.position is not None:
                 self.position.encode_and_store(q, nh, nkv, d, ctx, kv)
             elif kv.store:
                 ops.rope_store(q, nh, nkv, d, 0, None, None, kv.slot_mapping, kv.k_pages, kv.v_pages, kv.v_transposed)

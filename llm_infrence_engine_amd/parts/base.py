@@ -140,7 +140,8 @@ class PositionEncoding(Part):
     def encode_and_store(self, qkv: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int,
                          ctx: StepContext, kv: Optional[KVView]) -> None:
         """Encode positions into the q and k parts of ``qkv`` [N, (nh + 2 nkv) d] in place and, if ``kv``
-        stores, put k and v into its pages."""
+        stores, put k and v into its pages.  A part with ``adds_bias = True`` also takes ``bias=`` (float
+        [(nh + 2 nkv) d]) and adds it to q, k and v first."""
         raise NotImplementedError
 
 

@@ -14,6 +14,8 @@ from .base import PositionEncoding, register_part
 
 
 class RotaryHalf(PositionEncoding):
+    adds_bias = True   # encode_and_store takes ``bias`` and adds it to q, k, v before rotating and storing
+
     def __init__(self, prefix: str, head_dim: int, rotary_dim: int, theta: float):
         if rotary_dim % 2 or not 0 < rotary_dim <= head_dim:
             raise ValueError(f"rotary_dim {rotary_dim} must be even and within head_dim {head_dim}")
@@ -31,11 +33,11 @@ class RotaryHalf(PositionEncoding):
         return ops.qkv_rope_store(h.x, h.weight, h.eps, w_qkv, bias, num_heads, num_kv_heads, head_dim, ctx.positions,
                                   self.inv_freq, kv.slot_mapping, kv.k_pages, kv.v_pages, kv.v_transposed)
 
-    def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, ctx, kv):
+    def encode_and_store(self, qkv, num_heads, num_kv_heads, head_dim, ctx, kv, bias=None):
         store = kv is not None and kv.store
         ops.rope_store(qkv, num_heads, num_kv_heads, head_dim, self.rotary_dim, ctx.positions, self.inv_freq,
                        kv.slot_mapping if store else None, kv.k_pages if store else None,
-                       kv.v_pages if store else None, store and kv.v_transposed)
+                       kv.v_pages if store else None, store and kv.v_transposed, bias)
 
 
 class NoPosition(PositionEncoding):

@@ -132,8 +132,12 @@ def test_rope_store(ops, dtype, nh, nkv, d, rot):
     kp = torch.zeros(pages, nkv, page_size, d, dtype=dtype, device=DEV)
     vp = torch.zeros_like(kp)
     dev = qkv.to(DEV)
-    ops.rope_store(dev, nh, nkv, d, rot, pos.to(DEV), inv_freq.to(DEV), slots.to(DEV), kp, vp)
+    bias = torch.randn((nh + 2 * nkv) * d, generator=g) if rot != 16 else None   # with and without a late bias
+    ops.rope_store(dev, nh, nkv, d, rot, pos.to(DEV), inv_freq.to(DEV), slots.to(DEV), kp, vp,
+                   bias=None if bias is None else bias.to(DEV))
     x = qkv.double().view(N, nh + 2 * nkv, d)
+    if bias is not None:
+        x = x + bias.double().view(1, nh + 2 * nkv, d)
     want_q = rope_reference(x[:, :nh], pos, rot, inv_freq.double())
     want_k = rope_reference(x[:, nh:nh + nkv], pos, rot, inv_freq.double())
     got = dev.double().cpu().view(N, nh + 2 * nkv, d)
@@ -143,14 +147,14 @@ def test_rope_store(ops, dtype, nh, nkv, d, rot):
     torch.testing.assert_close(got[:, nh:nh + nkv], want_k, **t)
     small = pos < 200  # there the float angle is exact to ~1e-5
     torch.testing.assert_close(got[small][:, :nh], want_q[small], **tol(dtype))
-    assert torch.equal(got[:, nh + nkv:], x[:, nh + nkv:])
+    torch.testing.assert_close(got[:, nh + nkv:], x[:, nh + nkv:], **(tol(dtype) if bias is not None else dict(atol=0, rtol=0)))
     for n in range(N):
         s = int(slots[n])
         if s < 0:
             continue
         p, o = divmod(s, page_size)
         assert torch.equal(kp[p, :, o].cpu().double(), got[n, nh:nh + nkv])
-        assert torch.equal(vp[p, :, o].cpu().double(), x[n, nh + nkv:])
+        assert torch.equal(vp[p, :, o].cpu().double(), got[n, nh + nkv:])
     used = torch.zeros(pages * page_size, dtype=torch.bool)
     used[slots[slots >= 0].long()] = True
     assert (kp.cpu().permute(0, 2, 1, 3).reshape(pages * page_size, -1)[~used] == 0).all()
