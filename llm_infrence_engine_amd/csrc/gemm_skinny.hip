@@ -178,7 +178,12 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
     }
 }
 
+// Tuning knob: force (tiles per block, waves) for every launch; 0 leaves the choice to the heuristic below.
+int g_force_ntile = 0, g_force_waves = 0;
+
 // The shapes of block on offer: (tiles per block, waves).  LDS holds (waves - 1) * tiles * MT KB.
+// (Splitting K over blocks as well, with the last block to arrive adding the partial sums, was measured and
+// dropped: the device-scope fences it needs cost several microseconds per block on this chip.)
 template <int MT, int EPI, typename TO, bool NORM>
 int launch_cfg(const void* A, size_t lda, const bf16* W, size_t ldw, const float* bias, TO* out, size_t ldo, int M,
                int N, int K, hipStream_t stream, const float* norm_w, float eps, const int* rows) {
@@ -186,15 +191,15 @@ int launch_cfg(const void* A, size_t lda, const bf16* W, size_t ldw, const float
   const int steps = (K + 31) / 32;
   // as many tiles per block as still leaves a block for every CU; narrow outputs keep one tile per block
   // (two when there are several token groups, whose activations would otherwise be read once per tile)
-  int ntile = tiles >= 1024 ? 4 : (tiles >= 512 ? 2 : 1);
-  if (ntile == 1 && MT >= 2 && tiles >= 32) ntile = 2;
-#define GO(NT, WV) gemm_skinny_kernel<MT, NT, WV, EPI, TO, NORM><<<dim3((tiles + NT - 1) / NT), dim3(WV * MS_WAVE), 0, stream>>>(A, lda, W, ldw, bias, out, ldo, M, N, K, norm_w, eps, rows)
-  if (ntile == 4) GO(4, 4);
-  else if (ntile == 2) GO(2, 8);
-  else if (steps >= 32 || MT > 1) GO(1, 16);
-  else GO(1, 8);
+  // (measured on the 0.5B shapes at 8 and 64 rows; with several token groups the wide shape pays earlier)
+  int ntile = tiles >= 1024 ? 4 : (tiles >= 512 ? (MT >= 4 ? 4 : 2) : 1);
+  int waves = ntile == 4 ? (MT == 1 ? 8 : 4) : (ntile == 2 ? 8 : ((steps >= 32 || MT > 1) ? 16 : 8));
+  if (g_force_ntile) { ntile = g_force_ntile; waves = g_force_waves; }
+  if ((waves - 1) * ntile * MT > 60) return MS_UNSUPPORTED;  // LDS
+#define GO(NT, WV) if (ntile == NT && waves == WV) { if constexpr ((WV - 1) * NT * MT <= 60) { gemm_skinny_kernel<MT, NT, WV, EPI, TO, NORM><<<dim3((tiles + NT - 1) / NT), dim3(WV * MS_WAVE), 0, stream>>>(A, lda, W, ldw, bias, out, ldo, M, N, K, norm_w, eps, rows); return ms_launch_status(); } }
+  GO(4, 4) GO(4, 8) GO(2, 8) GO(2, 16) GO(1, 8) GO(1, 16)
 #undef GO
-  return ms_launch_status();
+  return MS_UNSUPPORTED;
 }
 
 template <int EPI, typename TO, bool NORM>
@@ -207,6 +212,13 @@ int launch_mt(const void* A, size_t lda, const bf16* W, size_t ldw, const float*
 }
 
 }  // namespace
+
+// Tuning knob for measurements: force the block shape (tiles per block, waves) out of (4,4) (4,8) (2,8) (2,16)
+// (1,8) (1,16) for every later ms_gemm_skinny* launch; (0, 0) gives the choice back to the heuristic.
+extern "C" void ms_gemm_skinny_force(int ntile, int waves) {
+  g_force_ntile = ntile;
+  g_force_waves = waves;
+}
 
 // epilogue 0: out[M,N] (out_dtype float or bfloat16) = product + bias
 // epilogue 1: out[M,N/2] bfloat16 = silu(gate) * up over interleaved rows of W (no bias)

@@ -304,6 +304,35 @@ def test_gemm_skinny(ops, M, N, K):
     assert torch.equal(ops.gemm_skinny(a[M - 1:], w, bias), out[M - 1:])
 
 
+@pytest.mark.parametrize("M", [3, 40])
+@pytest.mark.parametrize("shape", [(4, 4), (4, 8), (2, 8), (2, 16), (1, 8), (1, 16)])
+def test_gemm_skinny_block_shapes(ops, M, shape):
+    """Every block shape on offer gives the same numbers (to float rounding of another summation order)."""
+    from llm_infrence_engine_amd.kernels import build
+
+    lib = build.load()
+    g = torch.Generator().manual_seed(sum(shape) + M)
+    N, K = 1000, 1544
+    a = torch.randn(M, K, generator=g).bfloat16().to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16().to(DEV)
+    bias = torch.randn(N, generator=g).to(DEV)
+    want = a.double() @ w.double().T + bias.double()
+    x0 = torch.randn(M, N, generator=g).to(DEV)
+    try:
+        lib.ms_gemm_skinny_force(*shape)
+        x = x0.clone()
+        try:
+            ops.gemm_skinny(a, w, bias, ops.EPI_RESIDUAL, residual=x)
+        except RuntimeError as e:      # a shape that does not fit LDS with this many token groups is refused
+            assert "unsupported" in str(e) and (shape[1] - 1) * shape[0] * (1 if M <= 16 else 4) > 60
+            return
+        torch.testing.assert_close(x.double(), x0.double() + want, atol=3e-5, rtol=3e-5)
+        f = ops.gemm_skinny(a, w, bias, out_dtype=torch.float32)
+        torch.testing.assert_close(f.double(), want, atol=3e-5, rtol=3e-5)
+    finally:
+        lib.ms_gemm_skinny_force(0, 0)
+
+
 def test_gemm_skinny_refuses_what_it_cannot_take(ops):
     a = torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV)
     w = torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV)
