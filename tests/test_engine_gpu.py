@@ -218,3 +218,30 @@ def test_generation_with_hip_graphs(tiny, eng):
     got = llm.generate(prompts, eng.SamplingParams(max_new_tokens=10))
     assert [o.token_ids for o in got] == want
     assert llm.engine.runner.graphs.buckets
+
+
+def test_long_context_decode_splits_keys_and_matches_plain(eng, tmp_path):
+    """Past 2,048 keys a small decode batch spreads each request's keys over several blocks (and, with graphs,
+    switches to the long-context graphs): logits still follow the plain implementation."""
+    from llm_infrence_engine_amd.config import config_from_dict
+    from llm_infrence_engine_amd.engine import StepEntry, load_runner
+    from llm_infrence_engine_amd.kernels import ops
+
+    d = tmp_path / "m"
+    eng.write_random_model(d, config_from_dict(TINY["D"]), seed=5, dtype="bfloat16", std=0.08)
+    cfg, w = P.read_config(d), P.read_weights(d, torch.float64)
+    rng = np.random.default_rng(4)
+    n = ops.LONG_CONTEXT + 40
+    seqs = {r: [int(t) for t in rng.integers(0, cfg["vocab_size"], m)] for r, m in (("a", n), ("b", 300))}
+    exact = {r: P.forward(w, cfg, t).numpy() for r, t in seqs.items()}
+    noise = {r: np.abs(P.forward(w, cfg, t, act_dtype=torch.bfloat16).numpy() - exact[r]).max() for r, t in seqs.items()}
+    for graphs in (False, True):
+        r = load_runner(d, dtype="bfloat16", page_size=16, num_pages=160, max_requests=2, max_len=n + 16, hip_graphs=graphs)
+        cut = {"a": n - 60, "b": 240}
+        r.step([StepEntry("a", seqs["a"][:cut["a"]], []), StepEntry("b", seqs["b"][:cut["b"]], [])])
+        for i in range(60):
+            lg = r.step([StepEntry(q, [seqs[q][cut[q] + i]], [0]) for q in ("a", "b")]).cpu().numpy()
+            for row, q in zip(lg, ("a", "b")):
+                assert np.abs(row - exact[q][cut[q] + i]).max() < 3.0 * noise[q], (graphs, q, i)
+        if graphs:
+            assert sorted(r.graphs.buckets) == [(2, False), (2, True)]   # it crossed from short to long on the way
