@@ -57,20 +57,20 @@ def prefill_flops(cfg, tokens):
     return linear + attention
 
 
-def run_decode(eng_mod, model, batch, steps, warmup, vocab, seed):
+def run_decode(eng_mod, model, batch, steps, warmup, vocab, seed, prompt_len=PROMPT_LEN):
     """Prefill ``batch`` prompts, then time ``steps`` decode steps of the engine.  Returns seconds per step."""
     import numpy as np
     import torch
 
     rng = np.random.default_rng(seed)
     budget = max(4096, batch)
-    extra = -(-batch * PROMPT_LEN // budget) + 2     # requests admitted first decode while the others prefill
-    need = PROMPT_LEN + warmup + steps + extra
+    extra = -(-batch * prompt_len // budget) + 2     # requests admitted first decode while the others prefill
+    need = prompt_len + warmup + steps + extra
     pages = batch * (-(-need // BLOCK_SIZE) + 1)
     e = eng_mod.Engine(model, num_blocks=pages, block_size=BLOCK_SIZE, max_seqs=batch, max_len=CONTEXT_LIMIT,
                        max_num_batched_tokens=budget, hip_graphs=True)
     for _ in range(batch):
-        e.add_request(eng_mod.Request([int(t) for t in rng.integers(0, vocab, PROMPT_LEN)],
+        e.add_request(eng_mod.Request([int(t) for t in rng.integers(0, vocab, prompt_len)],
                                       max_new_tokens=warmup + steps + extra))
     while any(r.num_tokens - r.num_computed > 1 for r in e.running) or e.waiting:
         e.step()                                   # prompts in portions under the budget; first tokens sampled
@@ -84,7 +84,7 @@ def run_decode(eng_mod, model, batch, steps, warmup, vocab, seed):
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / steps
     assert all(rec.decode_batch == batch and rec.n_prefill_tokens == 0 for rec in e.steps[-steps:])
-    mean_context = PROMPT_LEN + warmup + (steps + 1) / 2
+    mean_context = prompt_len + warmup + (steps + 1) / 2
     return dt, mean_context
 
 
@@ -119,6 +119,7 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=MODEL["num_hidden_layers"],
                     help="fewer layers than the configuration has, if memory or time needs it (both numbers are reported)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points and the prefill")
+    ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN, help="prompt length of the decode run (default 512)")
     ap.add_argument("--only", choices=["prefill"], help="run one part alone (for profiles): the 2,048-token prefill")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -143,7 +144,7 @@ def main() -> int:
                                       "ms": round(pt * 1e3, 3)}}), flush=True)
         return 0
 
-    dt, ctx = run_decode(eng, model, a.batch, a.steps, a.warmup, vocab, seed=1)
+    dt, ctx = run_decode(eng, model, a.batch, a.steps, a.warmup, vocab, seed=1, prompt_len=a.prompt_len)
     value = a.batch / dt
     gbs = decode_bytes(cfg, a.batch, ctx) / dt / 1e9
     out = {
@@ -154,7 +155,7 @@ def main() -> int:
             "model": "Qwen2.5-0.5B shape, random weights", "layers": a.layers, "layers_of_config": MODEL["num_hidden_layers"],
             "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
             "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": vocab, "tied": True,
-            "global_batch": a.batch, "prompt_len": PROMPT_LEN, "seq_len": CONTEXT_LIMIT, "block_size": BLOCK_SIZE,
+            "global_batch": a.batch, "prompt_len": a.prompt_len, "seq_len": CONTEXT_LIMIT, "block_size": BLOCK_SIZE,
             "prefill_tokens": PREFILL_TOKENS, "parallelism": "single_gpu",
             "baseline": "reference CUDA-graph decode, batch 8, ctx 128, A10 bf16: 6.0 ms/step",
         },

@@ -375,7 +375,7 @@ def attention_mfma_supported(head_dim: int, page_size: int) -> bool:
 DECODE_WAVES = 1024       # waves a decode step's attention aims to put on the chip
 MAX_SPLITS = 32
 MIN_BLOCKS_PER_SPLIT = 8   # of 32 keys
-LONG_CONTEXT = 2048        # beyond this a small decode batch also splits its keys over blocks
+LONG_CONTEXT = 1024        # beyond this a small decode batch also splits its keys over blocks
 SPLIT_BELOW = 128          # ... when it has fewer (request, kv head) pairs than this
 
 
