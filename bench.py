@@ -35,6 +35,7 @@ PROMPT_LEN = 512
 CONTEXT_LIMIT = 8192
 BLOCK_SIZE = 16
 PREFILL_TOKENS = 2048
+DECODE_STEPS_PER_LAUNCH = 8   # decode steps queued in one graph launch (a stop id is noticed that many steps late at most)
 # the reference's own decode at batch 8: CUDA-graph step of 6.0 ms on an A10, context 128 (docs/RESULTS.md:38)
 BASELINE_TOKS = 8 / 6.0e-3
 
@@ -68,22 +69,25 @@ def run_decode(eng_mod, model, batch, steps, warmup, vocab, seed, prompt_len=PRO
     need = prompt_len + warmup + steps + extra
     pages = batch * (-(-need // BLOCK_SIZE) + 1)
     e = eng_mod.Engine(model, num_blocks=pages, block_size=BLOCK_SIZE, max_seqs=batch, max_len=CONTEXT_LIMIT,
-                       max_num_batched_tokens=budget, hip_graphs=True)
+                       max_num_batched_tokens=budget, hip_graphs=True, decode_steps_per_launch=DECODE_STEPS_PER_LAUNCH)
     for _ in range(batch):
         e.add_request(eng_mod.Request([int(t) for t in rng.integers(0, vocab, prompt_len)],
                                       max_new_tokens=warmup + steps + extra))
     while any(r.num_tokens - r.num_computed > 1 for r in e.running) or e.waiting:
         e.step()                                   # prompts in portions under the budget; first tokens sampled
-    for _ in range(warmup):
-        e.step()
+    def run(n):   # exactly n decode steps, several to a graph launch
+        done, first = 0, len(e.steps)
+        while done < n:
+            done += e.step(max_decode_steps=n - done).decode_steps
+        assert done == n and all(rec.decode_batch == batch and rec.n_prefill_tokens == 0 for rec in e.steps[first:])
+
+    run(warmup)
     assert len(e.running) == batch and all(r.num_tokens - r.num_computed == 1 for r in e.running)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(steps):
-        e.step()
+    run(steps)
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / steps
-    assert all(rec.decode_batch == batch and rec.n_prefill_tokens == 0 for rec in e.steps[-steps:])
     mean_context = prompt_len + warmup + (steps + 1) / 2
     return dt, mean_context
 

@@ -14,6 +14,11 @@ int ms_rms_norm(float* x, const void* delta, int delta_dtype, int n_partials, lo
 
 int ms_bias_add(void* x, const float* bias, int n_rows, int width, int dtype, hipStream_t stream);
 
+// tables / slots: host arrays of n_groups device pointers (block table int32 [rows, table_stride], slot mapping int32 [rows])
+int ms_decode_advance(const int* prev_tokens, int* token_ids, int* positions, int* context_lens, const int* n_live,
+                      const int* const* tables, int* const* slots, int n_groups, int table_stride, int page_size,
+                      int n_rows, hipStream_t stream);
+
 int ms_residual_add(float* x, const void* delta, long long total, int dtype, hipStream_t stream);
 
 int ms_silu_mul(const void* gate_up, void* out, int n_tokens, int intermediate, int dtype, hipStream_t stream);

@@ -13,6 +13,7 @@ from typing import Callable, List, Optional, Sequence
 
 import torch
 
+from ..cache.allocator import OutOfPages
 from ..config.engine_config import EngineConfig
 from ..parts.model import Model
 from ..sampling import Sampler
@@ -27,7 +28,12 @@ class Engine:
                  max_len: int = 1024, max_num_batched_tokens: int = 2048, max_prefill_chunk: Optional[int] = None,
                  on_token: Optional[Callable[[Request, int], None]] = None,
                  on_finish: Optional[Callable[[Request], None]] = None,
-                 clock: Callable[[], float] = time.perf_counter, hip_graphs: bool = False):
+                 clock: Callable[[], float] = time.perf_counter, hip_graphs: bool = False,
+                 decode_steps_per_launch: int = 1):
+        """``decode_steps_per_launch`` > 1 (with ``hip_graphs``): while every running request is decoding
+        greedily and nobody waits, up to that many decode steps run in one graph launch, each fed the argmax of
+        the one before on the device; a stop id is then noticed up to that many steps late (the surplus tokens
+        are dropped), so outputs do not change."""
         dtype = {torch.float32: "float32", torch.bfloat16: "bfloat16"}[model.rt.dtype]
         self.config = EngineConfig(dtype=dtype, block_size=block_size, num_blocks=num_blocks, max_seqs=max_seqs,
                                    max_len=max_len, max_num_batched_tokens=max_num_batched_tokens,
@@ -39,6 +45,7 @@ class Engine:
         self.scheduler = Scheduler(self.runner.manager, self.config, clock, on_token, on_finish)
         self.sampler = Sampler(model.rt.device)
         self.clock = clock
+        self.decode_steps_per_launch = max(1, decode_steps_per_launch) if self.runner.graphs is not None else 1
         self.steps: List[StepRecord] = []
         self.peak_running = 0
         self.peak_pages_in_use = 0
@@ -74,13 +81,46 @@ class Engine:
     def preemptions(self) -> int:
         return self.scheduler.preemptions
 
-    def step(self) -> StepRecord:
+    def _steps_ahead(self, sched, limit: int) -> int:
+        """How many decode steps the next launch may hold: a power of two within the configured limit and
+        within what every request still has to generate, if all of them decode greedily and nobody waits."""
+        limit = min(limit, self.decode_steps_per_launch)
+        if limit < 2 or self.scheduler.waiting or len(sched) > self.runner.graphs.max_batch:
+            return 1
+        for s in sched:
+            r = s.request
+            if s.count != 1 or s.start == 0 or not s.sample or r.temperature > 0.0:
+                return 1
+            limit = min(limit, r.max_new_tokens - len(r.output_ids), self.config.max_len - r.num_computed)
+        k = 1
+        while k * 2 <= limit:
+            k *= 2
+        if k > 1:
+            m = self.runner.manager
+            try:
+                for s in sched:
+                    m.grow(s.request.id, s.start + k)
+            except OutOfPages:
+                return 1           # what was grown stays with its request: it will need it soon anyway
+        return k
+
+    def step(self, max_decode_steps: int = 1 << 30) -> StepRecord:
         t0 = self.clock()
         sched = self.scheduler.schedule()
         useful = 0
         if not sched and self.scheduler.has_work():
             raise RuntimeError("the scheduler could place no request although work is waiting")
-        if sched:
+        ahead = self._steps_ahead(sched, max_decode_steps) if sched and self.decode_steps_per_launch > 1 else 1
+        if ahead > 1:
+            entries = [StepEntry(s.request.id, [s.request.output_ids[-1]]) for s in sched]
+            tokens = self.runner.decode_steps(entries, ahead)
+            for k in range(ahead):      # as the single steps would have: a finished request drops its later tokens
+                for i, s in enumerate(sched):
+                    if s.request.state == "running":
+                        s.request.num_computed += 1
+                        self.scheduler._emit(s.request, tokens[k][i])
+                        useful += 1
+        elif sched:
             entries, rows = [], []
             for s in sched:
                 toks = s.request.tokens[s.start:s.start + s.count]
@@ -96,12 +136,13 @@ class Engine:
             useful = self.scheduler.commit(sched, sampled)
         n_decode = sum(1 for s in sched if s.count == 1 and s.start > 0)
         n_prefill = sum(s.count for s in sched) - n_decode
+        decode_steps = ahead if n_decode else 0
         self.prefill_tokens_computed += n_prefill
         self.peak_running = max(self.peak_running, len(self.scheduler.running))
         in_use = max((g.allocator.num_in_use() for g in self.runner.manager.groups), default=0)
         self.peak_pages_in_use = max(self.peak_pages_in_use, in_use)
         rec = StepRecord(n_prefill, n_decode, useful, self.clock() - t0, self.scheduler.last_preempted,
-                         self.scheduler.last_admitted)
+                         self.scheduler.last_admitted, decode_steps)
         self.steps.append(rec)
         return rec
 

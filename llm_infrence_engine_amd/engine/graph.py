@@ -9,6 +9,10 @@ full width, the attention kernel spreads each request's keys over its waves itse
 for the life of the engine; only the choice between the attention's two launch shapes (contexts up to
 ``ops.LONG_CONTEXT`` or beyond) is made per step, and each has graphs of its own.  Rows that pad a batch up to its bucket read the null page and store nothing.
 The greedy choice (argmax) of every row is part of the graph.
+
+A graph may also hold several decode steps in a row: between two steps a small kernel moves every live
+request one position on, feeds it the token just chosen and looks up its new slots in the block tables, all
+on the device, so the host is needed once per launch instead of once per step.
 """
 from __future__ import annotations
 
@@ -34,13 +38,13 @@ def default_batch_sizes(max_batch: int) -> List[int]:
 
 
 class _Bucket:
-    def __init__(self, B: int, width: int, n_groups: int, device):
-        self.B, self.width = B, width
+    def __init__(self, B: int, width: int, n_groups: int, device, steps: int = 1):
+        self.B, self.width, self.steps = B, width, steps
         # layout of the static int32 buffer
         self.off: Dict[str, slice] = {}
         o = 0
         for name, n in (("token_ids", B), ("positions", B), ("token_req", B), ("q_start", B + 1),
-                        ("context_lens", B), ("state_slots", B), ("logit_rows", B)):
+                        ("context_lens", B), ("state_slots", B), ("logit_rows", B), ("n_live", 1)):
             self.off[name] = slice(o, o + n)
             o += n
         self.tables, self.slots = [], []
@@ -56,7 +60,7 @@ class _Bucket:
         self.last_rows = 0
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.logits: Optional[torch.Tensor] = None
-        self.tokens: Optional[torch.Tensor] = None
+        self.tokens = torch.zeros((steps, B), dtype=torch.int32, device=device)   # the argmax of every step
 
     def reset_host(self) -> None:
         """Every row a padding row: token 0 at position 0, one visible key on the null page, nothing stored."""
@@ -66,6 +70,7 @@ class _Bucket:
         a[self.off["q_start"]] = np.arange(B + 1)
         a[self.off["context_lens"]] = 1
         a[self.off["logit_rows"]] = np.arange(B)
+        a[self.off["n_live"]] = 0
         for s in self.slots:
             a[s] = -1
 
@@ -93,12 +98,12 @@ class DecodeGraphs:
     def max_batch(self) -> int:
         return self.sizes[-1]
 
-    def _bucket(self, n: int, long_context: bool) -> _Bucket:
+    def _bucket(self, n: int, long_context: bool, steps: int = 1) -> _Bucket:
         B = next(b for b in self.sizes if b >= n)
-        key = (B, long_context)
+        key = (B, long_context) if steps == 1 else (B, long_context, steps)
         bk = self.buckets.get(key)
         if bk is None:
-            bk = self.buckets[key] = _Bucket(B, self.width, len(self.manager.groups), self.runner.rt.device)
+            bk = self.buckets[key] = _Bucket(B, self.width, len(self.manager.groups), self.runner.rt.device, steps)
             self._capture(bk, long_context)
         return bk
 
@@ -118,34 +123,47 @@ class DecodeGraphs:
         cap = self.width * self.manager.page_size
         ctx.max_context_len = cap if long_context else min(cap, ops.LONG_CONTEXT)
         model = self.runner.model
+        d, o = bk.dev, bk.off
+        tables = [d[s].view(bk.B, bk.width) for s in bk.tables]
+        slots = [d[s] for s in bk.slots]
+
+        def advance(k):   # n_live is 0 in the buffer while capturing and warming up: nothing moves
+            ops.decode_advance(bk.tokens[k - 1], d[o["token_ids"]], d[o["positions"]], d[o["context_lens"]],
+                               d[o["n_live"]], tables, slots, self.manager.page_size)
+
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
             for _ in range(2):            # load kernels and settle allocations before capturing
-                model.forward(ctx, caches)
+                ops.sample(model.forward(ctx, caches), bk.tokens[0])
+            if bk.steps > 1:
+                advance(1)
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         bk.graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(bk.graph):
-            bk.logits = model.forward(ctx, caches)
-            bk.tokens = torch.empty(bk.B, dtype=torch.int32, device=bk.logits.device)
-            ops.sample(bk.logits, bk.tokens)
+            for k in range(bk.steps):
+                if k > 0:
+                    advance(k)
+                bk.logits = model.forward(ctx, caches)
+                ops.sample(bk.logits, bk.tokens[k])
         torch.cuda.synchronize()
 
-    def run(self, entries: List[StepEntry]):
-        """One decode step for ``entries`` (one token each, pages already grown).  Returns (logits [R, V],
-        greedy tokens int32 [R]); both are views of static buffers that the next replay overwrites."""
+    def run(self, entries: List[StepEntry], steps: int = 1):
+        """``steps`` decode steps for ``entries`` (one token each, pages already grown for all the steps).
+        Returns (logits [R, V] of the last step, greedy tokens int32 [steps, R]); both are views of static
+        buffers that the next replay overwrites."""
         m = self.manager
         R = len(entries)
         rows = np.fromiter((m.row(e.req_id) for e in entries), dtype=np.int32, count=R)
         pos = np.fromiter((m.computed(e.req_id) for e in entries), dtype=np.int32, count=R)
-        bk = self._bucket(R, int(pos.max()) + 1 > ops.LONG_CONTEXT)
+        bk = self._bucket(R, int(pos.max()) + steps > ops.LONG_CONTEXT, steps)
         a, o, ps = bk.np, bk.off, m.page_size
         toks = np.fromiter((e.tokens[0] for e in entries), dtype=np.int64, count=R)
         if toks.min() < 0 or toks.max() >= self.runner.model.spec.vocab_size:
             raise ValueError("a token id is outside the vocabulary")
-        if int(pos.max()) + 1 > m.max_len:
-            raise ValueError(f"a request would hold {int(pos.max()) + 1} tokens; the cache is made for {m.max_len}")
+        if int(pos.max()) + steps > m.max_len:
+            raise ValueError(f"a request would hold {int(pos.max()) + steps} tokens; the cache is made for {m.max_len}")
         if R < bk.last_rows:
             bk.reset_host()
         bk.last_rows = R
@@ -153,14 +171,15 @@ class DecodeGraphs:
         a[o["positions"]][:R] = pos
         a[o["context_lens"]][:R] = pos + 1
         a[o["state_slots"]][:R] = rows
-        used = int(pos.max()) // ps + 1
+        a[o["n_live"]] = R
+        used = (int(pos.max()) + steps - 1) // ps + 1
         for g, grp in enumerate(m.groups):
             t = a[bk.tables[g]].reshape(bk.B, bk.width)
             t[:R, :used] = grp.tables[rows, :used]
             page = t[np.arange(R), pos // ps]
-            if (page == 0).any():
-                raise RuntimeError("a token of this step has no page; grow the request before the step")
+            if (page == 0).any() or (t[np.arange(R), (pos + steps - 1) // ps] == 0).any():
+                raise RuntimeError("a token of this launch has no page; grow the requests before it")
             a[bk.slots[g]][:R] = page * ps + pos % ps
         bk.dev.copy_(bk.host, non_blocking=True)
         bk.graph.replay()
-        return bk.logits[:R], bk.tokens[:R]
+        return bk.logits[:R], bk.tokens[:, :R]

@@ -78,6 +78,7 @@ class StepRecord:
     duration: float
     n_preempted: int = 0
     n_admitted: int = 0
+    decode_steps: int = 0   # decode steps this record covers (several when one launch ran several steps)
 
 
 @dataclass

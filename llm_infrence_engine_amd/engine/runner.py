@@ -58,7 +58,8 @@ class ModelRunner:
         self.greedy_tokens = None
         if (self.graphs is not None and len(entries) <= self.graphs.max_batch
                 and all(len(e.tokens) == 1 and len(e.want) == 1 for e in entries)):
-            logits, self.greedy_tokens = self.graphs.run(entries)
+            logits, tokens = self.graphs.run(entries)
+            self.greedy_tokens = tokens[0]
             for e in entries:
                 m.advance(e.req_id, m.computed(e.req_id) + 1)
             return logits
@@ -75,6 +76,26 @@ class ModelRunner:
         for e in entries:
             m.advance(e.req_id, m.computed(e.req_id) + len(e.tokens))
         return logits
+
+
+    @torch.inference_mode()
+    def decode_steps(self, entries: List[StepEntry], steps: int) -> List[List[int]]:
+        """``steps`` greedy decode steps in one launch of a captured graph: every request of ``entries`` (one
+        token each, the one it is to be fed next) runs ``steps`` tokens ahead, each step fed the argmax of the
+        one before on the device.  Returns the chosen tokens, [steps][len(entries)]."""
+        if self.graphs is None:
+            raise RuntimeError("several decode steps per launch need hip_graphs")
+        m = self.manager
+        for e in entries:
+            if len(e.tokens) != 1:
+                raise ValueError("decode_steps takes one token per request")
+            m.grow(e.req_id, m.computed(e.req_id) + steps)
+        _, tokens = self.graphs.run(entries, steps)
+        out = tokens.tolist()
+        for e in entries:
+            m.advance(e.req_id, m.computed(e.req_id) + steps)
+        self.greedy_tokens = None
+        return out
 
 
 def load_runner(model_dir, dtype: str = "bfloat16", device: str = "cuda:0", page_size: int = 16,

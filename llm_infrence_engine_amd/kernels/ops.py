@@ -26,6 +26,7 @@ _SIGNATURES = {
                             _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "ms_qkv_rope_store": [_c_ptr, _c_ll, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                           _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "ms_decode_advance": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "ms_bias_add": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "ms_gemm_skinny": [_c_ptr, _c_ll, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int,
                        _c_ptr],
@@ -146,6 +147,31 @@ def bias_add(x: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
     _check(bias, "bias", torch.float32, (x.shape[-1],))
     _call("ms_bias_add", x.data_ptr(), bias.data_ptr(), x.numel() // x.shape[-1], x.shape[-1], _code(x.dtype), _stream())
     return x
+
+
+MAX_GROUPS = 4
+
+
+def decode_advance(prev_tokens: torch.Tensor, token_ids: torch.Tensor, positions: torch.Tensor,
+                   context_lens: torch.Tensor, n_live: torch.Tensor, tables, slots, page_size: int) -> None:
+    """Between two decode steps queued back to back: rows below ``n_live[0]`` move one position on, take
+    ``prev_tokens`` as their input and get their new slots from ``tables`` (one [rows, width] per cache group)."""
+    R = token_ids.numel()
+    for t, name in ((prev_tokens, "prev_tokens"), (token_ids, "token_ids"), (positions, "positions"),
+                    (context_lens, "context_lens")):
+        _check(t, name, torch.int32, (R,))
+    _check(n_live, "n_live", torch.int32, (1,))
+    if len(tables) != len(slots) or len(tables) > MAX_GROUPS:
+        raise ValueError(f"at most {MAX_GROUPS} cache groups, one table and one slot mapping each")
+    width = tables[0].shape[1] if tables else 1
+    for t, sl in zip(tables, slots):
+        _check(t, "table", torch.int32, (R, width))
+        _check(sl, "slots", torch.int32, (R,))
+    tp = (ctypes.c_void_p * max(1, len(tables)))(*[t.data_ptr() for t in tables])
+    sp = (ctypes.c_void_p * max(1, len(slots)))(*[t.data_ptr() for t in slots])
+    _call("ms_decode_advance", prev_tokens.data_ptr(), token_ids.data_ptr(), positions.data_ptr(),
+          context_lens.data_ptr(), n_live.data_ptr(), ctypes.cast(tp, ctypes.c_void_p), ctypes.cast(sp, ctypes.c_void_p),
+          len(tables), width, page_size, R, _stream())
 
 
 def residual_add(x: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:

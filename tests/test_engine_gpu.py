@@ -245,3 +245,29 @@ def test_long_context_decode_splits_keys_and_matches_plain(eng, tmp_path):
                 assert np.abs(row - exact[q][cut[q] + i]).max() < 3.0 * noise[q], (graphs, q, i)
         if graphs:
             assert sorted(r.graphs.buckets) == [(2, False), (2, True)]   # it crossed from short to long on the way
+
+
+def test_several_decode_steps_per_launch_change_nothing(tiny, eng):
+    """Up to 8 decode steps queued in one graph launch (tokens fed back on the device): the same outputs as step
+    by step, also when a stop id arrives in the middle of a launch, a request joins, or pages are scarce."""
+    name, d, cfg, w = tiny
+    rng = np.random.default_rng(31)
+    prompts = [[int(t) for t in rng.integers(0, cfg["vocab_size"], n)] for n in (9, 21, 5, 14)]
+    full = [P.greedy_generate(w, cfg, p, 30) for p in prompts]
+    stops = [(), (full[1][11],), (), (full[3][4],)]
+    want = [P.greedy_generate(w, cfg, p, 30, eos_ids=s) for p, s in zip(prompts, stops)]
+    model = eng.load_model(d, "float32")
+    for kw in (dict(num_blocks=None), dict(num_blocks=9)):            # plenty of pages; so few that launches shrink
+        e = eng.Engine(model, block_size=16, max_seqs=4, max_len=64, hip_graphs=True, decode_steps_per_launch=8, **kw)
+        reqs = [e.add_request(eng.Request(p, max_new_tokens=30, eos_ids=s)) for p, s in zip(prompts[:3], stops[:3])]
+        for _ in range(3):
+            e.step()
+        reqs.append(e.add_request(eng.Request(prompts[3], max_new_tokens=30, eos_ids=stops[3])))   # joins on the way
+        while e.has_work():
+            e.step()
+            e.runner.manager.check_invariants()
+        assert [r.output_ids for r in reqs] == want
+        assert [r.finish_reason for r in reqs] == ["length", "stop", "length", "stop"]
+        assert any(rec.decode_steps > 1 for rec in e.steps)
+        assert sum(rec.decode_steps for rec in e.steps) < len(e.steps) * 8
+        assert all(g.allocator.num_in_use() == 0 for g in e.runner.manager.groups)

@@ -409,7 +409,7 @@ def test_paged_attention_mfma(ops, nh, nkv, d, page_size, window, shape):
     if shape == "mixed":
         ctx, qlen = [70, 133, 201, 300], [70, 9, 1, 150]
     elif shape == "decode":
-        ctx, qlen = [1, 31, 32, 33, 600, 1500, 64, 17], [1] * 8
+        ctx, qlen = [1, 31, 32, 33, 600, 1000, 64, 17], [1] * 8
     else:   # few requests with long contexts: keys split over blocks and combined
         ctx, qlen = [2500, 1, 300], [1] * 3
     c = _paged_case(g, torch.bfloat16, nh, nkv, d, page_size, ctx, qlen, float("nan"))
