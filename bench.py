@@ -25,7 +25,7 @@ if ROOT not in sys.path:
 HBM_GBS = 8000.0
 PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "fp8": 5000.0, "fp32": 157.3}
 
-# Qwen2.5-0.5B's config.json sizes (BASELINE.json configs[2])
+# Qwen2.5-0.5B's config.json sizes
 MODEL = {
     "architectures": ["Qwen2ForCausalLM"], "num_hidden_layers": 24, "hidden_size": 896, "num_attention_heads": 14,
     "num_key_value_heads": 2, "intermediate_size": 4864, "vocab_size": 151936, "rope_theta": 1000000.0,
@@ -37,7 +37,7 @@ BLOCK_SIZE = 16
 PREFILL_TOKENS = 2048
 DECODE_STEPS_PER_LAUNCH = 8   # decode steps queued in one graph launch (a stop id is noticed that many steps late at most)
 # the reference's own decode at batch 8: CUDA-graph step of 6.0 ms on an A10, context 128 (docs/RESULTS.md:38)
-BASELINE_TOKS = 8 / 6.0e-3
+REFERENCE_TOKS = 8 / 6.0e-3
 
 
 def decode_bytes(cfg, batch, context, bytes_per_value=2):
@@ -154,13 +154,14 @@ def main() -> int:
     out = {
         "metric": "decode_tokens_per_s", "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1,
         "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": round(value / BASELINE_TOKS, 2), "dtype": "bf16", "data": "synthetic",
+        "scaling": "weak", "vs_baseline": round(value / REFERENCE_TOKS, 2), "dtype": "bf16", "data": "synthetic",
         "config": {
             "model": "Qwen2.5-0.5B shape, random weights", "layers": a.layers, "layers_of_config": MODEL["num_hidden_layers"],
             "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
             "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": vocab, "tied": True,
             "global_batch": a.batch, "prompt_len": a.prompt_len, "seq_len": CONTEXT_LIMIT, "block_size": BLOCK_SIZE,
             "prefill_tokens": PREFILL_TOKENS, "parallelism": "single_gpu",
+            "decode_steps_per_launch": DECODE_STEPS_PER_LAUNCH,
             "baseline": "reference CUDA-graph decode, batch 8, ctx 128, A10 bf16: 6.0 ms/step",
         },
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_GBS, "unit": "GB/s",

@@ -371,3 +371,52 @@ def test_toy_architecture_is_registered_built_and_stepped(fw, tmp_path):
     assert len(held[full]) == 6 and len(held[1 - full]) < 6
     runner.free_request("b"); runner.free_request("c")
     assert all(g.allocator.num_in_use() == 0 for g in runner.manager.groups)
+
+
+def test_rotary_part_and_block_alone(fw):
+    """The rotary part against the plain rotation (a partial rotary dimension too), and the pre-norm residual
+    arrangement against the plain layer, fed in two portions."""
+    rt = rt_for(fw, torch.float32)
+    d, nh, nkv = 32, 3, 1
+    for rot in (32, 16):
+        part = fw.parts.build_part("position", fw.config.PartSpec("rotary_half", "", {"head_dim": d, "rotary_dim": rot, "theta": 777.0}))
+        part.load(None, rt)
+        qkv = torch.randn(6, (nh + 2 * nkv) * d)
+
+        class Ctx:
+            positions = torch.tensor([0, 1, 5, 40, 41, 1000], dtype=torch.int32, device=DEV)
+        dev = qkv.to(DEV)
+        part.encode_and_store(dev, nh, nkv, d, Ctx, None)
+        x = qkv.double().view(6, nh + 2 * nkv, d)
+        cos, sin = P.rope_cos_sin(Ctx.positions.cpu(), rot, 777.0)
+        want = x.clone()
+        want[:, :nh + nkv, :rot] = P.apply_rope(x[:, :nh + nkv, :rot].transpose(0, 1), cos, sin).transpose(0, 1)
+        torch.testing.assert_close(dev.double().cpu().view(6, nh + 2 * nkv, d), want, atol=2e-4, rtol=0)
+
+    cfg = {"num_heads": 4, "num_kv_heads": 2, "head_dim": 16, "rms_norm_eps": 1e-5}
+    H, I, T = 64, 96, 21
+    spec = fw.config.Qwen2Config(vocab_size=50, hidden_size=H, intermediate_size=I, num_hidden_layers=1, num_attention_heads=4,
+                                 num_key_value_heads=2, rms_norm_eps=1e-5, rope_theta=300.0).to_spec()
+    model = fw.parts.Model(spec)
+    block = model.layers[0]
+    t = fw.weights.random_tensors(block.tensor_specs(), 9, std=0.3, dtype="float32")
+    block.load(getter(t, fw, rt), rt)
+    x = torch.randn(T, H)
+    w = {k: v.double() for k, v in t.items()}
+    cos, sin = P.rope_cos_sin(torch.arange(T), 16, 300.0)
+    want = P.decoder_layer(x.double(), w, 0, cfg, cos, sin)
+    layout = fw.cache.CacheLayout(model.run_needs())
+    m = fw.cache.CacheManager(layout, 4, 20, 2, 32)
+    pools = fw.cache.CachePools(layout, 4, 20, 2, rt)
+    builder = fw.engine.BatchBuilder(m, 50, rt.device)
+    m.add("x")
+    got, p = [], 0
+    for n in (13, 8):
+        m.grow("x", p + n)
+        ctx, tables, slots = builder.build([fw.engine.StepEntry("x", [1] * n, [])])
+        xs = x[p:p + n].to(DEV).clone()
+        pending = block.forward(xs, None, ctx, pools.kv_view(0, tables[0], slots[0]), None)
+        got.append((xs if pending is None else xs + pending.float()).cpu())
+        p += n
+        m.advance("x", p)
+    torch.testing.assert_close(torch.cat(got).double(), want, atol=2e-4, rtol=2e-4)
