@@ -33,7 +33,7 @@ int ms_gemm_generic(const void* A, const void* W, const float* bias, void* C, in
 int ms_gemm_skinny(const void* A, long long lda, const void* W, long long ldw, const float* bias, void* out,
                    long long ldo, int M, int N, int K, int epilogue, int out_dtype, hipStream_t stream);
 
-void ms_gemm_skinny_force(int ntile, int waves);
+void ms_gemm_skinny_force(int ntile, int waves, int token_groups);
 
 int ms_gemm_skinny_norm(const float* x, long long ldx, const int* rows, const float* norm_w, float eps, const void* W,
                         long long ldw, const float* bias, void* out, long long ldo, int M, int N, int K, int epilogue,

@@ -39,6 +39,7 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
   const int lane = threadIdx.x & (MS_WAVE - 1), wave = threadIdx.x / MS_WAVE;
   const int col = lane & 15, kq = lane >> 4;
   const int n0 = blockIdx.x * 16 * NTILE;
+  const int m0 = blockIdx.y * 16 * MT;   // token groups beyond MT per block go to further blocks along y
   const int total_steps = (K + 31) / 32;
 
   const bf16* wrow[NTILE];
@@ -48,7 +49,7 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
   size_t arow[MT];  // element offset of this lane's activation row and k slice
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
-    const int m = min(t * 16 + col, M - 1);
+    const int m = min(m0 + t * 16 + col, M - 1);
     arow[t] = (size_t)(rows ? rows[m] : m) * lda + kq * 8;  // rows: the activations are gathered rows of A
   }
 
@@ -66,8 +67,8 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
       pre[u][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-      if (EPI == EPI_RESIDUAL && wave == (u * MT + t) % WAVES && t * 16 + col < M) {
-        const float* o = reinterpret_cast<const float*>(out) + (size_t)(t * 16 + col) * ldo + nb;
+      if (EPI == EPI_RESIDUAL && wave == (u * MT + t) % WAVES && m0 + t * 16 + col < M) {
+        const float* o = reinterpret_cast<const float*>(out) + (size_t)(m0 + t * 16 + col) * ldo + nb;
 #pragma unroll
         for (int r = 0; r < 4; ++r) if (nb + r < N) pre[u][t][r] = o[r];
       }
@@ -156,7 +157,7 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
         sum *= 1.0f / sqrtf(total / (float)K + eps);
       }
       // lane holds out[m = t*16 + col][n = nb + r], r = 0..3
-      const int m = t * 16 + col;
+      const int m = m0 + t * 16 + col;
       const int nb = n0 + u * 16 + kq * 4;
       if (m >= M) continue;
       if (EPI == EPI_SWIGLU) {
@@ -179,7 +180,7 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
 }
 
 // Tuning knob: force (tiles per block, waves) for every launch; 0 leaves the choice to the heuristic below.
-int g_force_ntile = 0, g_force_waves = 0;
+int g_force_ntile = 0, g_force_waves = 0, g_force_mt = 0;
 
 // The shapes of block on offer: (tiles per block, waves).  LDS holds (waves - 1) * tiles * MT KB.
 // (Splitting K over blocks as well, with the last block to arrive adding the partial sums, was measured and
@@ -196,7 +197,7 @@ int launch_cfg(const void* A, size_t lda, const bf16* W, size_t ldw, const float
   int waves = ntile == 4 ? (MT == 1 ? 8 : 4) : (ntile == 2 ? 8 : ((steps >= 32 || MT > 1) ? 16 : 8));
   if (g_force_ntile) { ntile = g_force_ntile; waves = g_force_waves; }
   if ((waves - 1) * ntile * MT > 60) return MS_UNSUPPORTED;  // LDS
-#define GO(NT, WV) if (ntile == NT && waves == WV) { if constexpr ((WV - 1) * NT * MT <= 60) { gemm_skinny_kernel<MT, NT, WV, EPI, TO, NORM><<<dim3((tiles + NT - 1) / NT), dim3(WV * MS_WAVE), 0, stream>>>(A, lda, W, ldw, bias, out, ldo, M, N, K, norm_w, eps, rows); return ms_launch_status(); } }
+#define GO(NT, WV) if (ntile == NT && waves == WV) { if constexpr ((WV - 1) * NT * MT <= 60) { gemm_skinny_kernel<MT, NT, WV, EPI, TO, NORM><<<dim3((tiles + NT - 1) / NT, (M + 16 * MT - 1) / (16 * MT)), dim3(WV * MS_WAVE), 0, stream>>>(A, lda, W, ldw, bias, out, ldo, M, N, K, norm_w, eps, rows); return ms_launch_status(); } }
   GO(4, 4) GO(4, 8) GO(2, 8) GO(2, 16) GO(1, 8) GO(1, 16)
 #undef GO
   return MS_UNSUPPORTED;
@@ -206,18 +207,24 @@ template <int EPI, typename TO, bool NORM>
 int launch_mt(const void* A, size_t lda, const bf16* W, size_t ldw, const float* bias, TO* out, size_t ldo, int M,
               int N, int K, hipStream_t stream, const float* norm_w = nullptr, float eps = 0.f,
               const int* rows = nullptr) {
-  if (M <= 16) return launch_cfg<1, EPI, TO, NORM>(A, lda, W, ldw, bias, out, ldo, M, N, K, stream, norm_w, eps, rows);
-  if (M <= 32) return launch_cfg<2, EPI, TO, NORM>(A, lda, W, ldw, bias, out, ldo, M, N, K, stream, norm_w, eps, rows);
+  // Several token groups per block share the weight loads; a narrow output has too few tiles to fill the chip
+  // that way, so there every group gets blocks of its own (the weight tile is then re-read from L2).
+  const int tiles = (N + 15) / 16;
+  const int mt = g_force_mt ? g_force_mt : ((M <= 16 || tiles <= 128) ? 1 : (M <= 32 ? 2 : 4));
+  if (mt == 1) return launch_cfg<1, EPI, TO, NORM>(A, lda, W, ldw, bias, out, ldo, M, N, K, stream, norm_w, eps, rows);
+  if (mt == 2) return launch_cfg<2, EPI, TO, NORM>(A, lda, W, ldw, bias, out, ldo, M, N, K, stream, norm_w, eps, rows);
   return launch_cfg<4, EPI, TO, NORM>(A, lda, W, ldw, bias, out, ldo, M, N, K, stream, norm_w, eps, rows);
 }
 
 }  // namespace
 
 // Tuning knob for measurements: force the block shape (tiles per block, waves) out of (4,4) (4,8) (2,8) (2,16)
-// (1,8) (1,16) for every later ms_gemm_skinny* launch; (0, 0) gives the choice back to the heuristic.
-extern "C" void ms_gemm_skinny_force(int ntile, int waves) {
+// (1,8) (1,16), and the 16-token groups per block (1, 2 or 4; further groups go to further blocks), for every
+// later ms_gemm_skinny* launch; zeros give the choice back to the heuristic.
+extern "C" void ms_gemm_skinny_force(int ntile, int waves, int token_groups) {
   g_force_ntile = ntile;
   g_force_waves = waves;
+  g_force_mt = token_groups;
 }
 
 // epilogue 0: out[M,N] (out_dtype float or bfloat16) = product + bias

@@ -45,6 +45,7 @@ qkv_rope_store_kernel(const float* __restrict__ X, size_t ldx, const float* __re
   const int lane = threadIdx.x & (MS_WAVE - 1), wave = threadIdx.x / MS_WAVE;
   const int col = lane & 15, kq = lane >> 4;
   const int pairs_per_head = d / 32;
+  const int m0 = blockIdx.y * 16 * MT;                    // token groups beyond MT per block: further blocks along y
   const int head = blockIdx.x / pairs_per_head;          // 0..nh-1: q, then nkv k heads, then nkv v heads
   const int j0 = (blockIdx.x % pairs_per_head) * 16;      // first feature of the low tile within the head
   const int half = d / 2;
@@ -54,7 +55,7 @@ qkv_rope_store_kernel(const float* __restrict__ X, size_t ldx, const float* __re
   const bf16* w_hi = w_lo + (size_t)half * K;
   size_t xrow[MT];
 #pragma unroll
-  for (int t = 0; t < MT; ++t) xrow[t] = (size_t)min(t * 16 + col, M - 1) * ldx + kq * 8;
+  for (int t = 0; t < MT; ++t) xrow[t] = (size_t)min(m0 + t * 16 + col, M - 1) * ldx + kq * 8;
 
   // what the epilogue will need from memory is asked for now, so that it arrives under the main loop
   const int jl = j0 + kq * 4;
@@ -68,7 +69,7 @@ qkv_rope_store_kernel(const float* __restrict__ X, size_t ldx, const float* __re
   int pos_m[MT], slot_m[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
-    const int m = min(t * 16 + col, M - 1);
+    const int m = min(m0 + t * 16 + col, M - 1);
     pos_m[t] = positions[m];
     slot_m[t] = slot_mapping[m];
   }
@@ -127,7 +128,7 @@ qkv_rope_store_kernel(const float* __restrict__ X, size_t ldx, const float* __re
   const int row_lo = head * d + j;
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
-    const int m = t * 16 + col;
+    const int m = m0 + t * 16 + col;
     const int owner = t % WAVES;
     if (wave != owner || m >= M) continue;
     float total = 0.f;
@@ -197,7 +198,7 @@ int launch(const float* X, size_t ldx, const float* norm_w, float eps, const bf1
   // LDS holds (waves - 1) * 2 * MT KB
   int waves = 4;
   while (waves < (MT == 1 ? 16 : 8) && blocks * waves < 1024 && steps >= waves * 2) waves *= 2;
-#define GO(WV) qkv_rope_store_kernel<MT, WV><<<dim3(blocks), dim3(WV * MS_WAVE), 0, stream>>>(X, ldx, norm_w, eps, W, bias, positions, inv_freq, slot_mapping, q_out, k_pages, v_pages, M, K, nh, nkv, d, page_size, v_transposed)
+#define GO(WV) qkv_rope_store_kernel<MT, WV><<<dim3(blocks, (M + 16 * MT - 1) / (16 * MT)), dim3(WV * MS_WAVE), 0, stream>>>(X, ldx, norm_w, eps, W, bias, positions, inv_freq, slot_mapping, q_out, k_pages, v_pages, M, K, nh, nkv, d, page_size, v_transposed)
   if (waves == 4) GO(4); else if (waves == 8) GO(8); else { if constexpr (MT == 1) GO(16); }
 #undef GO
   return ms_launch_status();
@@ -221,8 +222,7 @@ extern "C" int ms_qkv_rope_store(const float* x, long long ldx, const float* nor
       !k_pages || !v_pages)
     return MS_BAD_ARG;
 #define GO(MT) return launch<MT>(x, ldx, norm_w, eps, (const bf16*)W, bias, positions, inv_freq, slot_mapping, (bf16*)q_out, (bf16*)k_pages, (bf16*)v_pages, M, K, num_heads, num_kv_heads, head_dim, page_size, v_transposed, stream)
-  if (M <= 16) GO(1);
-  if (M <= 32) GO(2);
-  GO(4);
+  // the packed projection is narrow (few tile pairs): every 16-token group gets blocks of its own
+  GO(1);
 #undef GO
 }

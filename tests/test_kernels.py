@@ -305,7 +305,7 @@ def test_gemm_skinny(ops, M, N, K):
 
 
 @pytest.mark.parametrize("M", [3, 40])
-@pytest.mark.parametrize("shape", [(4, 4), (4, 8), (2, 8), (2, 16), (1, 8), (1, 16)])
+@pytest.mark.parametrize("shape", [(4, 4, 0), (4, 8, 0), (2, 8, 0), (2, 16, 0), (1, 8, 0), (1, 16, 0), (4, 8, 1), (2, 8, 2)])
 def test_gemm_skinny_block_shapes(ops, M, shape):
     """Every block shape on offer gives the same numbers (to float rounding of another summation order)."""
     from llm_infrence_engine_amd.kernels import build
@@ -324,13 +324,13 @@ def test_gemm_skinny_block_shapes(ops, M, shape):
         try:
             ops.gemm_skinny(a, w, bias, ops.EPI_RESIDUAL, residual=x)
         except RuntimeError as e:      # a shape that does not fit LDS with this many token groups is refused
-            assert "unsupported" in str(e) and (shape[1] - 1) * shape[0] * (1 if M <= 16 else 4) > 60
+            assert "unsupported" in str(e) and (shape[1] - 1) * shape[0] * (shape[2] or (1 if M <= 16 else 4)) > 60
             return
         torch.testing.assert_close(x.double(), x0.double() + want, atol=3e-5, rtol=3e-5)
         f = ops.gemm_skinny(a, w, bias, out_dtype=torch.float32)
         torch.testing.assert_close(f.double(), want, atol=3e-5, rtol=3e-5)
     finally:
-        lib.ms_gemm_skinny_force(0, 0)
+        lib.ms_gemm_skinny_force(0, 0, 0)
 
 
 def test_gemm_skinny_refuses_what_it_cannot_take(ops):
