@@ -193,8 +193,8 @@ int launch_cfg(const void* A, size_t lda, const bf16* W, size_t ldw, const float
   // as many tiles per block as still leaves a block for every CU; narrow outputs keep one tile per block
   // (two when there are several token groups, whose activations would otherwise be read once per tile)
   // (measured on the 0.5B shapes at 8 and 64 rows; with several token groups the wide shape pays earlier)
-  int ntile = tiles >= 1024 ? 4 : (tiles >= 512 ? (MT >= 4 ? 4 : 2) : 1);
-  int waves = ntile == 4 ? (MT == 1 ? 8 : 4) : (ntile == 2 ? 8 : ((steps >= 32 || MT > 1) ? 16 : 8));
+  int ntile = tiles >= 512 ? 4 : 1;
+  int waves = ntile == 4 ? (MT <= 2 && (MT == 1 || tiles < 1024) ? 8 : 4) : ((steps >= 32 || MT > 1) ? 16 : 8);
   if (g_force_ntile) { ntile = g_force_ntile; waves = g_force_waves; }
   if ((waves - 1) * ntile * MT > 60) return MS_UNSUPPORTED;  // LDS
 #define GO(NT, WV) if (ntile == NT && waves == WV) { if constexpr ((WV - 1) * NT * MT <= 60) { gemm_skinny_kernel<MT, NT, WV, EPI, TO, NORM><<<dim3((tiles + NT - 1) / NT, (M + 16 * MT - 1) / (16 * MT)), dim3(WV * MS_WAVE), 0, stream>>>(A, lda, W, ldw, bias, out, ldo, M, N, K, norm_w, eps, rows); return ms_launch_status(); } }
@@ -210,7 +210,7 @@ int launch_mt(const void* A, size_t lda, const bf16* W, size_t ldw, const float*
   // Several token groups per block share the weight loads; a narrow output has too few tiles to fill the chip
   // that way, so there every group gets blocks of its own (the weight tile is then re-read from L2).
   const int tiles = (N + 15) / 16;
-  const int mt = g_force_mt ? g_force_mt : ((M <= 16 || tiles <= 128) ? 1 : (M <= 32 ? 2 : 4));
+  const int mt = g_force_mt ? g_force_mt : ((M <= 16 || tiles <= 128) ? 1 : ((M <= 32 || tiles < 1024) ? 2 : 4));
   if (mt == 1) return launch_cfg<1, EPI, TO, NORM>(A, lda, W, ldw, bias, out, ldo, M, N, K, stream, norm_w, eps, rows);
   if (mt == 2) return launch_cfg<2, EPI, TO, NORM>(A, lda, W, ldw, bias, out, ldo, M, N, K, stream, norm_w, eps, rows);
   return launch_cfg<4, EPI, TO, NORM>(A, lda, W, ldw, bias, out, ldo, M, N, K, stream, norm_w, eps, rows);
