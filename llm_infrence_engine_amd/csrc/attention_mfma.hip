@@ -7,7 +7,8 @@
 //   S^T[key, col]  = K[key, :] . Q^T[:, col]        A operand: 16 keys x 32 dims, read in place from the
 //                                                   page (a lane reads 16 contiguous bytes of one key);
 //                                                   B operand: the query, kept in registers
-//   online softmax per column in float (scores are in log2 units: scale * log2(e) is folded in)
+//   online softmax per column in float, in log2 units (scale * log2(e) is folded into the exponent's
+//   multiply-add); the running reference follows the maximum in steps, so rescaling is rare
 //   O^T[dim, col] += V^T[dim, key] . P^T[key, col]  B operand: P^T straight from the S^T accumulators (a lane
 //                                                   holds 4+4 keys of its own column: no transpose);
 //                                                   A operand: V^T, which is why value pages are stored
@@ -37,55 +38,92 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+constexpr float REF_SLACK = 8.0f;   // log2 units by which a column's maximum may run ahead of its reference
+
 template <int D>
-struct KVBlock {           // one block of 32 keys as this lane sees it
+struct KeyBlock {          // one block of 32 keys as this lane sees it
   bf16x8 k[2][D / 32];     // [16-key subtile][32-dim step]
+};
+template <int D>
+struct ValueBlock {        // and its values
   bf16x4 v[D / 16][2];     // [16-dim tile][subtile]: 4 keys of one dim
 };
 
-// The pages of the two 16-key halves of the block at `base`; past the context: the null page.
-__device__ __forceinline__ void pages_of(const int* __restrict__ table, int base, int key_hi, int page_size,
+// Page arithmetic: pages of a power of two (page_shift >= 0) need no division.
+struct PageGeom {
+  int size, shift;
+  __device__ __forceinline__ int index(int key) const { return shift >= 0 ? key >> shift : key / size; }
+  __device__ __forceinline__ int offset(int key) const { return shift >= 0 ? key & (size - 1) : key % size; }
+};
+
+// The pages of the two 16-key halves of the block at `base` (the same for every lane, so they are kept in
+// scalar registers and so is all address arithmetic that follows from them); past the context: the null page.
+__device__ __forceinline__ void pages_of(const int* __restrict__ table, int base, int key_hi, PageGeom pg,
                                          int* pages) {
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
     const int kb = base + u * 16;
-    pages[u] = kb <= key_hi ? table[kb / page_size] : 0;
+    pages[u] = kb <= key_hi ? __builtin_amdgcn_readfirstlane(table[pg.index(kb)]) : 0;
+  }
+}
+
+// Where the two 16-key halves of a block start inside their page's part of one kv head: uniform values.
+struct BlockPlace {
+  size_t head[2];   // element offset of (page, kv head) in either pool
+  int off[2];       // first key inside the page
+};
+
+__device__ __forceinline__ BlockPlace place_of(const int* pages, int base, int g, int nkv, PageGeom pg, int D) {
+  BlockPlace bp;
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    bp.head[u] = ((size_t)pages[u] * nkv + g) * pg.size * D;
+    bp.off[u] = pg.offset(base + u * 16);
+  }
+  return bp;
+}
+
+template <int D>
+__device__ __forceinline__ void load_keys(KeyBlock<D>& b, const bf16* __restrict__ k_pages, const BlockPlace& bp,
+                                          int lane) {
+  const int k_lane = (lane & 15) * D + (lane >> 4) * 8;   // this lane's key and dims inside a 16-key half
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const bf16* kp = k_pages + bp.head[u] + bp.off[u] * D;
+#pragma unroll
+    for (int s = 0; s < D / 32; ++s) b.k[u][s] = *reinterpret_cast<const bf16x8*>(kp + k_lane + s * 32);
   }
 }
 
 template <int D>
-__device__ __forceinline__ void load_block(KVBlock<D>& b, const bf16* __restrict__ k_pages,
-                                           const bf16* __restrict__ vt_pages, const int* pages,
-                                           int base, int g, int nkv, int page_size, int lane) {
-  const int col = lane & 15, kq = lane >> 4;
+__device__ __forceinline__ void load_values(ValueBlock<D>& b, const bf16* __restrict__ vt_pages,
+                                            const BlockPlace& bp, PageGeom pg, int lane) {
+  const int v_lane = (lane & 15) * pg.size + (lane >> 4) * 4;   // this lane's dim and keys inside a 16-dim tile
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
-    const int kb = base + u * 16;
-    const int page = pages[u];
-    const int off = kb % page_size;
-    const bf16* kp = k_pages + (((size_t)page * nkv + g) * page_size + off + col) * D + kq * 8;
+    const bf16* vp = vt_pages + bp.head[u] + bp.off[u];
 #pragma unroll
-    for (int s = 0; s < D / 32; ++s) b.k[u][s] = *reinterpret_cast<const bf16x8*>(kp + s * 32);
-    const bf16* vp = vt_pages + (((size_t)page * nkv + g) * D + col) * page_size + off + kq * 4;
-#pragma unroll
-    for (int c = 0; c < D / 16; ++c) b.v[c][u] = *reinterpret_cast<const bf16x4*>(vp + (size_t)c * 16 * page_size);
+    for (int c = 0; c < D / 16; ++c) b.v[c][u] = *reinterpret_cast<const bf16x4*>((vp + c * 16 * pg.size) + v_lane);
   }
 }
 
+// Two waves of a wide tile on every SIMD (256 registers each) hide each other's waits; narrow tiles fit anyway.
 template <int D, int NT, int WAVES, bool SPLIT>
-__global__ void __launch_bounds__(WAVES * MS_WAVE)
+__global__ void __launch_bounds__(WAVES * MS_WAVE, (NT > 1 ? 2 : 1))
 attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* __restrict__ k_pages,
                       const bf16* __restrict__ vt_pages, const int* __restrict__ block_table, int table_stride,
                       const int* __restrict__ q_start, const int* __restrict__ context_lens,
                       bf16* __restrict__ out, size_t out_stride, float* __restrict__ part_o,
-                      float* __restrict__ part_ml, int nh, int nkv, int page_size, float scale_log2e, int window,
-                      int min_blocks, int n_splits) {
+                      float* __restrict__ part_ml, int nh, int nkv, int page_size, int page_shift,
+                      float scale_log2e, int window, int min_blocks, int n_splits) {
   __shared__ float sm_m[WAVES][NT][16], sm_l[WAVES][NT][16];
   __shared__ f32x4 sm_o[WAVES > 1 ? WAVES - 1 : 1][D / 16][NT][MS_WAVE];
-  const int lane = threadIdx.x & (MS_WAVE - 1), wave = threadIdx.x / MS_WAVE;
+  const int lane = threadIdx.x & (MS_WAVE - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MS_WAVE);   // the same for the whole wave
   const int col16 = lane & 15, kq = lane >> 4;
   const int r = blockIdx.z, g = blockIdx.y;
   const int rep = nh / nkv;
+  const PageGeom pg = {page_size, page_shift};
   const int* table = block_table + (size_t)r * table_stride;
   // Without a window a wave's first key block is known before the request's lengths are: ask for its page
   // ids at once, so that they travel together with the lengths instead of after them.
@@ -93,7 +131,8 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
   const bool early = !SPLIT && window <= 0;
   if (early) {
 #pragma unroll
-    for (int u = 0; u < 2; ++u) first_pages[u] = table[min((wave * 32 + u * 16) / page_size, table_stride - 1)];
+    for (int u = 0; u < 2; ++u)
+      first_pages[u] = __builtin_amdgcn_readfirstlane(table[min(pg.index(wave * 32 + u * 16), table_stride - 1)]);
   }
   const int q0 = q_start[r];
   const int qlen = q_start[r + 1] - q0;
@@ -122,18 +161,15 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
   }
 
   // this lane's columns
-  int pos[NT], tok[NT], head[NT];
-  bool valid[NT];
+  int pos[NT];   // -1: an idle column (sees no key; its result is not written)
   bf16x8 qv[NT][D / 32];
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     const int c = c0 + t * 16 + col16;
-    valid[t] = c < ncols;
     const int cc = min(c, ncols - 1);
-    tok[t] = q0 + cc / rep;
-    head[t] = g * rep + cc % rep;
-    pos[t] = valid[t] ? start_pos + cc / rep : -1;
-    const bf16* qp = q + (size_t)tok[t] * q_stride + (size_t)head[t] * D + kq * 8;
+    const int tok = q0 + cc / rep, head = g * rep + cc % rep;
+    pos[t] = c < ncols ? start_pos + cc / rep : -1;
+    const bf16* qp = q + (size_t)tok * q_stride + (size_t)head * D + kq * 8;
 #pragma unroll
     for (int s = 0; s < D / 32; ++s) qv[t][s] = *reinterpret_cast<const bf16x8*>(qp + s * 32);
   }
@@ -148,7 +184,13 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
     for (int c = 0; c < D / 16; ++c) o[c][t] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  KVBlock<D> cur, nxt;
+  // A narrow tile (decode) has registers to spare and few waves to hide a wait behind: it fetches the next
+  // block's values early, together with its keys.  A wide tile fetches values at the top of the pass that
+  // uses them (the score products and the softmax run meanwhile, and so does the SIMD's other wave).
+  constexpr bool VALUES_EARLY = NT == 1;
+  KeyBlock<D> cur_k, nxt_k;
+  ValueBlock<D> cur_v, nxt_v;
+  BlockPlace cur_at, nxt_at;
   if (blk_begin + wave < blk_end) {
     const int base = (blk_begin + wave) * 32;
     int pages[2];
@@ -156,16 +198,21 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
 #pragma unroll
       for (int u = 0; u < 2; ++u) pages[u] = base + u * 16 <= key_hi ? first_pages[u] : 0;
     } else {
-      pages_of(table, base, key_hi, page_size, pages);
+      pages_of(table, base, key_hi, pg, pages);
     }
-    load_block<D>(cur, k_pages, vt_pages, pages, base, g, nkv, page_size, lane);
+    cur_at = place_of(pages, base, g, nkv, pg, D);
+    load_keys<D>(cur_k, k_pages, cur_at, lane);
+    if (VALUES_EARLY) load_values<D>(cur_v, vt_pages, cur_at, pg, lane);
   }
   for (int blk = blk_begin + wave; blk < blk_end; blk += WAVES) {
     const int base = blk * 32;
+    if (!VALUES_EARLY) load_values<D>(cur_v, vt_pages, cur_at, pg, lane);
     if (blk + WAVES < blk_end) {
       int pages[2];
-      pages_of(table, base + WAVES * 32, key_hi, page_size, pages);
-      load_block<D>(nxt, k_pages, vt_pages, pages, base + WAVES * 32, g, nkv, page_size, lane);
+      pages_of(table, base + WAVES * 32, key_hi, pg, pages);
+      nxt_at = place_of(pages, base + WAVES * 32, g, nkv, pg, D);
+      load_keys<D>(nxt_k, k_pages, nxt_at, lane);
+      if (VALUES_EARLY) load_values<D>(nxt_v, vt_pages, nxt_at, pg, lane);
     }
 
     // scores: s[u][t] holds keys base + u*16 + kq*4 + (0..3) of column t*16 + col16
@@ -176,7 +223,7 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
       for (int t = 0; t < NT; ++t) {
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int ks = 0; ks < D / 32; ++ks) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.k[u][ks], qv[t][ks], acc, 0, 0, 0);
+        for (int ks = 0; ks < D / 32; ++ks) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur_k.k[u][ks], qv[t][ks], acc, 0, 0, 0);
         s[u][t] = acc;
       }
 
@@ -188,24 +235,23 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
         for (int i = 0; i < 4; ++i)
           if (base + u * 16 + kq * 4 + i > key_hi) {
 #pragma unroll
-            for (int c = 0; c < D / 16; ++c) cur.v[c][u][i] = (__bf16)0.0f;
+            for (int c = 0; c < D / 16; ++c) cur_v.v[c][u][i] = (__bf16)0.0f;
           }
     }
 
     const bool unmasked = full_tile && base + 31 <= first_pos && (window <= 0 || base > key_hi - window);
     bf16x8 p[NT];
+    float corr[NT];
+    bool moved = false;
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
+      // the block's maximum of the raw scores (the scale is positive, so it is the maximum of the scaled ones too)
       float bm = -INFINITY;
       if (unmasked) {
 #pragma unroll
         for (int u = 0; u < 2; ++u)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const float v = s[u][t][i] * scale_log2e;
-            s[u][t][i] = v;
-            bm = fmaxf(bm, v);
-          }
+          for (int i = 0; i < 4; ++i) bm = fmaxf(bm, s[u][t][i]);
       } else {
 #pragma unroll
         for (int u = 0; u < 2; ++u)
@@ -213,40 +259,55 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
           for (int i = 0; i < 4; ++i) {
             const int key = base + u * 16 + kq * 4 + i;
             const bool see = key <= pos[t] && (window <= 0 || key > pos[t] - window);
-            const float v = see ? s[u][t][i] * scale_log2e : -INFINITY;
+            const float v = see ? s[u][t][i] : -INFINITY;
             s[u][t][i] = v;
             bm = fmaxf(bm, v);
           }
       }
       bm = fmaxf(bm, __shfl_xor(bm, 16, MS_WAVE));
       bm = fmaxf(bm, __shfl_xor(bm, 32, MS_WAVE));
-      const float m_new = fmaxf(m[t], bm);
-      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-      const float corr = fast_exp2(m[t] - m_safe);
+      bm *= scale_log2e;
+      // m is the reference that the exponents are taken against, not necessarily the maximum: it follows the
+      // maximum only when that has run ahead by more than REF_SLACK (a factor 2^REF_SLACK in the terms, far
+      // inside float's range), so that the accumulators are rescaled rarely.  Any reference gives the same
+      // softmax; all lanes of a column decide alike because bm is the same in all of them.
+      const bool step = bm > m[t] + REF_SLACK;
+      const float m_new = step ? bm : m[t];
+      corr[t] = step ? fast_exp2(m[t] - m_new) : 1.0f;   // m = -inf: 0
+      moved |= step;
       m[t] = m_new;
+      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
       float ls = 0.f;
 #pragma unroll
       for (int u = 0; u < 2; ++u)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const float e = fast_exp2(s[u][t][i] - m_safe);
+          const float e = fast_exp2(fmaf(s[u][t][i], scale_log2e, -m_safe));
           ls += e;
           p[t][u * 4 + i] = (__bf16)e;
         }
-      l[t] = l[t] * corr + ls;
+      l[t] = l[t] * corr[t] + ls;
+    }
+    if (NT == 1 || __builtin_amdgcn_ballot_w64(moved) != 0) {   // the same branch for the whole wave
 #pragma unroll
-      for (int c = 0; c < D / 16; ++c) o[c][t] *= corr;
+      for (int t = 0; t < NT; ++t)
+#pragma unroll
+        for (int c = 0; c < D / 16; ++c) o[c][t] *= corr[t];
     }
 
 #pragma unroll
     for (int c = 0; c < D / 16; ++c) {
       bf16x8 vv;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) { vv[i] = cur.v[c][0][i]; vv[4 + i] = cur.v[c][1][i]; }
+      for (int i = 0; i < 4; ++i) { vv[i] = cur_v.v[c][0][i]; vv[4 + i] = cur_v.v[c][1][i]; }
 #pragma unroll
       for (int t = 0; t < NT; ++t) o[c][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, p[t], o[c][t], 0, 0, 0);
     }
-    if (blk + WAVES < blk_end) cur = nxt;
+    if (blk + WAVES < blk_end) {
+      cur_k = nxt_k;
+      cur_at = nxt_at;
+      if (VALUES_EARLY) cur_v = nxt_v;
+    }
   }
 
 #pragma unroll
@@ -289,17 +350,19 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     const float lt = l[t];
-    if (!valid[t]) continue;
+    if (pos[t] < 0) continue;
+    const int c = c0 + t * 16 + col16;   // worked out again rather than kept through the loop
+    const int tok = q0 + c / rep, head = g * rep + c % rep;
     if (SPLIT) {
       // unnormalised: O, the running maximum (log2 units) and the sum; the combine kernel weighs the splits
-      const size_t slot = ((size_t)r * nh + head[t]) * n_splits + blockIdx.x;
+      const size_t slot = ((size_t)r * nh + head) * n_splits + blockIdx.x;
       float* po = part_o + slot * D + kq * 4;
 #pragma unroll
       for (int c = 0; c < D / 16; ++c) *reinterpret_cast<f32x4*>(po + c * 16) = o[c][t];
       if (kq == 0) { part_ml[slot * 2] = m[t]; part_ml[slot * 2 + 1] = lt; }
     } else {
       const float inv = 1.0f / lt;
-      bf16* op = out + (size_t)tok[t] * out_stride + (size_t)head[t] * D + kq * 4;
+      bf16* op = out + (size_t)tok * out_stride + (size_t)head * D + kq * 4;
 #pragma unroll
       for (int c = 0; c < D / 16; ++c) {
         bf16x4 w;
@@ -337,6 +400,15 @@ __global__ void attention_combine_kernel(const float* __restrict__ part_o, const
   }
 }
 
+int g_force_nt = 0, g_force_waves = 0;
+
+inline int page_shift_of(int page_size) {   // log2 of a power of two, else -1
+  if (page_size & (page_size - 1)) return -1;
+  int sh = 0;
+  while ((1 << sh) < page_size) ++sh;
+  return sh;
+}
+
 template <int D, int NT, int WAVES>
 int launch_general(const bf16* q, size_t q_stride, const bf16* k, const bf16* vt, const int* table, int table_stride,
                    const int* q_start, const int* ctx, bf16* out, size_t out_stride, int n_requests, int max_q_len,
@@ -344,7 +416,7 @@ int launch_general(const bf16* q, size_t q_stride, const bf16* k, const bf16* vt
   const int rep = nh / nkv;
   const int tiles = (max_q_len * rep + 16 * NT - 1) / (16 * NT);
   dim3 grid(tiles, nkv, n_requests), block(WAVES * MS_WAVE);
-  attention_mfma_kernel<D, NT, WAVES, false><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, q_start, ctx, out, out_stride, nullptr, nullptr, nh, nkv, page_size, scale * 1.4426950408889634f, window, 0, 0);
+  attention_mfma_kernel<D, NT, WAVES, false><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, q_start, ctx, out, out_stride, nullptr, nullptr, nh, nkv, page_size, page_shift_of(page_size), scale * 1.4426950408889634f, window, 0, 0);
   return ms_launch_status();
 }
 
@@ -354,12 +426,19 @@ int launch_split(const bf16* q, size_t q_stride, const bf16* k, const bf16* vt, 
                  int n_requests, int nh, int nkv, int page_size, float scale, int window, int min_blocks,
                  int n_splits, hipStream_t stream) {
   dim3 grid(n_splits, nkv, n_requests), block(4 * MS_WAVE);
-  attention_mfma_kernel<D, 1, 4, true><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, q_start, ctx, out, out_stride, part_o, part_ml, nh, nkv, page_size, scale * 1.4426950408889634f, window, min_blocks, n_splits);
+  attention_mfma_kernel<D, 1, 4, true><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, q_start, ctx, out, out_stride, part_o, part_ml, nh, nkv, page_size, page_shift_of(page_size), scale * 1.4426950408889634f, window, min_blocks, n_splits);
   attention_combine_kernel<D><<<dim3(n_requests * nh), dim3(D < 64 ? 64 : D), 0, stream>>>(part_o, part_ml, q_start, ctx, out, out_stride, nh, window, min_blocks, n_splits);
   return ms_launch_status();
 }
 
 }  // namespace
+
+// Tuning knob: force the general shape's tile width (16 * nt columns) and waves per tile; 0 restores the choice
+// by size.  Shapes outside the menu are refused at the call.
+extern "C" void ms_attention_mfma_force(int nt, int waves) {
+  g_force_nt = nt;
+  g_force_waves = waves;
+}
 
 // Whether the matrix-core kernels take this geometry (else the caller uses the generic kernel).
 extern "C" int ms_attention_mfma_supported(int head_dim, int page_size) {
@@ -376,15 +455,23 @@ extern "C" int ms_paged_attention_mfma(const void* q, long long q_stride, const 
                                        float scale, int window, hipStream_t stream) {
   if (n_requests <= 0 || max_q_len <= 0) return MS_OK;
   if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads || table_stride <= 0) return MS_BAD_ARG;
+  if (!(scale > 0.f)) return MS_BAD_ARG;   // maxima are taken of the raw scores
   if (!ms_attention_mfma_supported(head_dim, page_size)) return MS_UNSUPPORTED;
   if (q_stride % 8 || out_stride % 4 || ((uintptr_t)q % 16) || ((uintptr_t)out % 8)) return MS_UNSUPPORTED;
   if (n_requests > 65535 || num_kv_heads > 65535) return MS_UNSUPPORTED;
 #define GO(D, NT, WV) return launch_general<D, NT, WV>((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)vt_pages, block_table, table_stride, q_start, context_lens, (bf16*)out, out_stride, n_requests, max_q_len, num_heads, num_kv_heads, page_size, scale, window, stream)
-  // few columns (a decode step): one narrow tile per request, more waves over its keys
+  // Tile width (NT * 16 columns) and waves over a tile's keys.  Few columns (a decode step): one narrow tile
+  // per request and many waves over its keys.
   const int cols = max_q_len * (num_heads / num_kv_heads);
-  if (head_dim == 32) { if (cols > 16) GO(32, 4, 4); else GO(32, 1, 16); }
-  if (head_dim == 64) { if (cols > 16) GO(64, 4, 4); else GO(64, 1, 16); }
-  if (cols > 16) GO(128, 2, 4); else GO(128, 1, 8);
+  int nt = cols > 16 ? (head_dim == 128 ? 2 : 4) : 1;
+  int waves = nt > 1 ? 4 : (head_dim == 128 ? 8 : 16);
+  if (g_force_nt) { nt = g_force_nt; waves = g_force_waves; }
+#define PICK(D, NT, WV) if (head_dim == D && nt == NT && waves == WV) GO(D, NT, WV)
+  PICK(32, 4, 4); PICK(32, 4, 8); PICK(32, 2, 4); PICK(32, 2, 8); PICK(32, 1, 8); PICK(32, 1, 16);
+  PICK(64, 4, 4); PICK(64, 2, 4); PICK(64, 2, 8); PICK(64, 1, 4); PICK(64, 1, 8); PICK(64, 1, 16);
+  PICK(128, 2, 4); PICK(128, 1, 4); PICK(128, 1, 8);
+#undef PICK
+  return MS_UNSUPPORTED;
 #undef GO
 }
 
@@ -403,6 +490,7 @@ extern "C" int ms_paged_attention_mfma_decode(const void* q, long long q_stride,
   if (n_requests <= 0) return MS_OK;
   if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads || table_stride <= 0) return MS_BAD_ARG;
   if (num_heads / num_kv_heads > 16) return MS_UNSUPPORTED;
+  if (!(scale > 0.f)) return MS_BAD_ARG;
   if (!ms_attention_mfma_supported(head_dim, page_size)) return MS_UNSUPPORTED;
   if (min_blocks <= 0 || n_splits <= 0 || n_splits > 65535) return MS_BAD_ARG;
   if (q_stride % 8 || out_stride % 4 || ((uintptr_t)q % 16) || ((uintptr_t)out % 8) || ((uintptr_t)part_o % 16)) return MS_UNSUPPORTED;
