@@ -402,7 +402,8 @@ def _paged_case(g, dtype, nh, nkv, d, page_size, ctx, qlen, fill):
 
 
 @pytest.mark.parametrize("nh,nkv,d,page_size,window", [(14, 2, 64, 16, None), (6, 2, 32, 16, None), (8, 8, 128, 32, None),
-                                                        (4, 1, 64, 16, 40), (28, 4, 128, 16, None), (5, 5, 32, 64, 100)])
+                                                        (4, 1, 64, 16, 40), (28, 4, 128, 16, None), (5, 5, 32, 64, 100),
+                                                        (6, 2, 64, 48, None)])
 @pytest.mark.parametrize("shape", ["mixed", "decode", "long"])
 def test_paged_attention_mfma(ops, nh, nkv, d, page_size, window, shape):
     g = torch.Generator().manual_seed(nh * 100 + d)
@@ -431,6 +432,65 @@ def test_paged_attention_mfma(ops, nh, nkv, d, page_size, window, shape):
                                 torch.tensor(c["req"], dtype=torch.int32, device=DEV),
                                 torch.tensor(c["pos"], dtype=torch.int32, device=DEV), out2, nh, scale, window, v_transposed=True)
     torch.testing.assert_close(out2.double().cpu(), want, **tol(torch.bfloat16))
+
+
+def _run_mfma(ops, c, nh, d, ctx, qlen, window=None):
+    N = c["q"].shape[0]
+    out = torch.full((N, nh * d), float("nan"), dtype=torch.bfloat16, device=DEV)
+    q_start = torch.tensor([0] + list(np.cumsum(qlen)), dtype=torch.int32, device=DEV)
+    ops.paged_attention_mfma(c["q"].to(DEV), c["kp"].to(DEV), c["vt"].to(DEV), c["table"].to(DEV), q_start,
+                             torch.tensor(ctx, dtype=torch.int32, device=DEV), out, nh, 1.0 / math.sqrt(d), max(qlen),
+                             max(ctx), window)
+    return out.double().cpu()
+
+
+@pytest.mark.parametrize("d,shape", [(32, (4, 4)), (32, (4, 8)), (32, (2, 4)), (32, (2, 8)), (32, (1, 8)), (32, (1, 16)),
+                                     (64, (4, 4)), (64, (2, 4)), (64, (2, 8)), (64, (1, 4)), (64, (1, 8)), (64, (1, 16)),
+                                     (128, (2, 4)), (128, (1, 4)), (128, (1, 8))])
+def test_attention_mfma_tile_shapes(ops, d, shape):
+    """Every tile width and wave count of the menu gives the same answer (the choice by size picks among them)."""
+    from llm_infrence_engine_amd.kernels import build
+    nh, nkv = 6, 2
+    g = torch.Generator().manual_seed(d + shape[0] * 7 + shape[1])
+    ctx, qlen = [300, 97, 520], [130, 1, 45]
+    c = _paged_case(g, torch.bfloat16, nh, nkv, d, 16, ctx, qlen, float("nan"))
+    want = torch.cat([attention_reference(q.double(), k.double(), v.double(), 1.0 / math.sqrt(d), None).transpose(0, 1).reshape(-1, nh * d)
+                      for q, k, v in zip(c["qs"], c["ks"], c["vs"])])
+    lib = build.load()
+    lib.ms_attention_mfma_force(*shape)
+    try:
+        got = _run_mfma(ops, c, nh, d, ctx, qlen)
+    finally:
+        lib.ms_attention_mfma_force(0, 0)
+    torch.testing.assert_close(got, want, **tol(torch.bfloat16))
+
+
+@pytest.mark.parametrize("ramp", [0.5, 6.0, 60.0])
+def test_attention_mfma_when_the_maximum_keeps_rising(ops, ramp):
+    """Scores that grow along the context by ``ramp`` log2 units in all: the running reference of the softmax
+    stays (small ramp), moves once or moves at almost every block, and late keys dwarf the early ones."""
+    nh, nkv, d = 4, 2, 64
+    g = torch.Generator().manual_seed(int(ramp * 10))
+    ctx, qlen = [640, 333], [200, 1]
+    c = _paged_case(g, torch.bfloat16, nh, nkv, d, 16, ctx, qlen, float("nan"))
+    scale = 1.0 / math.sqrt(d)
+    # all queries share a direction u; key j carries (j / ctx) * ramp * ln2 / scale along it
+    u = torch.zeros(d); u[5] = 1.0
+    for r in range(len(ctx)):
+        c["qs"][r] = (c["qs"][r].float() * 0.05 + u).to(torch.bfloat16)
+        steps = torch.arange(ctx[r]).float() / ctx[r] * ramp * math.log(2.0) / scale
+        c["ks"][r] = (c["ks"][r].float() * 0.05 + steps[None, :, None] * u).to(torch.bfloat16)
+    # lay the changed keys and queries out again
+    rows, p = [], 0
+    for r in range(len(ctx)):
+        for j in range(ctx[r]):
+            c["kp"][c["table"][r, j // 16].item(), :, j % 16] = c["ks"][r][:, j]
+        rows.append(c["qs"][r].transpose(0, 1).reshape(qlen[r], nh * d))
+    c["q"] = torch.cat(rows)
+    want = torch.cat([attention_reference(q.double(), k.double(), v.double(), scale, None).transpose(0, 1).reshape(-1, nh * d)
+                      for q, k, v in zip(c["qs"], c["ks"], c["vs"])])
+    got = _run_mfma(ops, c, nh, d, ctx, qlen)
+    torch.testing.assert_close(got, want, **tol(torch.bfloat16))
 
 
 def test_attention_mfma_support_matrix(ops):
