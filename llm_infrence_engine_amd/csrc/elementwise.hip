@@ -252,6 +252,103 @@ __global__ void rope_store_kernel(T* __restrict__ qkv, const float* __restrict__
   }
 }
 
+// The same work 16 bytes at a time, four tokens to a block (64 threads each): the angles of a token are worked
+// out once and shared by all its heads, a thread rotates VEC pairs of one head and, for a key head, puts them
+// into the page from its registers; so one barrier (after the angles) is all.  Needs rot_dim / 2 and head_dim
+// to be multiples of VEC = 16 / sizeof(T) and rot_dim / 2 <= ROPE_MAX_HALF.
+constexpr int ROPE_TOKENS = 4, ROPE_GROUP = 64, ROPE_MAX_HALF = 128;
+
+template <typename T, int VEC>
+struct alignas(16) Packet { T v[VEC]; };
+
+template <typename T, int VEC>
+__global__ void __launch_bounds__(ROPE_TOKENS * ROPE_GROUP)
+rope_store_vec_kernel(T* __restrict__ qkv, const float* __restrict__ bias, const int* __restrict__ positions,
+                      const float* __restrict__ inv_freq, const int* __restrict__ slot_mapping,
+                      T* __restrict__ k_pages, T* __restrict__ v_pages, int n_tokens, int nh, int nkv, int d,
+                      int rot_dim, int page_size, int v_transposed) {
+  typedef Packet<T, VEC> Vec;
+  typedef Packet<float, VEC> FVec;
+  __shared__ float sm_cos[ROPE_TOKENS][ROPE_MAX_HALF], sm_sin[ROPE_TOKENS][ROPE_MAX_HALF];
+  const int tg = threadIdx.x / ROPE_GROUP, tl = threadIdx.x % ROPE_GROUP;
+  const int n = blockIdx.x * ROPE_TOKENS + tg;
+  const bool live = n < n_tokens;
+  const int half = rot_dim / 2;
+  if (live && half > 0) {
+    const float pos = (float)positions[n];
+    for (int j = tl; j < half; j += ROPE_GROUP) sincosf(pos * inv_freq[j], &sm_sin[tg][j], &sm_cos[tg][j]);
+  }
+  __syncthreads();
+  if (!live) return;
+  T* row = qkv + (size_t)n * (nh + 2 * nkv) * d;
+  long long slot = -1;
+  if (k_pages) slot = slot_mapping[n];
+  const long long page = slot >= 0 ? slot / page_size : 0;
+  const int off = slot >= 0 ? (int)(slot % page_size) : 0;
+
+  // rotated pairs of q and k heads: work item = (head, VEC consecutive j)
+  const int per_head = half / VEC;
+  for (int w = tl; w < (nh + nkv) * per_head; w += ROPE_GROUP) {
+    const int h = w / per_head, j = (w - h * per_head) * VEC;
+    T* x = row + (size_t)h * d;
+    Vec a = *reinterpret_cast<const Vec*>(x + j), b = *reinterpret_cast<const Vec*>(x + j + half);
+    FVec ba = {}, bb = {};
+    if (bias) {
+      ba = *reinterpret_cast<const FVec*>(bias + h * d + j);
+      bb = *reinterpret_cast<const FVec*>(bias + h * d + j + half);
+    }
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      const float x1 = to_float(a.v[i]) + ba.v[i], x2 = to_float(b.v[i]) + bb.v[i];
+      const float c = sm_cos[tg][j + i], sn = sm_sin[tg][j + i];
+      a.v[i] = from_float<T>(x1 * c - x2 * sn);
+      b.v[i] = from_float<T>(x2 * c + x1 * sn);
+    }
+    *reinterpret_cast<Vec*>(x + j) = a;
+    *reinterpret_cast<Vec*>(x + j + half) = b;
+    if (h >= nh && slot >= 0) {
+      T* dst = k_pages + (((size_t)page * nkv + (h - nh)) * page_size + off) * d;
+      *reinterpret_cast<Vec*>(dst + j) = a;
+      *reinterpret_cast<Vec*>(dst + j + half) = b;
+    }
+  }
+  // what is not rotated: the tails of q and k heads beyond rot_dim (bias, and the store of k), and v
+  const int tail_vecs = (d - rot_dim) / VEC;
+  for (int w = tl; w < (nh + nkv) * tail_vecs; w += ROPE_GROUP) {
+    const int h = w / tail_vecs, i0 = rot_dim + (w - h * tail_vecs) * VEC;
+    T* x = row + (size_t)h * d + i0;
+    Vec a = *reinterpret_cast<const Vec*>(x);
+    if (bias) {
+      const FVec bv = *reinterpret_cast<const FVec*>(bias + h * d + i0);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) a.v[i] = from_float<T>(to_float(a.v[i]) + bv.v[i]);
+      *reinterpret_cast<Vec*>(x) = a;
+    }
+    if (h >= nh && slot >= 0)
+      *reinterpret_cast<Vec*>(k_pages + (((size_t)page * nkv + (h - nh)) * page_size + off) * d + i0) = a;
+  }
+  const int v_vecs = d / VEC;
+  for (int w = tl; w < nkv * v_vecs; w += ROPE_GROUP) {
+    const int h = w / v_vecs, i0 = (w - h * v_vecs) * VEC;
+    T* x = row + (size_t)(nh + nkv + h) * d + i0;
+    Vec a = *reinterpret_cast<const Vec*>(x);
+    if (bias) {
+      const FVec bv = *reinterpret_cast<const FVec*>(bias + (nh + nkv + h) * d + i0);
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) a.v[i] = from_float<T>(to_float(a.v[i]) + bv.v[i]);
+      *reinterpret_cast<Vec*>(x) = a;
+    }
+    if (slot < 0) continue;
+    if (v_transposed) {   // [page][kv head][dim][page_size]: one element to each dim's row
+      T* dst = v_pages + (((size_t)page * nkv + h) * d + i0) * page_size + off;
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) dst[(size_t)i * page_size] = a.v[i];
+    } else {
+      *reinterpret_cast<Vec*>(v_pages + (((size_t)page * nkv + h) * page_size + off) * d + i0) = a;
+    }
+  }
+}
+
 extern "C" int ms_rope_store(void* qkv, const float* bias, const int* positions, const float* inv_freq, const int* slot_mapping,
                              void* k_pages, void* v_pages, int n_tokens, int num_heads, int num_kv_heads,
                              int head_dim, int rot_dim, int page_size, int v_transposed, int dtype,
@@ -262,6 +359,19 @@ extern "C" int ms_rope_store(void* qkv, const float* bias, const int* positions,
   if ((k_pages == nullptr) != (v_pages == nullptr)) return MS_BAD_ARG;
   if (k_pages && (page_size <= 0 || slot_mapping == nullptr)) return MS_BAD_ARG;
   if (rot_dim > 0 && (positions == nullptr || inv_freq == nullptr)) return MS_BAD_ARG;
+  {  // 16 bytes at a time where the sizes allow
+    const int vec = dtype == MS_BF16 ? 8 : 4;
+    const bool aligned = ((uintptr_t)qkv % 16) == 0 && ((uintptr_t)k_pages % 16) == 0 &&
+                         ((uintptr_t)v_pages % 16) == 0 && ((uintptr_t)bias % 16) == 0;
+    if ((dtype == MS_BF16 || dtype == MS_F32) && aligned && head_dim % vec == 0 && (rot_dim / 2) % vec == 0 &&
+        rot_dim / 2 <= ROPE_MAX_HALF) {
+      dim3 vgrid((n_tokens + ROPE_TOKENS - 1) / ROPE_TOKENS), vblock(ROPE_TOKENS * ROPE_GROUP);
+#define LAUNCH_VEC(T, VEC) rope_store_vec_kernel<T, VEC><<<vgrid, vblock, 0, stream>>>((T*)qkv, bias, positions, inv_freq, slot_mapping, (T*)k_pages, (T*)v_pages, n_tokens, num_heads, num_kv_heads, head_dim, rot_dim, page_size, v_transposed)
+      if (dtype == MS_BF16) LAUNCH_VEC(bf16, 8); else LAUNCH_VEC(float, 4);
+#undef LAUNCH_VEC
+      return ms_launch_status();
+    }
+  }
   dim3 grid(n_tokens), block(256);
 #define LAUNCH(T) rope_store_kernel<T><<<grid, block, 0, stream>>>((T*)qkv, bias, positions, inv_freq, slot_mapping, (T*)k_pages, (T*)v_pages, num_heads, num_kv_heads, head_dim, rot_dim, page_size, v_transposed)
   if (dtype == MS_F32) LAUNCH(float);

@@ -119,8 +119,12 @@ def rope_reference(x, pos, rot, inv):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("nh,nkv,d,rot", [(4, 2, 16, 16), (5, 1, 48, 48), (6, 3, 80, 32)])
-def test_rope_store(ops, dtype, nh, nkv, d, rot):
+@pytest.mark.parametrize("vt", [False, True])
+@pytest.mark.parametrize("nh,nkv,d,rot", [(4, 2, 16, 16), (5, 1, 48, 48), (6, 3, 80, 32), (3, 1, 20, 20), (2, 2, 24, 12),
+                                          (14, 2, 64, 64), (2, 1, 256, 256)])
+def test_rope_store(ops, dtype, nh, nkv, d, rot, vt):
+    """Sizes that the 16-byte kernel takes and sizes that fall to the element-wise one; values pages plain and
+    transposed; with and without a late bias; one token that is not stored."""
     g = torch.Generator().manual_seed(5)
     N, page_size, pages = 11, 4, 9
     qkv = torch.randn(N, (nh + 2 * nkv) * d, generator=g).to(dtype)
@@ -130,10 +134,10 @@ def test_rope_store(ops, dtype, nh, nkv, d, rot):
     theta = 1e6
     inv_freq = (1.0 / (theta ** (torch.arange(0, rot, 2, dtype=torch.float64) / rot))).float()
     kp = torch.zeros(pages, nkv, page_size, d, dtype=dtype, device=DEV)
-    vp = torch.zeros_like(kp)
+    vp = torch.zeros(pages, nkv, d, page_size, dtype=dtype, device=DEV) if vt else torch.zeros_like(kp)
     dev = qkv.to(DEV)
     bias = torch.randn((nh + 2 * nkv) * d, generator=g) if rot != 16 else None   # with and without a late bias
-    ops.rope_store(dev, nh, nkv, d, rot, pos.to(DEV), inv_freq.to(DEV), slots.to(DEV), kp, vp,
+    ops.rope_store(dev, nh, nkv, d, rot, pos.to(DEV), inv_freq.to(DEV), slots.to(DEV), kp, vp, v_transposed=vt,
                    bias=None if bias is None else bias.to(DEV))
     x = qkv.double().view(N, nh + 2 * nkv, d)
     if bias is not None:
@@ -154,7 +158,7 @@ def test_rope_store(ops, dtype, nh, nkv, d, rot):
             continue
         p, o = divmod(s, page_size)
         assert torch.equal(kp[p, :, o].cpu().double(), got[n, nh:nh + nkv])
-        assert torch.equal(vp[p, :, o].cpu().double(), got[n, nh + nkv:])
+        assert torch.equal((vp[p, :, :, o] if vt else vp[p, :, o]).cpu().double(), got[n, nh + nkv:])
     used = torch.zeros(pages * page_size, dtype=torch.bool)
     used[slots[slots >= 0].long()] = True
     assert (kp.cpu().permute(0, 2, 1, 3).reshape(pages * page_size, -1)[~used] == 0).all()
