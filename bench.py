@@ -31,6 +31,14 @@ MODEL = {
     "num_key_value_heads": 2, "intermediate_size": 4864, "vocab_size": 151936, "rope_theta": 1000000.0,
     "rms_norm_eps": 1e-6, "tie_word_embeddings": True,
 }
+# further shapes of the same architecture (Qwen2.5-7B and -32B config.json sizes), for --shape
+SHAPES = {
+    "0.5b": MODEL,
+    "7b": {**MODEL, "num_hidden_layers": 28, "hidden_size": 3584, "num_attention_heads": 28, "num_key_value_heads": 4,
+           "intermediate_size": 18944, "vocab_size": 152064, "tie_word_embeddings": False},
+    "32b": {**MODEL, "num_hidden_layers": 64, "hidden_size": 5120, "num_attention_heads": 40, "num_key_value_heads": 8,
+            "intermediate_size": 27648, "vocab_size": 152064, "tie_word_embeddings": False, "rms_norm_eps": 1e-5},
+}
 PROMPT_LEN = 512
 CONTEXT_LIMIT = 8192
 BLOCK_SIZE = 16
@@ -120,7 +128,9 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--layers", type=int, default=MODEL["num_hidden_layers"],
+    ap.add_argument("--shape", choices=sorted(SHAPES), default="0.5b",
+                    help="layer sizes: the default is the configuration the headline numbers are quoted on")
+    ap.add_argument("--layers", type=int, default=None,
                     help="fewer layers than the configuration has, if memory or time needs it (both numbers are reported)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points and the prefill")
     ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN, help="prompt length of the decode run (default 512)")
@@ -135,7 +145,10 @@ def main() -> int:
     import llm_infrence_engine_amd as eng
     from llm_infrence_engine_amd.config import config_from_dict
 
-    d = dict(MODEL)
+    shape = SHAPES[a.shape]
+    if a.layers is None:
+        a.layers = shape["num_hidden_layers"]
+    d = dict(shape)
     d["num_hidden_layers"] = a.layers
     cfg = config_from_dict(d)
     with tempfile.TemporaryDirectory() as folder:
@@ -154,11 +167,13 @@ def main() -> int:
     out = {
         "metric": "decode_tokens_per_s", "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1,
         "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": round(value / REFERENCE_TOKS, 2), "dtype": "bf16", "data": "synthetic",
+        "scaling": "weak", "vs_baseline": round(value / REFERENCE_TOKS, 2) if a.shape == "0.5b" else None,
+        "dtype": "bf16", "data": "synthetic",
         "config": {
-            "model": "Qwen2.5-0.5B shape, random weights", "layers": a.layers, "layers_of_config": MODEL["num_hidden_layers"],
+            "model": f"Qwen2.5-{a.shape.upper()} shape, random weights", "layers": a.layers,
+            "layers_of_config": shape["num_hidden_layers"],
             "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
-            "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": vocab, "tied": True,
+            "head_dim": cfg.head_dim, "intermediate": cfg.intermediate_size, "vocab": vocab, "tied": cfg.tie_word_embeddings,
             "global_batch": a.batch, "prompt_len": a.prompt_len, "seq_len": CONTEXT_LIMIT, "block_size": BLOCK_SIZE,
             "prefill_tokens": PREFILL_TOKENS, "parallelism": "single_gpu",
             "decode_steps_per_launch": DECODE_STEPS_PER_LAUNCH,

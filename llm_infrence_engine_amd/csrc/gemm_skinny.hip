@@ -26,11 +26,19 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 enum { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_RESIDUAL = 3 };
 
+// g * sigmoid(g) through the hardware's exp2 and reciprocal (each good to about one unit in the last place of
+// a float; the result is rounded to bfloat16)
+__device__ __forceinline__ float fast_silu(float g) {
+  return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g));
+}
+
+// The tiles are dealt out evenly: the first `rem` blocks take q + 1 tiles, the others q (at most NTILE), so that
+// every CU streams about the same share of W.
 template <int MT, int NTILE, int WAVES, int EPI, typename TO, bool NORM>
 __global__ void __launch_bounds__(WAVES * MS_WAVE)
 gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restrict__ W, size_t ldw,
                    const float* __restrict__ bias, TO* __restrict__ out, size_t ldo, int M, int N, int K,
-                   const float* __restrict__ norm_w, float eps, const int* __restrict__ rows) {
+                   const float* __restrict__ norm_w, float eps, const int* __restrict__ rows, int q, int rem) {
   constexpr int ITEMS = NTILE * MT;
   __shared__ f32x4 red[WAVES - 1][ITEMS][MS_WAVE];
   __shared__ float red_ss[NORM ? WAVES : 1][MT][16];
@@ -38,7 +46,8 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
   const float* X = (const float*)Av;
   const int lane = threadIdx.x & (MS_WAVE - 1), wave = threadIdx.x / MS_WAVE;
   const int col = lane & 15, kq = lane >> 4;
-  const int n0 = blockIdx.x * 16 * NTILE;
+  const int nt = q + ((int)blockIdx.x < rem ? 1 : 0);   // tiles of this block, at most NTILE
+  const int n0 = ((int)blockIdx.x * q + min((int)blockIdx.x, rem)) * 16;
   const int m0 = blockIdx.y * 16 * MT;   // token groups beyond MT per block go to further blocks along y
   const int total_steps = (K + 31) / 32;
 
@@ -58,7 +67,7 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
   f32x4 bv[NTILE];        // bias of this lane's 4 features per tile
 #pragma unroll
   for (int u = 0; u < NTILE; ++u) {
-    const int nb = n0 + u * 16 + kq * 4;
+    const int nb = u < nt ? n0 + u * 16 + kq * 4 : N;   // N: nothing of this tile is this block's
     bv[u] = f32x4{0.f, 0.f, 0.f, 0.f};
     if (bias && EPI != EPI_SWIGLU) {
 #pragma unroll
@@ -93,7 +102,7 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
 #pragma unroll
     for (int u = 0; u < NTILE; ++u) {
       wv[u] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-      if (in) wv[u] = *reinterpret_cast<const bf16x8*>(wrow[u] + k);
+      if (in && u < nt) wv[u] = *reinterpret_cast<const bf16x8*>(wrow[u] + k);
     }
     f32x4 nw0 = {0.f, 0.f, 0.f, 0.f}, nw1 = {0.f, 0.f, 0.f, 0.f};
     if (NORM && in) {
@@ -119,7 +128,8 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
         if (in) av = *reinterpret_cast<const bf16x8*>(A + arow[t] + k);
       }
 #pragma unroll
-      for (int u = 0; u < NTILE; ++u) acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[u], av, acc[u][t], 0, 0, 0);
+      for (int u = 0; u < NTILE; ++u)
+        if (u < nt) acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[u], av, acc[u][t], 0, 0, 0);
     }
   }
 
@@ -137,7 +147,7 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
       const int item = u * MT + t, owner = item % WAVES;
-      if (wave != owner) red[wave < owner ? wave : wave - 1][item][lane] = acc[u][t];
+      if (wave != owner && u < nt) red[wave < owner ? wave : wave - 1][item][lane] = acc[u][t];
     }
   __syncthreads();
 
@@ -146,7 +156,7 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
       const int item = u * MT + t, owner = item % WAVES;
-      if (wave != owner) continue;
+      if (wave != owner || u >= nt) continue;
       // sum in wave order: the waves below the owner, the owner itself, the waves above
       f32x4 sum = {0.f, 0.f, 0.f, 0.f};
       for (int w = 0; w < WAVES; ++w) sum += w == owner ? acc[u][t] : red[w < owner ? w : w - 1][item][lane];
@@ -166,7 +176,7 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
         for (int p = 0; p < 2; ++p) {
           if (nb + 2 * p + 1 < N) {
             const float g = sum[2 * p], up = sum[2 * p + 1];
-            out[(size_t)m * ldo + nb / 2 + p] = from_float<TO>(g / (1.0f + expf(-g)) * up);
+            out[(size_t)m * ldo + nb / 2 + p] = from_float<TO>(fast_silu(g) * up);
           }
         }
       } else {
@@ -185,20 +195,39 @@ int g_force_ntile = 0, g_force_waves = 0, g_force_mt = 0;
 // The shapes of block on offer: (tiles per block, waves).  LDS holds (waves - 1) * tiles * MT KB.
 // (Splitting K over blocks as well, with the last block to arrive adding the partial sums, was measured and
 // dropped: the device-scope fences it needs cost several microseconds per block on this chip.)
+inline bool forced() { return g_force_ntile || g_force_waves || g_force_mt; }
+
+inline int compute_units() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) n = v;
+    else n = 256;
+  }
+  return n;
+}
+
 template <int MT, int EPI, typename TO, bool NORM>
 int launch_cfg(const void* A, size_t lda, const bf16* W, size_t ldw, const float* bias, TO* out, size_t ldo, int M,
                int N, int K, hipStream_t stream, const float* norm_w, float eps, const int* rows) {
   const int tiles = (N + 15) / 16;
   const int steps = (K + 31) / 32;
-  // as many tiles per block as still leaves a block for every CU; narrow outputs keep one tile per block
-  // (two when there are several token groups, whose activations would otherwise be read once per tile)
-  // (measured on the 0.5B shapes at 8 and 64 rows; with several token groups the wide shape pays earlier)
-  int ntile = tiles >= 512 ? 4 : 1;
-  int waves = ntile == 4 ? (MT <= 2 && (MT == 1 || tiles < 1024) ? 8 : 4) : ((steps >= 32 || MT > 1) ? 16 : 8);
-  if (g_force_ntile) { ntile = g_force_ntile; waves = g_force_waves; }
-  if ((waves - 1) * ntile * MT > 60) return MS_UNSUPPORTED;  // LDS
-#define GO(NT, WV) if (ntile == NT && waves == WV) { if constexpr ((WV - 1) * NT * MT <= 60) { gemm_skinny_kernel<MT, NT, WV, EPI, TO, NORM><<<dim3((tiles + NT - 1) / NT, (M + 16 * MT - 1) / (16 * MT)), dim3(WV * MS_WAVE), 0, stream>>>(A, lda, W, ldw, bias, out, ldo, M, N, K, norm_w, eps, rows); return ms_launch_status(); } }
-  GO(4, 4) GO(4, 8) GO(2, 8) GO(2, 16) GO(1, 8) GO(1, 16)
+  const int groups = (M + 16 * MT - 1) / (16 * MT);
+  const int cus = compute_units();
+  // Every CU should stream an equal share of the matrix: an output of up to four tiles per CU has them dealt
+  // out evenly over as many blocks as there are CUs; a narrower one has a block per tile, a wider one four
+  // tiles to a block.  (Measured on the 0.5B shapes at 8 and 64 rows.)
+  int ntile, blocks;
+  if (tiles <= cus) { ntile = 1; blocks = tiles; }
+  else if (tiles <= 4 * cus && groups == 1) { blocks = cus; ntile = (tiles + cus - 1) / cus; }
+  else { ntile = 4; blocks = (tiles + 3) / 4; }
+  int waves = ntile >= 3 ? (MT <= 2 && (MT == 1 || tiles < 1024) ? 8 : 4) : ((steps >= 32 || MT > 1) ? 16 : 8);
+  if (g_force_ntile) { ntile = g_force_ntile; waves = g_force_waves; blocks = (tiles + ntile - 1) / ntile; }
+  const int q = tiles / blocks, rem = tiles % blocks;   // blocks * q + rem tiles; q + (rem > 0) <= ntile
+  if (q + (rem ? 1 : 0) > ntile || (waves - 1) * ntile * MT > 60) return MS_UNSUPPORTED;  // LDS
+#define GO(NT, WV) if (ntile == NT && waves == WV) { if constexpr ((WV - 1) * NT * MT <= 60) { gemm_skinny_kernel<MT, NT, WV, EPI, TO, NORM><<<dim3(blocks, groups), dim3(WV * MS_WAVE), 0, stream>>>(A, lda, W, ldw, bias, out, ldo, M, N, K, norm_w, eps, rows, q, rem); return ms_launch_status(); } }
+  GO(4, 4) GO(4, 8) GO(3, 8) GO(2, 8) GO(2, 16) GO(1, 8) GO(1, 16)
 #undef GO
   return MS_UNSUPPORTED;
 }
@@ -218,9 +247,10 @@ int launch_mt(const void* A, size_t lda, const bf16* W, size_t ldw, const float*
 
 }  // namespace
 
-// Tuning knob for measurements: force the block shape (tiles per block, waves) out of (4,4) (4,8) (2,8) (2,16)
-// (1,8) (1,16), and the 16-token groups per block (1, 2 or 4; further groups go to further blocks), for every
-// later ms_gemm_skinny* launch; zeros give the choice back to the heuristic.
+// Tuning knob for measurements: force the block shape (tiles per block, waves) out of (4,4) (4,8) (3,8) (2,8)
+// (2,16) (1,8) (1,16), and the 16-token groups per block (1, 2 or 4; further groups go to further blocks), for
+// every later ms_gemm_skinny* launch; zeros give the choice back to the heuristic.  While anything is forced,
+// products of up to 16 rows stay in this kernel instead of going to ms_gemm_stream.
 extern "C" void ms_gemm_skinny_force(int ntile, int waves, int token_groups) {
   g_force_ntile = ntile;
   g_force_waves = waves;
@@ -234,6 +264,10 @@ extern "C" int ms_gemm_skinny(const void* A, long long lda, const void* W, long 
                               long long ldo, int M, int N, int K, int epilogue, int out_dtype, hipStream_t stream) {
   if (M <= 0 || N <= 0) return MS_OK;
   if (M > 64) return MS_UNSUPPORTED;
+  if (M <= 16 && !forced()) {   // one token group: the streaming kernel, where it takes the shape
+    const int rc = ms_gemm_stream(A, lda, nullptr, nullptr, 0.f, W, ldw, bias, out, ldo, M, N, K, epilogue, out_dtype, 0, 0, stream);
+    if (rc != MS_UNSUPPORTED) return rc;
+  }
   if (K <= 0 || K % 8 || lda % 8 || ldw % 8 || lda < K || ldw < K) return MS_UNSUPPORTED;
   if (((uintptr_t)A | (uintptr_t)W) % 16) return MS_UNSUPPORTED;
   const bf16* w = (const bf16*)W;
@@ -262,6 +296,10 @@ extern "C" int ms_gemm_skinny_norm(const float* x, long long ldx, const int* row
                                    int N, int K, int epilogue, int out_dtype, hipStream_t stream) {
   if (M <= 0 || N <= 0) return MS_OK;
   if (M > 64) return MS_UNSUPPORTED;
+  if (M <= 16 && !forced()) {
+    const int rc = ms_gemm_stream(x, ldx, rows, norm_w, eps, W, ldw, bias, out, ldo, M, N, K, epilogue, out_dtype, 1, 0, stream);
+    if (rc != MS_UNSUPPORTED) return rc;
+  }
   if (K <= 0 || K % 8 || ldx % 4 || ldw % 8 || ldx < K || ldw < K) return MS_UNSUPPORTED;
   if (((uintptr_t)x | (uintptr_t)W | (uintptr_t)norm_w) % 16) return MS_UNSUPPORTED;
   const bf16* w = (const bf16*)W;

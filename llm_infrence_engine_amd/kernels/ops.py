@@ -30,6 +30,8 @@ _SIGNATURES = {
     "ms_bias_add": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "ms_gemm_skinny": [_c_ptr, _c_ll, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int,
                        _c_ptr],
+    "ms_gemm_stream": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int,
+                       _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "ms_residual_add": [_c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr],
     "ms_silu_mul": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "ms_rope_store": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int,
@@ -329,6 +331,46 @@ def gemm_skinny_norm(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w: 
         raise ValueError(f"epilogue {epilogue} is not available with the folded norm")
     _call("ms_gemm_skinny_norm", x.data_ptr(), K, _ptr(rows), norm_weight.data_ptr(), float(eps), w.data_ptr(), K,
           _ptr(bias), out.data_ptr(), ldo, M, N, K, epilogue, _code(out_dtype), _stream())
+    return out
+
+
+STREAM_MAX_ROWS = 16
+
+
+def gemm_stream(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, epilogue: int = EPI_STORE,
+                out_dtype: torch.dtype = torch.bfloat16, residual: Optional[torch.Tensor] = None,
+                norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0,
+                rows: Optional[torch.Tensor] = None, any_shape: bool = True) -> torch.Tensor:
+    """The streaming kernel for up to 16 rows, called by name (``gemm_skinny`` and ``gemm_skinny_norm`` go to it by
+    themselves for the shapes it is faster on): ``a`` bfloat16 [M, K], or with ``norm_weight`` the float32
+    residual stream whose RMS norm is folded in.  With ``any_shape`` every shape it can compute is taken;
+    a shape it cannot raises."""
+    norm = norm_weight is not None
+    _check(a, "a", torch.float32 if norm else torch.bfloat16, contiguous=False)
+    _check(w, "w", torch.bfloat16)
+    if a.dim() != 2 or a.stride(1) != 1 or w.shape[1] != a.shape[1]:
+        raise ValueError(f"shapes do not fit: a {list(a.shape)} (stride {a.stride()}), w {list(w.shape)}")
+    K, N = a.shape[1], w.shape[0]
+    M = a.shape[0]
+    if rows is not None:
+        _check(rows, "rows", torch.int32)
+        M = rows.numel()
+    if norm:
+        _check(norm_weight, "norm_weight", torch.float32, (K,))
+    if bias is not None:
+        _check(bias, "bias", torch.float32, (N,))
+    if epilogue == EPI_STORE:
+        out, ldo = torch.empty((M, N), dtype=out_dtype, device=a.device), N
+    elif epilogue == EPI_SWIGLU:
+        out, ldo, out_dtype = torch.empty((M, N // 2), dtype=torch.bfloat16, device=a.device), N // 2, torch.bfloat16
+    elif epilogue == EPI_RESIDUAL:
+        _check(residual, "residual", torch.float32, (M, N))
+        out, ldo, out_dtype = residual, N, torch.float32
+    else:
+        raise ValueError(f"unknown epilogue {epilogue}")
+    _call("ms_gemm_stream", a.data_ptr(), a.stride(0) if a.shape[0] > 1 else K, _ptr(rows), _ptr(norm_weight), float(eps),
+          w.data_ptr(), K, _ptr(bias), out.data_ptr(), ldo, M, N, K, epilogue, _code(out_dtype), int(norm),
+          int(any_shape), _stream())
     return out
 
 

@@ -309,9 +309,12 @@ def test_gemm_skinny(ops, M, N, K):
 
 
 @pytest.mark.parametrize("M", [3, 40])
-@pytest.mark.parametrize("shape", [(4, 4, 0), (4, 8, 0), (2, 8, 0), (2, 16, 0), (1, 8, 0), (1, 16, 0), (4, 8, 1), (2, 8, 2)])
+@pytest.mark.parametrize("shape", [(4, 4, 0), (4, 8, 0), (3, 8, 0), (2, 8, 0), (2, 16, 0), (1, 8, 0), (1, 16, 0),
+                                   (4, 8, 1), (3, 8, 1), (2, 8, 2)])
 def test_gemm_skinny_block_shapes(ops, M, shape):
-    """Every block shape on offer gives the same numbers (to float rounding of another summation order)."""
+    """Every block shape on offer (tiles per block, waves, token groups per block) gives the same numbers (to
+    float rounding of another summation order), also with the gated epilogue and the folded norm.  A forced
+    shape also keeps few rows in this kernel; unforced they go to the streaming kernel, which must agree."""
     from llm_infrence_engine_amd.kernels import build
 
     lib = build.load()
@@ -333,8 +336,62 @@ def test_gemm_skinny_block_shapes(ops, M, shape):
         torch.testing.assert_close(x.double(), x0.double() + want, atol=3e-5, rtol=3e-5)
         f = ops.gemm_skinny(a, w, bias, out_dtype=torch.float32)
         torch.testing.assert_close(f.double(), want, atol=3e-5, rtol=3e-5)
+        # gated epilogue over interleaved rows, norm folded in: against the default shape
+        x32 = torch.randn(M, K, generator=g).to(DEV)
+        nw = (1 + 0.1 * torch.randn(K, generator=g)).to(DEV)
+        got = ops.gemm_skinny_norm(x32, nw, 1e-6, w, None, ops.EPI_SWIGLU)
+        lib.ms_gemm_skinny_force(0, 0, 0)
+        ref = ops.gemm_skinny_norm(x32, nw, 1e-6, w, None, ops.EPI_SWIGLU)
+        torch.testing.assert_close(got.double(), ref.double(), atol=1e-2, rtol=1e-2)
     finally:
         lib.ms_gemm_skinny_force(0, 0, 0)
+
+
+@pytest.mark.parametrize("M", [1, 5, 8, 16])
+@pytest.mark.parametrize("N,K", [(896, 4864), (1152, 896), (330, 72), (52, 200), (9728, 904), (1000, 9000), (4000, 2056),
+                                 (16384, 64)])
+def test_gemm_stream(ops, M, N, K):
+    """The streaming kernel at every shape it can compute: one or several stages, a last k-step that K fills in
+    part, one to four tiles of rows to a block, rows that run out in the last block; every epilogue, the folded
+    norm with gathered rows; a row's numbers do not depend on the rest of the batch."""
+    g = torch.Generator().manual_seed(M * 1000 + N + K)
+    a = torch.randn(M, K, generator=g).bfloat16().to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16().to(DEV)
+    bias = torch.randn(N, generator=g).to(DEV)
+    want = a.double() @ w.double().T
+    out = ops.gemm_stream(a, w, bias)
+    torch.testing.assert_close(out.double(), want + bias.double(), **tol(torch.bfloat16))
+    f = ops.gemm_stream(a, w, None, out_dtype=torch.float32)
+    torch.testing.assert_close(f.double(), want, atol=3e-5, rtol=3e-5)
+    x = torch.randn(M, N, generator=g).to(DEV)
+    x0 = x.clone()
+    ops.gemm_stream(a, w, bias, ops.EPI_RESIDUAL, residual=x)
+    torch.testing.assert_close(x.double(), x0.double() + want + bias.double(), atol=3e-5, rtol=3e-5)
+    act = ops.gemm_stream(a, w, None, ops.EPI_SWIGLU)
+    torch.testing.assert_close(act.double(), torch.nn.functional.silu(want[:, 0::2]) * want[:, 1::2], **tol(torch.bfloat16))
+    assert torch.equal(ops.gemm_stream(a[M - 1:], w, bias), out[M - 1:])
+    # the folded norm over gathered rows of a taller residual stream
+    xs = torch.randn(M + 3, K, generator=g).to(DEV)
+    nw = (1 + 0.1 * torch.randn(K, generator=g)).to(DEV)
+    rows = torch.randperm(M + 3, generator=g)[:M].to(torch.int32).to(DEV)
+    xr = xs[rows.long()].double()
+    h = (xr * nw.double()).float().bfloat16().double() * torch.rsqrt((xr * xr).mean(-1, keepdim=True) + 1e-5)
+    got = ops.gemm_stream(xs, w, bias, out_dtype=torch.float32, norm_weight=nw, eps=1e-5, rows=rows)
+    torch.testing.assert_close(got.double(), h @ w.double().T + bias.double(), atol=2e-4, rtol=2e-4)
+    gated = ops.gemm_stream(xs, w, None, ops.EPI_SWIGLU, norm_weight=nw, eps=1e-5, rows=rows)
+    hw = h @ w.double().T
+    torch.testing.assert_close(gated.double(), torch.nn.functional.silu(hw[:, 0::2]) * hw[:, 1::2], **tol(torch.bfloat16))
+
+
+def test_gemm_stream_refuses_what_it_cannot_take(ops):
+    w = torch.zeros(64, 64, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(RuntimeError, match="unsupported"):
+        ops.gemm_stream(torch.zeros(17, 64, dtype=torch.bfloat16, device=DEV), w)            # more than 16 rows
+    with pytest.raises(RuntimeError, match="unsupported"):
+        ops.gemm_stream(torch.zeros(2, 36, dtype=torch.bfloat16, device=DEV),
+                        torch.zeros(8, 36, dtype=torch.bfloat16, device=DEV))                 # K no multiple of 8
+    with pytest.raises(RuntimeError, match="unsupported"):                                   # not the shape it is for
+        ops.gemm_stream(torch.zeros(2, 64, dtype=torch.bfloat16, device=DEV), w, any_shape=False)
 
 
 def test_gemm_skinny_refuses_what_it_cannot_take(ops):
