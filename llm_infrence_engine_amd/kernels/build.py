@@ -3,12 +3,15 @@
 ``build()`` always compiles.  ``load()`` takes the library that is there and compiles only when there
 is none, printing a line per file so that a first call in a fresh checkout shows progress.  The
 library sits beside this file; when that folder cannot be written (a read-only checkout) it goes to a
-per-user folder under the system's temporary directory instead.  There is no fallback: without the
-library every op raises.
+folder under the system's temporary directory instead, named for the user and for the sources' contents, so
+that a library built from other sources is never picked up there.  Beside the library lies a stamp with the
+hash of the sources it was built from; ``load()`` says so on stderr when the stamp and the sources differ.
+There is no fallback: without the library every op raises.
 """
 from __future__ import annotations
 
 import ctypes
+import hashlib
 import os
 import shutil
 import subprocess
@@ -53,8 +56,22 @@ def _writable(d: Path) -> bool:
         return False
 
 
+def source_hash() -> str:
+    """A short hash of everything the library is compiled from."""
+    h = hashlib.sha256()
+    for f in sorted(list(CSRC.glob("*.hip")) + list(CSRC.glob("*.h"))):
+        h.update(f.name.encode())
+        h.update(f.read_bytes())
+    h.update(" ".join(FLAGS).encode())
+    return h.hexdigest()[:12]
+
+
 def _fallback_dir() -> Path:
-    return Path(tempfile.gettempdir()) / f"llm_infrence_engine_amd-{os.getuid()}"
+    return Path(tempfile.gettempdir()) / f"llm_infrence_engine_amd-{os.getuid()}-{source_hash()}"
+
+
+def _stamp_of(lib: Path) -> Path:
+    return lib.with_suffix(".stamp")
 
 
 def library_path() -> Path | None:
@@ -109,6 +126,7 @@ def build(verbose: bool = True) -> Path:
     if r.returncode != 0:
         raise KernelLibraryError(f"linking {LIB_NAME} failed:\n{r.stdout}\n{r.stderr}")
     os.replace(tmp, out_dir / LIB_NAME)
+    _stamp_of(out_dir / LIB_NAME).write_text(source_hash() + "\n")
     say(f"linked {out_dir / LIB_NAME}")
     global _lib
     _lib = None
@@ -125,6 +143,12 @@ def load() -> ctypes.CDLL:
     path = library_path()
     if path is None:
         path = build(verbose=True)
+    else:
+        stamp = _stamp_of(path)
+        built_from = stamp.read_text().strip() if stamp.is_file() else "unknown sources"
+        if built_from != source_hash():
+            print(f"[kernels] {path} was built from {built_from}, the sources under {CSRC} are {source_hash()}: "
+                  f"build it again (llm_infrence_engine_amd.kernels.build.build())", file=sys.stderr, flush=True)
     try:
         _lib = ctypes.CDLL(str(path))
     except OSError as e:
