@@ -46,7 +46,7 @@ struct KeyBlock {          // one block of 32 keys as this lane sees it
 };
 template <int D>
 struct ValueBlock {        // and its values
-  bf16x4 v[D / 16][2];     // [16-dim tile][subtile]: 4 keys of one dim
+  bf16x4 v[D / 16][2];     // [16-dim tile][subtile]: 4 keys of one dim; the two subtiles are one MFMA operand
 };
 
 // Page arithmetic: pages of a power of two (page_shift >= 0) need no division.
@@ -241,18 +241,24 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
 
     const bool unmasked = full_tile && base + 31 <= first_pos && (window <= 0 || base > key_hi - window);
     bf16x8 p[NT];
-    float corr[NT];
+    float corr[NT], bmax[NT];
     bool moved = false;
+    // the block's maxima of the raw scores (the scale is positive, so they are the maxima of the scaled ones
+    // too); one branch for the whole tile, so that what follows is straight-line code for all its columns
+    if (unmasked) {
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
-      // the block's maximum of the raw scores (the scale is positive, so it is the maximum of the scaled ones too)
-      float bm = -INFINITY;
-      if (unmasked) {
+      for (int t = 0; t < NT; ++t) {
+        float bm = -INFINITY;
 #pragma unroll
         for (int u = 0; u < 2; ++u)
 #pragma unroll
           for (int i = 0; i < 4; ++i) bm = fmaxf(bm, s[u][t][i]);
-      } else {
+        bmax[t] = bm;
+      }
+    } else {
+#pragma unroll
+      for (int t = 0; t < NT; ++t) {
+        float bm = -INFINITY;
 #pragma unroll
         for (int u = 0; u < 2; ++u)
 #pragma unroll
@@ -263,7 +269,13 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
             s[u][t][i] = v;
             bm = fmaxf(bm, v);
           }
+        bmax[t] = bm;
       }
+    }
+    float m_safe[NT];
+#pragma unroll
+    for (int t = 0; t < NT; ++t) {
+      float bm = bmax[t];
       bm = fmaxf(bm, __shfl_xor(bm, 16, MS_WAVE));
       bm = fmaxf(bm, __shfl_xor(bm, 32, MS_WAVE));
       bm *= scale_log2e;
@@ -276,17 +288,7 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
       corr[t] = step ? fast_exp2(m[t] - m_new) : 1.0f;   // m = -inf: 0
       moved |= step;
       m[t] = m_new;
-      const float m_safe = m_new == -INFINITY ? 0.f : m_new;
-      float ls = 0.f;
-#pragma unroll
-      for (int u = 0; u < 2; ++u)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float e = fast_exp2(fmaf(s[u][t][i], scale_log2e, -m_safe));
-          ls += e;
-          p[t][u * 4 + i] = (__bf16)e;
-        }
-      l[t] = l[t] * corr[t] + ls;
+      m_safe[t] = m_new == -INFINITY ? 0.f : m_new;
     }
     if (NT == 1 || __builtin_amdgcn_ballot_w64(moved) != 0) {   // the same branch for the whole wave
 #pragma unroll
@@ -294,14 +296,27 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
 #pragma unroll
         for (int c = 0; c < D / 16; ++c) o[c][t] *= corr[t];
     }
-
+    // column by column, so that the products of one column run on the matrix cores while the next column's
+    // exponentials are taken
 #pragma unroll
-    for (int c = 0; c < D / 16; ++c) {
-      bf16x8 vv;
+    for (int t = 0; t < NT; ++t) {
+      float ls = 0.f;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) { vv[i] = cur_v.v[c][0][i]; vv[4 + i] = cur_v.v[c][1][i]; }
+      for (int u = 0; u < 2; ++u)
 #pragma unroll
-      for (int t = 0; t < NT; ++t) o[c][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, p[t], o[c][t], 0, 0, 0);
+        for (int i = 0; i < 4; ++i) {
+          const float e = fast_exp2(fmaf(s[u][t][i], scale_log2e, -m_safe[t]));
+          ls += e;
+          p[t][u * 4 + i] = (__bf16)e;
+        }
+      l[t] = l[t] * corr[t] + ls;
+#pragma unroll
+      for (int c = 0; c < D / 16; ++c) {
+        bf16x8 vv;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { vv[i] = cur_v.v[c][0][i]; vv[4 + i] = cur_v.v[c][1][i]; }
+        o[c][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, p[t], o[c][t], 0, 0, 0);
+      }
     }
     if (blk + WAVES < blk_end) {
       cur_k = nxt_k;
@@ -467,7 +482,7 @@ extern "C" int ms_paged_attention_mfma(const void* q, long long q_stride, const 
   int waves = nt > 1 ? 4 : (head_dim == 128 ? 8 : 16);
   if (g_force_nt) { nt = g_force_nt; waves = g_force_waves; }
 #define PICK(D, NT, WV) if (head_dim == D && nt == NT && waves == WV) GO(D, NT, WV)
-  PICK(32, 4, 4); PICK(32, 4, 8); PICK(32, 2, 4); PICK(32, 2, 8); PICK(32, 1, 8); PICK(32, 1, 16);
+  PICK(32, 4, 4); PICK(32, 2, 4); PICK(32, 2, 8); PICK(32, 1, 8); PICK(32, 1, 16);
   PICK(64, 4, 4); PICK(64, 2, 4); PICK(64, 2, 8); PICK(64, 1, 4); PICK(64, 1, 8); PICK(64, 1, 16);
   PICK(128, 2, 4); PICK(128, 1, 4); PICK(128, 1, 8);
 #undef PICK
