@@ -46,6 +46,24 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
   return t;
 }
 
+// g * sigmoid(g) through the hardware's exp2 and reciprocal (each good to about one unit in the last place of
+// a float; the callers round the result to bfloat16)
+__device__ __forceinline__ float fast_silu(float g) {
+  return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g));
+}
+
+// Compute units of the current device (256 on an MI355X); asked once.
+static inline int ms_compute_units() {
+  static int n = 0;
+  if (n == 0) {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) n = v;
+    else n = 256;
+  }
+  return n;
+}
+
 static inline int ms_launch_status() {
   return hipGetLastError() == hipSuccess ? MS_OK : MS_LAUNCH_FAILED;
 }

@@ -26,12 +26,6 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 enum { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_RESIDUAL = 3 };
 
-// g * sigmoid(g) through the hardware's exp2 and reciprocal (each good to about one unit in the last place of
-// a float; the result is rounded to bfloat16)
-__device__ __forceinline__ float fast_silu(float g) {
-  return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g));
-}
-
 // The tiles are dealt out evenly: the first `rem` blocks take q + 1 tiles, the others q (at most NTILE), so that
 // every CU streams about the same share of W.
 template <int MT, int NTILE, int WAVES, int EPI, typename TO, bool NORM>
@@ -197,24 +191,13 @@ int g_force_ntile = 0, g_force_waves = 0, g_force_mt = 0;
 // dropped: the device-scope fences it needs cost several microseconds per block on this chip.)
 inline bool forced() { return g_force_ntile || g_force_waves || g_force_mt; }
 
-inline int compute_units() {
-  static int n = 0;
-  if (n == 0) {
-    int dev = 0, v = 0;
-    if (hipGetDevice(&dev) == hipSuccess &&
-        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) n = v;
-    else n = 256;
-  }
-  return n;
-}
-
 template <int MT, int EPI, typename TO, bool NORM>
 int launch_cfg(const void* A, size_t lda, const bf16* W, size_t ldw, const float* bias, TO* out, size_t ldo, int M,
                int N, int K, hipStream_t stream, const float* norm_w, float eps, const int* rows) {
   const int tiles = (N + 15) / 16;
   const int steps = (K + 31) / 32;
   const int groups = (M + 16 * MT - 1) / (16 * MT);
-  const int cus = compute_units();
+  const int cus = ms_compute_units();
   // Every CU should stream an equal share of the matrix: an output of up to four tiles per CU has them dealt
   // out evenly over as many blocks as there are CUs; a narrower one has a block per tile, a wider one four
   // tiles to a block.  (Measured on the 0.5B shapes at 8 and 64 rows.)

@@ -31,12 +31,6 @@ typedef __attribute__((ext_vector_type(4))) unsigned u32x4;   // a 16-byte piece
 
 enum { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_RESIDUAL = 3 };
 
-// g * sigmoid(g) through the hardware's exp2 and reciprocal (each good to about one unit in the last place of
-// a float; the result is rounded to bfloat16)
-__device__ __forceinline__ float fast_silu(float g) {
-  return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g));
-}
-
 constexpr int WAVES = 16;     // waves of a block
 constexpr int WI_MAX = 6;     // weight loads a wave has in flight per stage (WAVES * WI_MAX KB of W per stage)
 constexpr int XI_BF16 = 6;    // activation loads a wave has in flight per stage: bfloat16 rows (16 bytes a lane),
@@ -250,17 +244,6 @@ gemm_stream_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
   }
 }
 
-inline int compute_units() {
-  static int n = 0;
-  if (n == 0) {
-    int dev = 0, v = 0;
-    if (hipGetDevice(&dev) == hipSuccess &&
-        hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0) n = v;
-    else n = 256;
-  }
-  return n;
-}
-
 constexpr int LDS_BUDGET = 120 * 1024;   // of the CU's 160 KB, for the stage buffers
 
 template <int NT, int EPI, typename TO, bool NORM>
@@ -282,7 +265,7 @@ int launch(const void* A, size_t lda, const bf16* W, size_t ldw, const float* bi
 template <int EPI, typename TO, bool NORM>
 int plan(const void* A, size_t lda, const bf16* W, size_t ldw, const float* bias, TO* out, size_t ldo, int M, int N,
          int K, const float* norm_w, float eps, const int* rows, bool any_shape, hipStream_t stream) {
-  const int cus = compute_units();
+  const int cus = ms_compute_units();
   const int units = (N + 3) / 4;
   // Where this kernel wins, by measurement against ms_gemm_skinny (which costs less to set up and has no LDS
   // stage between the loads and the matrix cores): few rows of W per CU and many columns, at up to 8 tokens:
