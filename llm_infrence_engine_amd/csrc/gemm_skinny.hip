@@ -56,7 +56,17 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
     arow[t] = (size_t)(rows ? rows[m] : m) * lda + kq * 8;  // rows: the activations are gathered rows of A
   }
 
-  // what the epilogue will need from memory is asked for now, so that it arrives under the main loop
+  f32x4 acc[NTILE][MT];
+  float ss[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    ss[t] = 0.f;
+#pragma unroll
+    for (int u = 0; u < NTILE; ++u) acc[u][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  // What the epilogue will need from memory is asked for now, so that it arrives under the main loop (after
+  // the row addresses above, which may themselves wait for a load: these must not wait behind it).
   f32x4 pre[NTILE][MT];   // the residual values this wave will add to (EPI_RESIDUAL)
   f32x4 bv[NTILE];        // bias of this lane's 4 features per tile
 #pragma unroll
@@ -78,17 +88,9 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
     }
   }
 
-  f32x4 acc[NTILE][MT];
-  float ss[MT];
-#pragma unroll
-  for (int t = 0; t < MT; ++t) {
-    ss[t] = 0.f;
-#pragma unroll
-    for (int u = 0; u < NTILE; ++u) acc[u][t] = f32x4{0.f, 0.f, 0.f, 0.f};
-  }
-
-  // the loads of several steps are in flight together: the kernel lives on memory parallelism
-#pragma unroll (MT * NTILE <= 2 ? 8 : 4)
+  // A wave has one step's loads in flight; the memory parallelism comes from the 8 or 16 waves of a block.
+  // (Issuing the loads of several steps before the first is used was measured and did not help: a CU pulls
+  // 25 to 43 GB/s however many loads it has in flight.)
   for (int s = wave; s < total_steps; s += WAVES) {
     const int k = s * 32;
     const bool in = k + kq * 8 < K;  // K is a multiple of 8: a lane's 8 values are all inside or all outside

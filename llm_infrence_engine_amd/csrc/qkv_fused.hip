@@ -79,7 +79,6 @@ qkv_rope_store_kernel(const float* __restrict__ X, size_t ldx, const float* __re
 #pragma unroll
   for (int t = 0; t < MT; ++t) { lo[t] = hi[t] = f32x4{0.f, 0.f, 0.f, 0.f}; ss[t] = 0.f; }
 
-#pragma unroll (MT == 1 ? 4 : 2)
   for (int s = wave; s < total_steps; s += WAVES) {
     const int k = s * 32;
     const bool in = k + kq * 8 < K;
