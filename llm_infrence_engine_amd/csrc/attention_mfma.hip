@@ -389,12 +389,18 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
   }
 }
 
-// out[r, h, :] = sum_s 2^(m_s - M) O_s / sum_s 2^(m_s - M) l_s over the splits that request r used
+// out[r, h, :] = sum_s 2^(m_s - M) O_s / sum_s 2^(m_s - M) l_s over the splits that request r used.
+// One block per (request, head): the splits' maxima and sums are fetched side by side (a thread each), the
+// weights are worked out once into LDS, then a thread per dim adds the weighted partial results in split order.
+constexpr int COMBINE_MAX_SPLITS = 64;
+
 template <int D>
-__global__ void attention_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                         const int* __restrict__ q_start, const int* __restrict__ context_lens,
-                                         bf16* __restrict__ out, size_t out_stride, int nh, int window,
-                                         int min_blocks, int n_splits) {
+__global__ void __launch_bounds__(D < 64 ? 64 : D)
+attention_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                         const int* __restrict__ q_start, const int* __restrict__ context_lens,
+                         bf16* __restrict__ out, size_t out_stride, int nh, int window, int min_blocks,
+                         int n_splits) {
+  __shared__ float sm_m[COMBINE_MAX_SPLITS], sm_w[COMBINE_MAX_SPLITS];
   const int r = blockIdx.x / nh, h = blockIdx.x % nh;
   const int key_hi = context_lens[r] - 1;
   const int key_lo = window > 0 ? max(0, key_hi - window + 1) : 0;
@@ -402,15 +408,28 @@ __global__ void attention_combine_kernel(const float* __restrict__ part_o, const
   const int per = max(min_blocks, (blocks + n_splits - 1) / n_splits);
   const int used = (blocks + per - 1) / per;
   const size_t slot0 = ((size_t)r * nh + h) * n_splits;
+  const int t = threadIdx.x;
+  float l_mine = 0.f;
+  if (t < used) {
+    sm_m[t] = part_ml[(slot0 + t) * 2];
+    l_mine = part_ml[(slot0 + t) * 2 + 1];
+  }
+  __syncthreads();
   float big = -INFINITY;
-  for (int s = 0; s < used; ++s) big = fmaxf(big, part_ml[(slot0 + s) * 2]);
+  for (int s = 0; s < used; ++s) big = fmaxf(big, sm_m[s]);
+  if (t < used) sm_w[t] = fast_exp2(sm_m[t] - big);
+  __syncthreads();
+  // the denominator in split order; sm_m now carries the splits' sums
+  if (t < used) sm_m[t] = sm_w[t] * l_mine;
+  __syncthreads();
   float den = 0.f;
-  for (int s = 0; s < used; ++s) den += fast_exp2(part_ml[(slot0 + s) * 2] - big) * part_ml[(slot0 + s) * 2 + 1];
+  for (int s = 0; s < used; ++s) den += sm_m[s];
   const float inv = 1.0f / den;
   bf16* op = out + (size_t)q_start[r] * out_stride + (size_t)h * D;
-  for (int d = threadIdx.x; d < D; d += blockDim.x) {
+  for (int d = t; d < D; d += blockDim.x) {
     float acc = 0.f;
-    for (int s = 0; s < used; ++s) acc += fast_exp2(part_ml[(slot0 + s) * 2] - big) * part_o[(slot0 + s) * D + d];
+#pragma unroll 8
+    for (int s = 0; s < used; ++s) acc += sm_w[s] * part_o[(slot0 + s) * D + d];
     op[d] = __float2bfloat16(acc * inv);
   }
 }
@@ -507,7 +526,7 @@ extern "C" int ms_paged_attention_mfma_decode(const void* q, long long q_stride,
   if (num_heads / num_kv_heads > 16) return MS_UNSUPPORTED;
   if (!(scale > 0.f)) return MS_BAD_ARG;
   if (!ms_attention_mfma_supported(head_dim, page_size)) return MS_UNSUPPORTED;
-  if (min_blocks <= 0 || n_splits <= 0 || n_splits > 65535) return MS_BAD_ARG;
+  if (min_blocks <= 0 || n_splits <= 0 || n_splits > COMBINE_MAX_SPLITS) return MS_BAD_ARG;
   if (q_stride % 8 || out_stride % 4 || ((uintptr_t)q % 16) || ((uintptr_t)out % 8) || ((uintptr_t)part_o % 16)) return MS_UNSUPPORTED;
   if (n_requests > 65535 || num_kv_heads > 65535) return MS_UNSUPPORTED;
 #define GO(D) return launch_split<D>((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)vt_pages, block_table, table_stride, q_start, context_lens, (bf16*)out, out_stride, (float*)part_o, (float*)part_ml, n_requests, num_heads, num_kv_heads, page_size, scale, window, min_blocks, n_splits, stream)
