@@ -200,19 +200,22 @@ int launch_cfg(const void* A, size_t lda, const bf16* W, size_t ldw, const float
   const int steps = (K + 31) / 32;
   const int groups = (M + 16 * MT - 1) / (16 * MT);
   const int cus = ms_compute_units();
-  // Every CU should stream an equal share of the matrix: an output of up to four tiles per CU has them dealt
-  // out evenly over as many blocks as there are CUs; a narrower one has a block per tile, a wider one four
-  // tiles to a block.  (Measured on the 0.5B shapes at 8 and 64 rows.)
+  // Every CU should stream an equal share of the matrix: the tiles are dealt out evenly over a whole number of
+  // blocks per CU, of up to four tiles each (no last round that only some CUs take part in); an output with
+  // fewer tiles than CUs has a block per tile; with several token groups four tiles go to a block.
+  // (Measured on the 0.5B shapes at 8 and 64 rows and on the 7B shapes at 8.)
   int ntile, blocks;
   if (tiles <= cus) { ntile = 1; blocks = tiles; }
-  else if (tiles <= 4 * cus && groups == 1) { blocks = cus; ntile = (tiles + cus - 1) / cus; }
-  else { ntile = 4; blocks = (tiles + 3) / 4; }
+  else if (groups == 1) {   // a whole number of blocks per CU, of up to four tiles each
+    blocks = cus * ((tiles + 4 * cus - 1) / (4 * cus));
+    ntile = (tiles + blocks - 1) / blocks;
+  } else { ntile = 4; blocks = (tiles + 3) / 4; }
   int waves = ntile >= 3 ? (MT <= 2 && (MT == 1 || tiles < 1024) ? 8 : 4) : ((steps >= 32 || MT > 1) ? 16 : 8);
   if (g_force_ntile) { ntile = g_force_ntile; waves = g_force_waves; blocks = (tiles + ntile - 1) / ntile; }
   const int q = tiles / blocks, rem = tiles % blocks;   // blocks * q + rem tiles; q + (rem > 0) <= ntile
   if (q + (rem ? 1 : 0) > ntile || (waves - 1) * ntile * MT > 60) return MS_UNSUPPORTED;  // LDS
 #define GO(NT, WV) if (ntile == NT && waves == WV) { if constexpr ((WV - 1) * NT * MT <= 60) { gemm_skinny_kernel<MT, NT, WV, EPI, TO, NORM><<<dim3(blocks, groups), dim3(WV * MS_WAVE), 0, stream>>>(A, lda, W, ldw, bias, out, ldo, M, N, K, norm_w, eps, rows, q, rem); return ms_launch_status(); } }
-  GO(4, 4) GO(4, 8) GO(3, 8) GO(2, 8) GO(2, 16) GO(1, 8) GO(1, 16)
+  GO(4, 4) GO(4, 8) GO(3, 4) GO(3, 8) GO(2, 8) GO(2, 16) GO(1, 8) GO(1, 16)
 #undef GO
   return MS_UNSUPPORTED;
 }
@@ -232,7 +235,7 @@ int launch_mt(const void* A, size_t lda, const bf16* W, size_t ldw, const float*
 
 }  // namespace
 
-// Tuning knob for measurements: force the block shape (tiles per block, waves) out of (4,4) (4,8) (3,8) (2,8)
+// Tuning knob for measurements: force the block shape (tiles per block, waves) out of (4,4) (4,8) (3,4) (3,8) (2,8)
 // (2,16) (1,8) (1,16), and the 16-token groups per block (1, 2 or 4; further groups go to further blocks), for
 // every later ms_gemm_skinny* launch; zeros give the choice back to the heuristic.  While anything is forced,
 // products of up to 16 rows stay in this kernel instead of going to ms_gemm_stream.

@@ -309,7 +309,7 @@ def test_gemm_skinny(ops, M, N, K):
 
 
 @pytest.mark.parametrize("M", [3, 40])
-@pytest.mark.parametrize("shape", [(4, 4, 0), (4, 8, 0), (3, 8, 0), (2, 8, 0), (2, 16, 0), (1, 8, 0), (1, 16, 0),
+@pytest.mark.parametrize("shape", [(4, 4, 0), (4, 8, 0), (3, 4, 0), (3, 8, 0), (2, 8, 0), (2, 16, 0), (1, 8, 0), (1, 16, 0),
                                    (4, 8, 1), (3, 8, 1), (2, 8, 2)])
 def test_gemm_skinny_block_shapes(ops, M, shape):
     """Every block shape on offer (tiles per block, waves, token groups per block) gives the same numbers (to
