@@ -31,6 +31,12 @@ typedef __attribute__((ext_vector_type(4))) unsigned u32x4;   // a 16-byte piece
 
 enum { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_RESIDUAL = 3 };
 
+// id / parts for the small numbers that occur here (id < 4096, parts <= 16) by a multiplication: dividing by a
+// run-time value costs some twenty instructions even when both are the same for the whole wave, and the item
+// arithmetic below would do it two dozen times before the first load is issued.
+__device__ __forceinline__ int small_inverse(int parts) { return (65536 + parts - 1) / parts; }
+__device__ __forceinline__ int small_div(int id, int inverse) { return (id * inverse) >> 16; }
+
 constexpr int WAVES = 16;     // waves of a block
 constexpr int WI_MAX = 6;     // weight loads a wave has in flight per stage (WAVES * WI_MAX KB of W per stage)
 constexpr int XI_BF16 = 6;    // activation loads a wave has in flight per stage: bfloat16 rows (16 bytes a lane),
@@ -58,6 +64,7 @@ gemm_stream_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
   const int C8cap = min(KC, (K + 31) / 32 * 32) / 8;   // pieces per row of a full stage
   const int pitch = C8cap + 1;                          // odd, so that 16 rows read at one column hit 16 banks
   const int parts = (C8cap + 63) / 64;                  // loads per row and stage
+  const int parts_inv = small_inverse(parts);
   u32x4* wst = smem;
   u32x4* xst = smem + (size_t)rcap * pitch;
 
@@ -84,7 +91,7 @@ gemm_stream_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
 #pragma unroll
   for (int j = 0; j < XI_MAX; ++j) {
     const int id = wave + j * WAVES;
-    xtok[j] = id / parts;
+    xtok[j] = small_div(id, parts_inv);
     xpart[j] = id - xtok[j] * parts;
     if (xtok[j] >= M) xtok[j] = -1;
     xoff[j] = xtok[j] < 0 ? 0 : (size_t)(rows ? rows[xtok[j]] : xtok[j]) * lda;
@@ -99,12 +106,13 @@ gemm_stream_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
   // global -> registers for the stage that starts at column k0 and has S8 pieces per row
   auto issue = [&](int k0, int S8) {
     const int parts_s = (S8 + 63) / 64;
+    const int inv_s = parts_s == parts ? parts_inv : small_inverse(parts_s);
     // the weights first: they come from HBM, the activations from L2
 #pragma unroll
     for (int j = 0; j < WI_MAX; ++j) {
       const int id = wave + j * WAVES;
       if (id >= R * parts_s) break;   // the same for the whole wave
-      const int row = id / parts_s, c = (id - row * parts_s) * 64 + lane;
+      const int row = small_div(id, inv_s), c = (id - row * parts_s) * 64 + lane;
       wreg[j] = *reinterpret_cast<const u32x4*>(W + (size_t)min(r0 + row, N - 1) * ldw + k0 + (size_t)min(c, S8 - 1) * 8);
     }
 #pragma unroll
@@ -127,6 +135,7 @@ gemm_stream_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
   // registers -> LDS
   auto commit = [&](int S8) {
     const int parts_s = (S8 + 63) / 64;
+    const int inv_s = parts_s == parts ? parts_inv : small_inverse(parts_s);
 #pragma unroll
     for (int j = 0; j < XI_MAX; ++j) {
       const int c = xpart[j] * 64 + lane;
@@ -152,7 +161,7 @@ gemm_stream_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
     for (int j = 0; j < WI_MAX; ++j) {
       const int id = wave + j * WAVES;
       if (id >= R * parts_s) break;
-      const int row = id / parts_s, c = (id - row * parts_s) * 64 + lane;
+      const int row = small_div(id, inv_s), c = (id - row * parts_s) * 64 + lane;
       if (c < S8) wst[row * pitch + c] = wreg[j];
     }
     // a last k-step that K fills only in part reads zeros for the rest
@@ -268,11 +277,11 @@ int plan(const void* A, size_t lda, const bf16* W, size_t ldw, const float* bias
   const int cus = ms_compute_units();
   const int units = (N + 3) / 4;
   // Where this kernel wins, by measurement against ms_gemm_skinny (which costs less to set up and has no LDS
-  // stage between the loads and the matrix cores): few rows of W per CU and many columns, at up to 8 tokens:
-  // the down projection of the 0.5B shape, 896 x 4864: 7.8 us against 9.6 at 8 tokens, 7.0 against 8.0 at one.
-  // There a block of the other kernel spends its time on the activations, which it reads as MFMA operands,
-  // one load a k-step.  Wider or shorter matrices and larger batches were slower here by 5 to 30 %.
-  if (!any_shape && (units > cus || K < 2048 || M > 8)) return MS_UNSUPPORTED;
+  // stage between the loads and the matrix cores): few rows of W per CU and many columns: the down projection
+  // of the 0.5B shape, 896 x 4864: 6.2 us against 8.0 at one token, 7.1 against 9.5 at 8, 10.0 against 11.0 at
+  // 16.  There a block of the other kernel spends its time on the activations, which it reads as MFMA operands,
+  // one load a k-step.  Wider or shorter matrices were slower here by 5 to 30 %.
+  if (!any_shape && (units > cus || K < 2048)) return MS_UNSUPPORTED;
   if (units > 16 * cus) return MS_UNSUPPORTED;   // more than 64 rows to a block
   const int blocks = units < cus ? units : cus;
   const int q = units / blocks, rem = units % blocks;
