@@ -45,9 +45,9 @@ qkv_rope_store_kernel(const float* __restrict__ X, size_t ldx, const float* __re
   const int lane = threadIdx.x & (MS_WAVE - 1), wave = threadIdx.x / MS_WAVE;
   const int col = lane & 15, kq = lane >> 4;
   const int pairs_per_head = d / 32;
-  const int m0 = blockIdx.y * 16 * MT;                    // token groups beyond MT per block: further blocks along y
-  const int head = blockIdx.x / pairs_per_head;          // 0..nh-1: q, then nkv k heads, then nkv v heads
-  const int j0 = (blockIdx.x % pairs_per_head) * 16;      // first feature of the low tile within the head
+  const int m0 = blockIdx.z * 16 * MT;                    // token groups beyond MT per block: further blocks along z
+  const int head = blockIdx.y;                           // 0..nh-1: q, then nkv k heads, then nkv v heads
+  const int j0 = blockIdx.x * 16;                         // first feature of the low tile within the head
   const int half = d / 2;
   const int total_steps = (K + 31) / 32;
 
@@ -167,8 +167,10 @@ qkv_rope_store_kernel(const float* __restrict__ X, size_t ldx, const float* __re
     }
     const long long slot = slot_m[t];
     if (slot < 0) continue;
-    const long long page = slot / page_size;
-    const int off = (int)(slot % page_size);
+    // a page of a power of two (the usual case) needs no division
+    const bool pow2 = (page_size & (page_size - 1)) == 0;
+    const long long page = pow2 ? slot >> (31 - __builtin_clz(page_size)) : slot / page_size;
+    const int off = pow2 ? (int)(slot & (page_size - 1)) : (int)(slot % page_size);
     if (head < nh + nkv) {
       bf16* kp = k_pages + (((size_t)page * nkv + (head - nh)) * page_size + off) * d + j;
       *reinterpret_cast<bf16x4*>(kp) = pa;
@@ -197,7 +199,7 @@ int launch(const float* X, size_t ldx, const float* norm_w, float eps, const bf1
   // LDS holds (waves - 1) * 2 * MT KB
   int waves = 4;
   while (waves < (MT == 1 ? 16 : 8) && blocks * waves < 1024 && steps >= waves * 2) waves *= 2;
-#define GO(WV) qkv_rope_store_kernel<MT, WV><<<dim3(blocks, (M + 16 * MT - 1) / (16 * MT)), dim3(WV * MS_WAVE), 0, stream>>>(X, ldx, norm_w, eps, W, bias, positions, inv_freq, slot_mapping, q_out, k_pages, v_pages, M, K, nh, nkv, d, page_size, v_transposed)
+#define GO(WV) qkv_rope_store_kernel<MT, WV><<<dim3(d / 32, nh + 2 * nkv, (M + 16 * MT - 1) / (16 * MT)), dim3(WV * MS_WAVE), 0, stream>>>(X, ldx, norm_w, eps, W, bias, positions, inv_freq, slot_mapping, q_out, k_pages, v_pages, M, K, nh, nkv, d, page_size, v_transposed)
   if (waves == 4) GO(4); else if (waves == 8) GO(8); else { if constexpr (MT == 1) GO(16); }
 #undef GO
   return ms_launch_status();
