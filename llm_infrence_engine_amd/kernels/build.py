@@ -133,6 +133,42 @@ def build(verbose: bool = True) -> Path:
     return out_dir / LIB_NAME
 
 
+def resource_usage() -> dict:
+    """What every kernel of the library needs, from the compiler's own report: {kernel: {"vgprs", "agprs",
+    "scratch" (bytes a lane: registers spilled to memory), "lds", "occupancy"}}.  Compiles the device code of
+    every source again (no library is written)."""
+    import re
+
+    hipcc = _hipcc()
+
+    def one(src: Path):
+        cmd = [hipcc, *FLAGS, "-I", str(CSRC), "-c", "--cuda-device-only", "-Rpass-analysis=kernel-resource-usage",
+               "-o", os.devnull, str(src)]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise KernelLibraryError(f"hipcc failed on {src.name}:\n{r.stdout}\n{r.stderr}")
+        found, name = {}, None
+        keys = {"VGPRs": "vgprs", "AGPRs": "agprs", "ScratchSize [bytes/lane]": "scratch", "LDS Size [bytes/block]": "lds",
+                "Occupancy [waves/SIMD]": "occupancy"}
+        for line in r.stderr.splitlines():
+            m = re.search(r"remark:\s+(.*?): (\S+) \[-Rpass-analysis", line)
+            if not m:
+                continue
+            what, value = m.group(1).strip(), m.group(2)
+            if what == "Function Name":
+                name = value
+                found[name] = {}
+            elif name and what in keys:
+                found[name][keys[what]] = int(value)
+        return found
+
+    out = {}
+    with ThreadPoolExecutor(max(1, min(len(sources()), os.cpu_count() or 4, 16))) as pool:
+        for d in pool.map(one, sources()):
+            out.update(d)
+    return out
+
+
 def load() -> ctypes.CDLL:
     """The loaded library; built first if it does not exist yet."""
     global _lib

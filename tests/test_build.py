@@ -19,3 +19,20 @@ def test_fallback_folder_is_per_user_and_per_sources():
 
 def test_stamp_lies_beside_the_library(tmp_path):
     assert build._stamp_of(tmp_path / build.LIB_NAME) == tmp_path / "libminiserve_gfx950.stamp"
+
+
+def test_no_kernel_spills_registers_to_memory():
+    """The compiler's own report for every kernel of the library: none keeps registers in scratch memory (a spill
+    in a decode kernel has doubled its time before it was seen) and none asks for more static LDS than a block
+    may have.  Compiles the device code of all sources (about 20 s); skipped where there is no hipcc."""
+    import pytest
+
+    try:
+        build._hipcc()
+    except build.KernelLibraryError:
+        pytest.skip("no hipcc here")
+    usage = build.resource_usage()
+    assert len(usage) > 100
+    spills = {k: v["scratch"] for k, v in usage.items() if v.get("scratch", 0) > 0}
+    assert not spills, f"kernels that spill registers: {spills}"
+    assert all(v.get("lds", 0) <= 64 * 1024 for v in usage.values())
