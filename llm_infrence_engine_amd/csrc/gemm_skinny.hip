@@ -77,13 +77,19 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
 #pragma unroll
       for (int r = 0; r < 4; ++r) if (nb + r < N) bv[u][r] = bias[nb + r];
     }
+    // a lane's four features in one 16-byte access where the row is whole and aligned (the usual case)
+    const bool whole = nb + 3 < N && (ldo & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
       pre[u][t] = f32x4{0.f, 0.f, 0.f, 0.f};
       if (EPI == EPI_RESIDUAL && wave == (u * MT + t) % WAVES && m0 + t * 16 + col < M) {
         const float* o = reinterpret_cast<const float*>(out) + (size_t)(m0 + t * 16 + col) * ldo + nb;
+        if (whole) {
+          pre[u][t] = *reinterpret_cast<const f32x4*>(o);
+        } else {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) if (nb + r < N) pre[u][t][r] = o[r];
+          for (int r = 0; r < 4; ++r) if (nb + r < N) pre[u][t][r] = o[r];
+        }
       }
     }
   }
@@ -177,9 +183,13 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
         }
       } else {
         TO* o = out + (size_t)m * ldo + nb;
+        if (sizeof(TO) == 4 && nb + 3 < N && (ldo & 3) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0) {
+          *reinterpret_cast<f32x4*>(o) = sum + bv[u] + pre[u][t];
+        } else {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          if (nb + r < N) o[r] = from_float<TO>(sum[r] + bv[u][r] + pre[u][t][r]);
+          for (int r = 0; r < 4; ++r) {
+            if (nb + r < N) o[r] = from_float<TO>(sum[r] + bv[u][r] + pre[u][t][r]);
+          }
         }
       }
     }
