@@ -34,7 +34,7 @@ int ms_gemm_skinny(const void* A, long long lda, const void* W, long long ldw, c
                    long long ldo, int M, int N, int K, int epilogue, int out_dtype, hipStream_t stream);
 
 void ms_gemm_skinny_force(int ntile, int waves, int token_groups);
-void ms_attention_mfma_force(int nt, int waves);
+void ms_attention_mfma_force(int nt, int waves, int dim_shares);
 
 int ms_gemm_stream(const void* A, long long lda, const int* rows, const float* norm_w, float eps, const void* W,
                    long long ldw, const float* bias, void* out, long long ldo, int M, int N, int K, int epilogue,

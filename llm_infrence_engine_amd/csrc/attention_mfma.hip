@@ -44,9 +44,9 @@ template <int D>
 struct KeyBlock {          // one block of 32 keys as this lane sees it
   bf16x8 k[2][D / 32];     // [16-key subtile][32-dim step]
 };
-template <int D>
-struct ValueBlock {        // and its values
-  bf16x4 v[D / 16][2];     // [16-dim tile][subtile]: 4 keys of one dim; the two subtiles are one MFMA operand
+template <int CT>
+struct ValueBlock {        // and its values, for the CT tiles of 16 dims that this block works out
+  bf16x4 v[CT][2];         // [16-dim tile][subtile]: 4 keys of one dim; the two subtiles are one MFMA operand
 };
 
 // Page arithmetic: pages of a power of two (page_shift >= 0) need no division.
@@ -95,20 +95,25 @@ __device__ __forceinline__ void load_keys(KeyBlock<D>& b, const bf16* __restrict
   }
 }
 
-template <int D>
-__device__ __forceinline__ void load_values(ValueBlock<D>& b, const bf16* __restrict__ vt_pages,
-                                            const BlockPlace& bp, PageGeom pg, int lane) {
-  const int v_lane = (lane & 15) * pg.size + (lane >> 4) * 4;   // this lane's dim and keys inside a 16-dim tile
+template <int CT>
+__device__ __forceinline__ void load_values(ValueBlock<CT>& b, const bf16* __restrict__ vt_pages,
+                                            const BlockPlace& bp, PageGeom pg, int dim0, int lane) {
+  const int v_lane = (dim0 + (lane & 15)) * pg.size + (lane >> 4) * 4;   // this lane's dim and keys inside a tile
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
     const bf16* vp = vt_pages + bp.head[u] + bp.off[u];
 #pragma unroll
-    for (int c = 0; c < D / 16; ++c) b.v[c][u] = *reinterpret_cast<const bf16x4*>((vp + c * 16 * pg.size) + v_lane);
+    for (int c = 0; c < CT; ++c) b.v[c][u] = *reinterpret_cast<const bf16x4*>((vp + c * 16 * pg.size) + v_lane);
   }
 }
 
 // Two waves of a wide tile on every SIMD (256 registers each) hide each other's waits; narrow tiles fit anyway.
-template <int D, int NT, int WAVES, bool SPLIT>
+//
+// VS > 1 (narrow tiles only) shares one tile among VS blocks: each works out all scores and the whole softmax
+// but only D / VS of the output's dims, so it reads all keys and 1 / VS of the values.  A compute unit draws
+// its data at a small fraction of the chip's rate, so when a step has fewer tiles than the chip has units this
+// shortens the longest chain without a second kernel; the blocks write disjoint dims and share nothing.
+template <int D, int NT, int WAVES, bool SPLIT, int VS>
 __global__ void __launch_bounds__(WAVES * MS_WAVE, (NT > 1 ? 2 : 1))
 attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* __restrict__ k_pages,
                       const bf16* __restrict__ vt_pages, const int* __restrict__ block_table, int table_stride,
@@ -117,7 +122,10 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
                       float* __restrict__ part_ml, int nh, int nkv, int page_size, int page_shift,
                       float scale_log2e, int window, int min_blocks, int n_splits) {
   __shared__ float sm_m[WAVES][NT][16], sm_l[WAVES][NT][16];
-  __shared__ f32x4 sm_o[WAVES > 1 ? WAVES - 1 : 1][D / 16][NT][MS_WAVE];
+  static_assert(VS == 1 || (NT == 1 && !SPLIT), "only narrow tiles of the general shape share their dims out");
+  static_assert((D / 16) % VS == 0, "whole tiles of 16 dims to a block");
+  constexpr int CT = D / 16 / VS;
+  __shared__ f32x4 sm_o[WAVES > 1 ? WAVES - 1 : 1][CT][NT][MS_WAVE];
   const int lane = threadIdx.x & (MS_WAVE - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MS_WAVE);   // the same for the whole wave
   const int col16 = lane & 15, kq = lane >> 4;
@@ -139,7 +147,9 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
   const int start_pos = context_lens[r] - qlen;
   const int ncols = qlen * rep;
   // late tiles of a prompt see the most keys: they go first so that the long ones do not finish last
-  const int c0 = SPLIT ? 0 : (gridDim.x - 1 - blockIdx.x) * 16 * NT;
+  const int tile = VS > 1 ? blockIdx.x / VS : blockIdx.x, n_tiles = VS > 1 ? gridDim.x / VS : gridDim.x;
+  const int dim0 = VS > 1 ? (blockIdx.x % VS) * CT * 16 : 0;   // the first of this block's output dims
+  const int c0 = SPLIT ? 0 : (n_tiles - 1 - tile) * 16 * NT;
   if (c0 >= ncols) return;
 
   // key range of the tile: from the first column's window start to the last column's own position
@@ -175,13 +185,13 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
   }
 
   float m[NT], l[NT];
-  f32x4 o[D / 16][NT];
+  f32x4 o[CT][NT];
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     m[t] = -INFINITY;
     l[t] = 0.f;
 #pragma unroll
-    for (int c = 0; c < D / 16; ++c) o[c][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int c = 0; c < CT; ++c) o[c][t] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
   // A narrow tile (decode) has registers to spare and few waves to hide a wait behind: it fetches the next
@@ -189,7 +199,7 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
   // uses them (the score products and the softmax run meanwhile, and so does the SIMD's other wave).
   constexpr bool VALUES_EARLY = NT == 1;
   KeyBlock<D> cur_k, nxt_k;
-  ValueBlock<D> cur_v, nxt_v;
+  ValueBlock<CT> cur_v, nxt_v;
   BlockPlace cur_at, nxt_at;
   if (blk_begin + wave < blk_end) {
     const int base = (blk_begin + wave) * 32;
@@ -202,17 +212,17 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
     }
     cur_at = place_of(pages, base, g, nkv, pg, D);
     load_keys<D>(cur_k, k_pages, cur_at, lane);
-    if (VALUES_EARLY) load_values<D>(cur_v, vt_pages, cur_at, pg, lane);
+    if (VALUES_EARLY) load_values<CT>(cur_v, vt_pages, cur_at, pg, dim0, lane);
   }
   for (int blk = blk_begin + wave; blk < blk_end; blk += WAVES) {
     const int base = blk * 32;
-    if (!VALUES_EARLY) load_values<D>(cur_v, vt_pages, cur_at, pg, lane);
+    if (!VALUES_EARLY) load_values<CT>(cur_v, vt_pages, cur_at, pg, dim0, lane);
     if (blk + WAVES < blk_end) {
       int pages[2];
       pages_of(table, base + WAVES * 32, key_hi, pg, pages);
       nxt_at = place_of(pages, base + WAVES * 32, g, nkv, pg, D);
       load_keys<D>(nxt_k, k_pages, nxt_at, lane);
-      if (VALUES_EARLY) load_values<D>(nxt_v, vt_pages, nxt_at, pg, lane);
+      if (VALUES_EARLY) load_values<CT>(nxt_v, vt_pages, nxt_at, pg, dim0, lane);
     }
 
     // scores: s[u][t] holds keys base + u*16 + kq*4 + (0..3) of column t*16 + col16
@@ -235,7 +245,7 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
         for (int i = 0; i < 4; ++i)
           if (base + u * 16 + kq * 4 + i > key_hi) {
 #pragma unroll
-            for (int c = 0; c < D / 16; ++c) cur_v.v[c][u][i] = (__bf16)0.0f;
+            for (int c = 0; c < CT; ++c) cur_v.v[c][u][i] = (__bf16)0.0f;
           }
     }
 
@@ -294,7 +304,7 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
 #pragma unroll
       for (int t = 0; t < NT; ++t)
 #pragma unroll
-        for (int c = 0; c < D / 16; ++c) o[c][t] *= corr[t];
+        for (int c = 0; c < CT; ++c) o[c][t] *= corr[t];
     }
     // column by column, so that the products of one column run on the matrix cores while the next column's
     // exponentials are taken
@@ -311,7 +321,7 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
         }
       l[t] = l[t] * corr[t] + ls;
 #pragma unroll
-      for (int c = 0; c < D / 16; ++c) {
+      for (int c = 0; c < CT; ++c) {
         bf16x8 vv;
 #pragma unroll
         for (int i = 0; i < 4; ++i) { vv[i] = cur_v.v[c][0][i]; vv[4 + i] = cur_v.v[c][1][i]; }
@@ -337,7 +347,7 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
       if (kq == 0) { sm_m[wave][t][col16] = m[t]; sm_l[wave][t][col16] = l[t]; }
       if (wave > 0) {
 #pragma unroll
-        for (int c = 0; c < D / 16; ++c) sm_o[wave - 1][c][t][lane] = o[c][t];
+        for (int c = 0; c < CT; ++c) sm_o[wave - 1][c][t][lane] = o[c][t];
       }
     }
     __syncthreads();
@@ -350,12 +360,12 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
       const float f0 = fast_exp2(m[t] - safe);
       float lsum = l[t] * f0;
 #pragma unroll
-      for (int c = 0; c < D / 16; ++c) o[c][t] *= f0;
+      for (int c = 0; c < CT; ++c) o[c][t] *= f0;
       for (int w = 1; w < WAVES; ++w) {
         const float f = fast_exp2(sm_m[w][t][col16] - safe);
         lsum += f * sm_l[w][t][col16];
 #pragma unroll
-        for (int c = 0; c < D / 16; ++c) o[c][t] += sm_o[w - 1][c][t][lane] * f;
+        for (int c = 0; c < CT; ++c) o[c][t] += sm_o[w - 1][c][t][lane] * f;
       }
       m[t] = big;
       l[t] = lsum;
@@ -373,13 +383,13 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
       const size_t slot = ((size_t)r * nh + head) * n_splits + blockIdx.x;
       float* po = part_o + slot * D + kq * 4;
 #pragma unroll
-      for (int c = 0; c < D / 16; ++c) *reinterpret_cast<f32x4*>(po + c * 16) = o[c][t];
+      for (int c = 0; c < CT; ++c) *reinterpret_cast<f32x4*>(po + c * 16) = o[c][t];
       if (kq == 0) { part_ml[slot * 2] = m[t]; part_ml[slot * 2 + 1] = lt; }
     } else {
       const float inv = 1.0f / lt;
-      bf16* op = out + (size_t)tok * out_stride + (size_t)head * D + kq * 4;
+      bf16* op = out + (size_t)tok * out_stride + (size_t)head * D + dim0 + kq * 4;
 #pragma unroll
-      for (int c = 0; c < D / 16; ++c) {
+      for (int c = 0; c < CT; ++c) {
         bf16x4 w;
 #pragma unroll
         for (int i = 0; i < 4; ++i) w[i] = (__bf16)(o[c][t][i] * inv);
@@ -434,7 +444,7 @@ attention_combine_kernel(const float* __restrict__ part_o, const float* __restri
   }
 }
 
-int g_force_nt = 0, g_force_waves = 0;
+int g_force_nt = 0, g_force_waves = 0, g_force_vs = 0;
 
 inline int page_shift_of(int page_size) {   // log2 of a power of two, else -1
   if (page_size & (page_size - 1)) return -1;
@@ -443,14 +453,14 @@ inline int page_shift_of(int page_size) {   // log2 of a power of two, else -1
   return sh;
 }
 
-template <int D, int NT, int WAVES>
+template <int D, int NT, int WAVES, int VS>
 int launch_general(const bf16* q, size_t q_stride, const bf16* k, const bf16* vt, const int* table, int table_stride,
                    const int* q_start, const int* ctx, bf16* out, size_t out_stride, int n_requests, int max_q_len,
                    int nh, int nkv, int page_size, float scale, int window, hipStream_t stream) {
   const int rep = nh / nkv;
   const int tiles = (max_q_len * rep + 16 * NT - 1) / (16 * NT);
-  dim3 grid(tiles, nkv, n_requests), block(WAVES * MS_WAVE);
-  attention_mfma_kernel<D, NT, WAVES, false><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, q_start, ctx, out, out_stride, nullptr, nullptr, nh, nkv, page_size, page_shift_of(page_size), scale * 1.4426950408889634f, window, 0, 0);
+  dim3 grid(tiles * VS, nkv, n_requests), block(WAVES * MS_WAVE);
+  attention_mfma_kernel<D, NT, WAVES, false, VS><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, q_start, ctx, out, out_stride, nullptr, nullptr, nh, nkv, page_size, page_shift_of(page_size), scale * 1.4426950408889634f, window, 0, 0);
   return ms_launch_status();
 }
 
@@ -460,18 +470,20 @@ int launch_split(const bf16* q, size_t q_stride, const bf16* k, const bf16* vt, 
                  int n_requests, int nh, int nkv, int page_size, float scale, int window, int min_blocks,
                  int n_splits, hipStream_t stream) {
   dim3 grid(n_splits, nkv, n_requests), block(4 * MS_WAVE);
-  attention_mfma_kernel<D, 1, 4, true><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, q_start, ctx, out, out_stride, part_o, part_ml, nh, nkv, page_size, page_shift_of(page_size), scale * 1.4426950408889634f, window, min_blocks, n_splits);
+  attention_mfma_kernel<D, 1, 4, true, 1><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, q_start, ctx, out, out_stride, part_o, part_ml, nh, nkv, page_size, page_shift_of(page_size), scale * 1.4426950408889634f, window, min_blocks, n_splits);
   attention_combine_kernel<D><<<dim3(n_requests * nh), dim3(D < 64 ? 64 : D), 0, stream>>>(part_o, part_ml, q_start, ctx, out, out_stride, nh, window, min_blocks, n_splits);
   return ms_launch_status();
 }
 
 }  // namespace
 
-// Tuning knob: force the general shape's tile width (16 * nt columns) and waves per tile; 0 restores the choice
-// by size.  Shapes outside the menu are refused at the call.
-extern "C" void ms_attention_mfma_force(int nt, int waves) {
+// Tuning knob: force the general shape's tile width (16 * nt columns), waves per tile and (narrow tiles) the
+// number of blocks that share a tile's dims; 0 restores the choice by size.  Shapes outside the menu are
+// refused at the call.
+extern "C" void ms_attention_mfma_force(int nt, int waves, int dim_shares) {
   g_force_nt = nt;
   g_force_waves = waves;
+  g_force_vs = dim_shares;
 }
 
 // Whether the matrix-core kernels take this geometry (else the caller uses the generic kernel).
@@ -493,17 +505,33 @@ extern "C" int ms_paged_attention_mfma(const void* q, long long q_stride, const 
   if (!ms_attention_mfma_supported(head_dim, page_size)) return MS_UNSUPPORTED;
   if (q_stride % 8 || out_stride % 4 || ((uintptr_t)q % 16) || ((uintptr_t)out % 8)) return MS_UNSUPPORTED;
   if (n_requests > 65535 || num_kv_heads > 65535) return MS_UNSUPPORTED;
-#define GO(D, NT, WV) return launch_general<D, NT, WV>((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)vt_pages, block_table, table_stride, q_start, context_lens, (bf16*)out, out_stride, n_requests, max_q_len, num_heads, num_kv_heads, page_size, scale, window, stream)
+#define GO(D, NT, WV, VS) return launch_general<D, NT, WV, VS>((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)vt_pages, block_table, table_stride, q_start, context_lens, (bf16*)out, out_stride, n_requests, max_q_len, num_heads, num_kv_heads, page_size, scale, window, stream)
   // Tile width (NT * 16 columns) and waves over a tile's keys.  Few columns (a decode step): one narrow tile
   // per request and many waves over its keys.
   const int cols = max_q_len * (num_heads / num_kv_heads);
   int nt = cols > 16 ? (head_dim == 128 ? 2 : 4) : 1;
   int waves = nt > 1 ? 4 : (head_dim == 128 ? 8 : 16);
+  // narrow tiles, far fewer of them than compute units: blocks share a tile's dims while that leaves half the
+  // units free (with every unit busy the keys' repeated reading costs more than the shorter chains save:
+  // 64 requests at 1,000 keys took 12.1 us shared two ways against 11.1)
+  int vs = 1;
+  if (nt == 1) {
+    const long long tiles = (long long)n_requests * num_kv_heads * ((cols + 15) / 16);
+    const int cus = ms_compute_units();
+    while (vs < 4 && (head_dim / 16) % (vs * 2) == 0 && tiles * vs * 4 <= cus) vs *= 2;
+  }
   if (g_force_nt) { nt = g_force_nt; waves = g_force_waves; }
-#define PICK(D, NT, WV) if (head_dim == D && nt == NT && waves == WV) GO(D, NT, WV)
+  if (g_force_vs) vs = g_force_vs;
+  if (nt > 1) vs = 1;
+#define PICK(D, NT, WV) if (head_dim == D && nt == NT && waves == WV && vs == 1) GO(D, NT, WV, 1)
+#define PICK_SHARED(D, WV, VS) if (head_dim == D && nt == 1 && waves == WV && vs == VS) GO(D, 1, WV, VS)
   PICK(32, 4, 4); PICK(32, 2, 4); PICK(32, 2, 8); PICK(32, 1, 8); PICK(32, 1, 16);
   PICK(64, 4, 4); PICK(64, 2, 4); PICK(64, 2, 8); PICK(64, 1, 4); PICK(64, 1, 8); PICK(64, 1, 16);
   PICK(128, 2, 4); PICK(128, 1, 4); PICK(128, 1, 8);
+  PICK_SHARED(32, 16, 2);
+  PICK_SHARED(64, 16, 2); PICK_SHARED(64, 16, 4); PICK_SHARED(64, 8, 2); PICK_SHARED(64, 8, 4);
+  PICK_SHARED(128, 8, 2); PICK_SHARED(128, 8, 4);
+#undef PICK_SHARED
 #undef PICK
   return MS_UNSUPPORTED;
 #undef GO

@@ -505,14 +505,17 @@ def _run_mfma(ops, c, nh, d, ctx, qlen, window=None):
     return out.double().cpu()
 
 
-@pytest.mark.parametrize("d,shape", [(32, (4, 4)), (32, (2, 4)), (32, (2, 8)), (32, (1, 8)), (32, (1, 16)),
-                                     (64, (4, 4)), (64, (2, 4)), (64, (2, 8)), (64, (1, 4)), (64, (1, 8)), (64, (1, 16)),
-                                     (128, (2, 4)), (128, (1, 4)), (128, (1, 8))])
+@pytest.mark.parametrize("d,shape", [(32, (4, 4, 1)), (32, (2, 4, 1)), (32, (2, 8, 1)), (32, (1, 8, 1)), (32, (1, 16, 1)),
+                                     (64, (4, 4, 1)), (64, (2, 4, 1)), (64, (2, 8, 1)), (64, (1, 4, 1)), (64, (1, 8, 1)),
+                                     (64, (1, 16, 1)), (128, (2, 4, 1)), (128, (1, 4, 1)), (128, (1, 8, 1)),
+                                     (32, (1, 16, 2)), (64, (1, 16, 2)), (64, (1, 16, 4)), (64, (1, 8, 2)), (64, (1, 8, 4)),
+                                     (128, (1, 8, 2)), (128, (1, 8, 4))])
 def test_attention_mfma_tile_shapes(ops, d, shape):
-    """Every tile width and wave count of the menu gives the same answer (the choice by size picks among them)."""
+    """Every tile width, wave count and number of blocks to a narrow tile on the menu gives the same answer (the
+    choice by size picks among them)."""
     from llm_infrence_engine_amd.kernels import build
     nh, nkv = 6, 2
-    g = torch.Generator().manual_seed(d + shape[0] * 7 + shape[1])
+    g = torch.Generator().manual_seed(d + shape[0] * 7 + shape[1] + shape[2] * 1000)
     ctx, qlen = [300, 97, 520], [130, 1, 45]
     c = _paged_case(g, torch.bfloat16, nh, nkv, d, 16, ctx, qlen, float("nan"))
     want = torch.cat([attention_reference(q.double(), k.double(), v.double(), 1.0 / math.sqrt(d), None).transpose(0, 1).reshape(-1, nh * d)
@@ -522,7 +525,7 @@ def test_attention_mfma_tile_shapes(ops, d, shape):
     try:
         got = _run_mfma(ops, c, nh, d, ctx, qlen)
     finally:
-        lib.ms_attention_mfma_force(0, 0)
+        lib.ms_attention_mfma_force(0, 0, 0)
     torch.testing.assert_close(got, want, **tol(torch.bfloat16))
 
 
