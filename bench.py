@@ -122,6 +122,34 @@ def run_prefill(eng_mod, model, vocab, seed, repeats=5):
     return best
 
 
+def run_serving(eng_mod, model, vocab, seed, n_requests=64, new_tokens=256, lo=128, hi=4096, max_seqs=64,
+                budget=4096):
+    """The whole engine on a queue of requests: prompts of lo..hi tokens (uniform), ``new_tokens`` decoded for
+    each, admitted as pages and slots allow, prompts in portions beside the decoding of earlier requests."""
+    import numpy as np
+    import torch
+
+    rng = np.random.default_rng(seed)
+    lens = [int(n) for n in rng.integers(lo, hi + 1, n_requests)]
+    pages = max_seqs * (-(-(hi + new_tokens) // BLOCK_SIZE) + 1)
+    e = eng_mod.Engine(model, num_blocks=pages, block_size=BLOCK_SIZE, max_seqs=max_seqs, max_len=CONTEXT_LIMIT,
+                       max_num_batched_tokens=budget, hip_graphs=True, decode_steps_per_launch=DECODE_STEPS_PER_LAUNCH)
+    reqs = [eng_mod.Request([int(t) for t in rng.integers(0, vocab, n)], max_new_tokens=new_tokens) for n in lens]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for r in reqs:
+        e.add_request(r)
+    while e.has_work():
+        e.step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    made = sum(len(r.output_ids) for r in reqs)
+    mixed = sum(1 for rec in e.steps if rec.n_prefill_tokens and rec.decode_batch)
+    return {"seconds": round(dt, 3), "requests": n_requests, "prompt_tokens": sum(lens), "new_tokens": made,
+            "new_tokens_per_s": round(made / dt, 1), "all_tokens_per_s": round((sum(lens) + made) / dt, 1),
+            "launches": len(e.steps), "mixed_launches": mixed, "preemptions": e.preemptions}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
     ap.add_argument("--gpus", type=int, default=1)
@@ -134,7 +162,9 @@ def main() -> int:
                     help="fewer layers than the configuration has, if memory or time needs it (both numbers are reported)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points and the prefill")
     ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN, help="prompt length of the decode run (default 512)")
-    ap.add_argument("--only", choices=["prefill"], help="run one part alone (for profiles): the 2,048-token prefill")
+    ap.add_argument("--only", choices=["prefill", "serve"],
+                    help="run one part alone: the 2,048-token prefill (for profiles), or a queue of 64 requests with "
+                         "prompts of 128 to 4,096 tokens and 256 decoded tokens each through the scheduler")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(f"bench.py measures one GPU; --gpus {a.gpus} is not supported by this single-GPU engine")
@@ -159,6 +189,11 @@ def main() -> int:
         pt = run_prefill(eng, model, vocab, seed=2, repeats=3)
         print(json.dumps({"prefill": {"value": round(PREFILL_TOKENS / pt, 1), "tokens": PREFILL_TOKENS,
                                       "ms": round(pt * 1e3, 3)}}), flush=True)
+        return 0
+
+    if a.only == "serve":
+        run_serving(eng, model, vocab, seed=4, n_requests=8, new_tokens=16)       # warms up graphs and the library
+        print(json.dumps({"serving": run_serving(eng, model, vocab, seed=5)}), flush=True)
         return 0
 
     dt, ctx = run_decode(eng, model, a.batch, a.steps, a.warmup, vocab, seed=1, prompt_len=a.prompt_len)

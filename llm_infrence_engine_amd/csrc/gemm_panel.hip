@@ -1,0 +1,333 @@
+// out[M,N] = A[M,K] . W[N,K]^T for 17 to 64 tokens (a decode step of a larger batch) and a W of many rows,
+// bfloat16 in, float accumulation on the matrix cores (v_mfma_f32_16x16x32_bf16).
+//
+// With this many tokens the activations, not the weights, are most of what a block has to load when it reads
+// them as MFMA operands k-step by k-step: every 16-row tile of W needs all of A again, and what a CU can pull
+// through its load path (from L2 as from memory) is about 1/256 of what the chip can.  So here every block
+// loads A once, whole, into LDS (the panel: bfloat16, K padded to a multiple of 32 with zeros, rows one
+// 16-byte piece apart in the banks), and then streams its share of W against it: the 16-row tiles of W are dealt
+// out evenly over as many blocks as the chip has CUs, and inside a block
+//   * rounds of 16 tiles go to the 16 waves whole (no sum across waves);
+//   * the tiles left over (all of them, for a block with fewer than 16) are shared, each among floor(16 / left)
+//     waves that take the tile's k-steps in turn; their accumulators are added through LDS (over the panel,
+//     which is no longer needed) in wave order.
+// Either way an element's sum runs in an order that depends on the shape of the product alone.
+//
+// The weight tile is the A operand and the panel the B operand of the MFMA: a lane ends up with 4 consecutive
+// output features of one token.  Epilogues and the folded RMS norm as in gemm_skinny: plain (+ bias) to bfloat16
+// or float; gated activation over interleaved rows (2j: gate j, 2j+1: up j); the residual sum out += product
+// (+ bias) on a float matrix.  With NORM the activations are the float residual stream: the panel holds
+// bfloat16(x * norm_weight), the squares are summed on the way in a fixed order, and the accumulators are
+// scaled by rsqrt(mean(x^2) + eps) before the epilogue.
+#include "common.h"
+#include "api.h"
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) unsigned u32x4;   // a 16-byte piece: 8 bfloat16
+
+enum { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_RESIDUAL = 3 };
+
+constexpr int WAVES = 16;       // waves of a block
+constexpr int BATCH = 4;        // panel loads a wave has in flight
+constexpr int MAX_TOKENS = 64;
+constexpr int MAX_PARTS = 4;    // 64-piece (512-column) loads per row of A at most: K <= 2048
+
+// id / parts for the small numbers that occur here (id < 4096, parts <= 16) by a multiplication
+__device__ __forceinline__ int small_inverse(int parts) { return (65536 + parts - 1) / parts; }
+__device__ __forceinline__ int small_div(int id, int inverse) { return (id * inverse) >> 16; }
+
+template <int TT, int EPI, typename TO, bool NORM>
+__global__ void __launch_bounds__(WAVES * MS_WAVE)
+gemm_panel_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restrict__ W, size_t ldw,
+                  const float* __restrict__ bias, TO* __restrict__ out, size_t ldo, int M, int N, int K,
+                  const float* __restrict__ norm_w, float eps, const int* __restrict__ rows, int q, int rem) {
+  // weight fragments a wave asks for before it multiplies them (with four token tiles the registers, 128 to a
+  // lane with 16 waves on the CU, hold fewer)
+  constexpr int DEPTH = TT >= 4 ? 7 : 8;
+  extern __shared__ u32x4 smem[];   // the panel [tokens][pitch]; afterwards the waves' partial sums
+  __shared__ float ss_part[MAX_TOKENS * MAX_PARTS];
+  __shared__ float inv_rms[MAX_TOKENS];
+  const bf16* A = (const bf16*)Av;
+  const float* X = (const float*)Av;
+  const int lane = threadIdx.x & (MS_WAVE - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MS_WAVE);   // the same for the whole wave
+  const int col = lane & 15, kq = lane >> 4;
+  const int K8 = K / 8, S = (K + 31) / 32;
+  const int pitch = S * 4 + 1;              // odd, so that 16 rows read at one column hit 16 different banks
+  const int parts = (K8 + 63) / 64;         // loads of 64 lanes x 8 columns per row of A
+  u32x4* xst = smem;
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+
+  // ---- this block's tiles of W: dealt out evenly (the first `rem` blocks take one more).  Rounds of 16 tiles go
+  // to the 16 waves whole; the tiles left over are shared, each among g waves that take its k-steps in turn.
+  const int b = blockIdx.x;
+  const int T = q + (b < rem ? 1 : 0);
+  const int t0 = b * q + min(b, rem);
+  const int T_whole = T & ~(WAVES - 1), T_left = T - T_whole;
+  const int g = T_left ? WAVES / T_left : 1;
+  int left_tile = 0, j = 0;     // this wave's shared tile (if below T_left) and its place among that tile's waves
+  if (T_left) {
+    left_tile = small_div(wave, small_inverse(g));
+    j = wave - left_tile * g;
+  }
+  const bool shares = T_left && left_tile < T_left;
+
+  bf16x8 wa[DEPTH];
+  // fragments of DEPTH k-steps (s0, s0 + step, ...) of a tile: lane (col, kq) holds row col, columns kq * 8 ..
+  auto fetch = [&](int tile, int s0, int step) {
+    const bf16* wrow = W + (size_t)min((t0 + tile) * 16 + col, N - 1) * ldw;   // rows past N repeat the last
+#pragma unroll
+    for (int p = 0; p < DEPTH; ++p) {
+      const int s = s0 + p * step;
+      if (s >= S) break;   // the same for the whole wave
+      const int k = s * 32 + kq * 8;
+      wa[p] = *reinterpret_cast<const bf16x8*>(wrow + min(k, K - 8));   // K is a multiple of 8: a piece is in or out
+      if (k >= K) wa[p] = __builtin_bit_cast(bf16x8, zero);
+    }
+  };
+  // the wave's first fragments are asked for before the panel is built: they come from memory, the panel
+  // from L2, and neither waits for the other
+  if (T_whole) fetch(wave, 0, 1);
+  else if (shares) fetch(left_tile, j, g);
+
+  // ---- the panel.  A wave keeps to one 512-column part of the rows (so it loads that part of the norm weights
+  // once) and takes every (16 / parts2)-th token, BATCH of them in flight.
+  {
+    const int parts2 = parts <= 1 ? 1 : (parts <= 2 ? 2 : 4);
+    const int part = wave & (parts2 - 1);
+    const int tok_step = WAVES / parts2;
+    const int c = part * 64 + lane;
+    const bool in = c < K8;   // lanes past the row's end (and whole waves, when parts is 3) load nothing new
+    const int cc = min(c, K8 - 1) * 8;
+    f32x4 nwf[2];
+    if (NORM) {
+      nwf[0] = *reinterpret_cast<const f32x4*>(norm_w + cc);
+      nwf[1] = *reinterpret_cast<const f32x4*>(norm_w + cc + 4);
+    }
+    if (part < parts) {
+      for (int base = wave / parts2; base < M; base += tok_step * BATCH) {
+        u32x4 piece[NORM ? 1 : BATCH];
+        f32x4 xf[NORM ? BATCH : 1][2];
+#pragma unroll
+        for (int i = 0; i < BATCH; ++i) {
+          const int tok = base + i * tok_step;
+          if (tok >= M) break;   // the same for the whole wave
+          const size_t at = (size_t)(rows ? rows[tok] : tok) * lda + cc;
+          if (NORM) {
+            xf[i][0] = *reinterpret_cast<const f32x4*>(X + at);
+            xf[i][1] = *reinterpret_cast<const f32x4*>(X + at + 4);
+          } else {
+            piece[i] = *reinterpret_cast<const u32x4*>(A + at);
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < BATCH; ++i) {
+          const int tok = base + i * tok_step;
+          if (tok >= M) break;
+          u32x4 pc;
+          if (NORM) {
+            bf16x8 h;
+            float ss = 0.f;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const float x0 = in ? xf[i][0][e] : 0.f, x1 = in ? xf[i][1][e] : 0.f;
+              ss = fmaf(x0, x0, ss);
+              ss = fmaf(x1, x1, ss);
+              h[e] = (__bf16)(x0 * nwf[0][e]);
+              h[4 + e] = (__bf16)(x1 * nwf[1][e]);
+            }
+            pc = __builtin_bit_cast(u32x4, h);
+            ss = wave_sum(ss);   // the lanes of a load in a fixed tree
+            if (lane == 0) ss_part[tok * parts + part] = ss;
+          } else {
+            pc = piece[i];
+          }
+          if (in) xst[tok * pitch + c] = pc;
+        }
+      }
+    }
+    // a last k-step that K fills only in part reads zeros for the rest
+    const int padn = S * 4 - K8;   // 0..3
+    for (int t = threadIdx.x; t < M * padn; t += WAVES * MS_WAVE) {
+      const int rr = t / padn;
+      xst[rr * pitch + K8 + t - rr * padn] = zero;
+    }
+  }
+  __syncthreads();
+  if (NORM) {
+    if (threadIdx.x < M) {   // a token's parts in order
+      float total = 0.f;
+      for (int p = 0; p < parts; ++p) total += ss_part[threadIdx.x * parts + p];
+      inv_rms[threadIdx.x] = 1.0f / sqrtf(total / (float)K + eps);
+    }
+    __syncthreads();
+  }
+
+  int xrow[TT];   // idle columns repeat the last token; their results are not stored
+#pragma unroll
+  for (int tt = 0; tt < TT; ++tt) xrow[tt] = min(tt * 16 + col, M - 1) * pitch + kq;
+
+  // what a lane holds of a finished tile: out[token tt * 16 + col][n0 + kq * 4 + (0..3)]
+  auto finish = [&](int tl, f32x4* sum) {
+    const int nb = (t0 + tl) * 16 + kq * 4;
+    f32x4 bv = {0.f, 0.f, 0.f, 0.f};
+    if (bias && EPI != EPI_SWIGLU) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) if (nb + r < N) bv[r] = bias[nb + r];
+    }
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) {
+      const int m = tt * 16 + col;
+      if (m >= M) continue;
+      f32x4 v = sum[tt];
+      if (NORM) v *= inv_rms[m];
+      if (EPI == EPI_SWIGLU) {
+        // rows nb, nb+1 are (gate, up) of feature nb/2; rows nb+2, nb+3 of feature nb/2 + 1
+#pragma unroll
+        for (int p = 0; p < 2; ++p)
+          if (nb + 2 * p + 1 < N) out[(size_t)m * ldo + nb / 2 + p] = from_float<TO>(fast_silu(v[2 * p]) * v[2 * p + 1]);
+      } else {
+        TO* o = out + (size_t)m * ldo + nb;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          if (nb + r >= N) continue;
+          if (EPI == EPI_RESIDUAL) o[r] = from_float<TO>(to_float(o[r]) + v[r] + bv[r]);
+          else o[r] = from_float<TO>(v[r] + bv[r]);
+        }
+      }
+    }
+  };
+
+  f32x4 acc[TT];
+  // the fetched fragments of k-steps s0, s0 + step, ... times the panel
+  auto multiply = [&](int s0, int step) {
+#pragma unroll
+    for (int p = 0; p < DEPTH; ++p) {
+      const int s = s0 + p * step;
+      if (s >= S) break;
+#pragma unroll
+      for (int tt = 0; tt < TT; ++tt) {
+        const bf16x8 xb = __builtin_bit_cast(bf16x8, xst[xrow[tt] + 4 * s]);
+        acc[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[p], xb, acc[tt], 0, 0, 0);
+      }
+    }
+  };
+
+  for (int tile = wave; tile < T_whole; tile += WAVES) {   // whole tiles: no sum across waves
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) acc[tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < S; s0 += DEPTH) {
+      if (tile != wave || s0 != 0) fetch(tile, s0, 1);   // the first were fetched above
+      multiply(s0, 1);
+    }
+    finish(tile, acc);
+  }
+  if (!T_left) return;   // the same for the whole block
+
+  if (shares) {
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) acc[tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int s0 = j; s0 < S; s0 += g * DEPTH) {
+      if (T_whole || s0 != j) fetch(T_whole + left_tile, s0, g);
+      multiply(s0, g);
+    }
+  }
+  // the first wave of a shared tile adds the others' accumulators in wave order
+  __syncthreads();   // nobody reads the panel any more
+  f32x4* red = reinterpret_cast<f32x4*>(smem);   // [WAVES][TT][64]
+  if (shares && j > 0) {
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) red[(wave * TT + tt) * MS_WAVE + lane] = acc[tt];
+  }
+  __syncthreads();
+  if (shares && j == 0) {
+    for (int w = 1; w < g; ++w) {
+#pragma unroll
+      for (int tt = 0; tt < TT; ++tt) acc[tt] += red[((wave + w) * TT + tt) * MS_WAVE + lane];
+    }
+    finish(T_whole + left_tile, acc);
+  }
+}
+
+constexpr int LDS_BUDGET = 144 * 1024;   // of the CU's 160 KB, for the panel
+
+template <int TT, int EPI, typename TO, bool NORM>
+int launch(const void* A, size_t lda, const bf16* W, size_t ldw, const float* bias, TO* out, size_t ldo, int M, int N,
+           int K, const float* norm_w, float eps, const int* rows, int blocks, int q, int rem, size_t lds,
+           hipStream_t stream) {
+  static bool raised = false;   // once per instantiation: allow more dynamic LDS than the default 64 KB
+  if (!raised) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_panel_kernel<TT, EPI, TO, NORM>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BUDGET) != hipSuccess)
+      return MS_LAUNCH_FAILED;
+    raised = true;
+  }
+  gemm_panel_kernel<TT, EPI, TO, NORM><<<dim3(blocks), dim3(WAVES * MS_WAVE), lds, stream>>>(
+      A, lda, W, ldw, bias, out, ldo, M, N, K, norm_w, eps, rows, q, rem);
+  return ms_launch_status();
+}
+
+template <int EPI, typename TO, bool NORM>
+int plan(const void* A, size_t lda, const bf16* W, size_t ldw, const float* bias, TO* out, size_t ldo, int M, int N,
+         int K, const float* norm_w, float eps, const int* rows, bool any_shape, hipStream_t stream) {
+  const int cus = ms_compute_units();
+  const int tiles = (N + 15) / 16;
+  // Where this kernel wins over ms_gemm_skinny, by measurement: more than 16 tokens and at least a tile of W
+  // for every CU (with fewer blocks than CUs the panel, which every block loads whole, costs more than it saves).
+  if (!any_shape && (M <= 16 || tiles < cus)) return MS_UNSUPPORTED;
+  const int tt = (M + 15) / 16;
+  const int S = (K + 31) / 32;
+  if ((K / 8 + 63) / 64 > MAX_PARTS) return MS_UNSUPPORTED;
+  size_t lds = (size_t)M * (S * 4 + 1) * 16;
+  if (lds > (size_t)LDS_BUDGET) return MS_UNSUPPORTED;   // the panel has to fit whole
+  const size_t red = (size_t)WAVES * tt * MS_WAVE * 16;
+  if (lds < red) lds = red;
+  const int blocks = tiles < cus ? tiles : cus;
+  const int q = tiles / blocks, rem = tiles % blocks;
+#define GO(TTV) if (tt == TTV) return launch<TTV, EPI, TO, NORM>(A, lda, W, ldw, bias, out, ldo, M, N, K, norm_w, eps, rows, blocks, q, rem, lds, stream)
+  GO(1); GO(2); GO(3); GO(4);
+#undef GO
+  return MS_UNSUPPORTED;
+}
+
+}  // namespace
+
+// The product of up to 64 rows with W[N,K]^T, the rows held whole in LDS.  norm = 0: A is bfloat16 [M, lda];
+// norm = 1: A is the float residual stream and the RMS norm (norm_w[K], eps) is folded in; rows (int32 [M], may
+// be null) gathers the rows of A.
+// epilogue 0: out[M,N] (out_dtype float or bfloat16) = product + bias
+// epilogue 1: out[M,N/2] bfloat16 = silu(gate) * up over interleaved rows of W (no bias)
+// epilogue 3: out[M,N] float += product + bias (not with norm)
+// MS_UNSUPPORTED for shapes it does not take (the caller then uses ms_gemm_skinny): with any_shape = 0 all but
+// those it is the faster kernel for; with any_shape = 1 (tests, measurements) only those it cannot compute
+// (rows that do not fit LDS whole: M * (K + 40) * 2 bytes over 144 KB, or K over 2048).
+extern "C" int ms_gemm_panel(const void* A, long long lda, const int* rows, const float* norm_w, float eps,
+                             const void* W, long long ldw, const float* bias, void* out, long long ldo, int M, int N,
+                             int K, int epilogue, int out_dtype, int norm, int any_shape, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return MS_OK;
+  if (M > MAX_TOKENS) return MS_UNSUPPORTED;
+  if (K <= 0 || K % 8 || ldw % 8 || lda < K || ldw < K || lda % (norm ? 4 : 8)) return MS_UNSUPPORTED;
+  if (((uintptr_t)A | (uintptr_t)W) % 16 || (norm && ((uintptr_t)norm_w % 16))) return MS_UNSUPPORTED;
+  if (norm && !norm_w) return MS_BAD_ARG;
+  const bf16* w = (const bf16*)W;
+#define RUN(EPI, TO, NORMV) return plan<EPI, TO, NORMV>(A, lda, w, ldw, bias, (TO*)out, ldo, M, N, K, norm_w, eps, rows, any_shape != 0, stream)
+  if (epilogue == EPI_STORE) {
+    if (ldo < N) return MS_BAD_ARG;
+    if (out_dtype == MS_BF16) { if (norm) RUN(EPI_STORE, bf16, true); else RUN(EPI_STORE, bf16, false); }
+    if (out_dtype == MS_F32) { if (norm) RUN(EPI_STORE, float, true); else RUN(EPI_STORE, float, false); }
+    return MS_BAD_ARG;
+  }
+  if (epilogue == EPI_SWIGLU) {
+    if (N % 2 || ldo < N / 2 || out_dtype != MS_BF16 || bias) return MS_BAD_ARG;
+    if (norm) RUN(EPI_SWIGLU, bf16, true); else RUN(EPI_SWIGLU, bf16, false);
+  }
+  if (epilogue == EPI_RESIDUAL) {
+    if (ldo < N || out_dtype != MS_F32 || norm) return MS_BAD_ARG;
+    RUN(EPI_RESIDUAL, float, false);
+  }
+#undef RUN
+  return MS_BAD_ARG;
+}

@@ -258,6 +258,10 @@ extern "C" int ms_gemm_skinny(const void* A, long long lda, const void* W, long 
     const int rc = ms_gemm_stream(A, lda, nullptr, nullptr, 0.f, W, ldw, bias, out, ldo, M, N, K, epilogue, out_dtype, 0, 0, stream);
     if (rc != MS_UNSUPPORTED) return rc;
   }
+  if (M > 16 && !forced()) {    // several: the kernel that holds the activations in LDS, where it takes the shape
+    const int rc = ms_gemm_panel(A, lda, nullptr, nullptr, 0.f, W, ldw, bias, out, ldo, M, N, K, epilogue, out_dtype, 0, 0, stream);
+    if (rc != MS_UNSUPPORTED) return rc;
+  }
   if (K <= 0 || K % 8 || lda % 8 || ldw % 8 || lda < K || ldw < K) return MS_UNSUPPORTED;
   if (((uintptr_t)A | (uintptr_t)W) % 16) return MS_UNSUPPORTED;
   const bf16* w = (const bf16*)W;
@@ -288,6 +292,10 @@ extern "C" int ms_gemm_skinny_norm(const float* x, long long ldx, const int* row
   if (M > 64) return MS_UNSUPPORTED;
   if (M <= 16 && !forced()) {
     const int rc = ms_gemm_stream(x, ldx, rows, norm_w, eps, W, ldw, bias, out, ldo, M, N, K, epilogue, out_dtype, 1, 0, stream);
+    if (rc != MS_UNSUPPORTED) return rc;
+  }
+  if (M > 16 && !forced()) {
+    const int rc = ms_gemm_panel(x, ldx, rows, norm_w, eps, W, ldw, bias, out, ldo, M, N, K, epilogue, out_dtype, 1, 0, stream);
     if (rc != MS_UNSUPPORTED) return rc;
   }
   if (K <= 0 || K % 8 || ldx % 4 || ldw % 8 || ldx < K || ldw < K) return MS_UNSUPPORTED;

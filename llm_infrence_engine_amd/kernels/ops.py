@@ -32,6 +32,8 @@ _SIGNATURES = {
                        _c_ptr],
     "ms_gemm_stream": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int,
                        _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "ms_gemm_panel": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int,
+                      _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "ms_residual_add": [_c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr],
     "ms_silu_mul": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "ms_rope_store": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int,
@@ -337,14 +339,9 @@ def gemm_skinny_norm(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w: 
 STREAM_MAX_ROWS = 16
 
 
-def gemm_stream(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, epilogue: int = EPI_STORE,
-                out_dtype: torch.dtype = torch.bfloat16, residual: Optional[torch.Tensor] = None,
-                norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0,
-                rows: Optional[torch.Tensor] = None, any_shape: bool = True) -> torch.Tensor:
-    """The streaming kernel for up to 16 rows, called by name (``gemm_skinny`` and ``gemm_skinny_norm`` go to it by
-    themselves for the shapes it is faster on): ``a`` bfloat16 [M, K], or with ``norm_weight`` the float32
-    residual stream whose RMS norm is folded in.  With ``any_shape`` every shape it can compute is taken;
-    a shape it cannot raises."""
+def _gemm_by_name(entry: str, a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], epilogue: int,
+                  out_dtype: torch.dtype, residual: Optional[torch.Tensor], norm_weight: Optional[torch.Tensor],
+                  eps: float, rows: Optional[torch.Tensor], any_shape: bool) -> torch.Tensor:
     norm = norm_weight is not None
     _check(a, "a", torch.float32 if norm else torch.bfloat16, contiguous=False)
     _check(w, "w", torch.bfloat16)
@@ -368,10 +365,34 @@ def gemm_stream(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] =
         out, ldo, out_dtype = residual, N, torch.float32
     else:
         raise ValueError(f"unknown epilogue {epilogue}")
-    _call("ms_gemm_stream", a.data_ptr(), a.stride(0) if a.shape[0] > 1 else K, _ptr(rows), _ptr(norm_weight), float(eps),
+    _call(entry, a.data_ptr(), a.stride(0) if a.shape[0] > 1 else K, _ptr(rows), _ptr(norm_weight), float(eps),
           w.data_ptr(), K, _ptr(bias), out.data_ptr(), ldo, M, N, K, epilogue, _code(out_dtype), int(norm),
           int(any_shape), _stream())
     return out
+
+
+def gemm_stream(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, epilogue: int = EPI_STORE,
+                out_dtype: torch.dtype = torch.bfloat16, residual: Optional[torch.Tensor] = None,
+                norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0,
+                rows: Optional[torch.Tensor] = None, any_shape: bool = True) -> torch.Tensor:
+    """The streaming kernel for up to 16 rows, called by name (``gemm_skinny`` and ``gemm_skinny_norm`` go to it by
+    themselves for the shapes it is faster on): ``a`` bfloat16 [M, K], or with ``norm_weight`` the float32
+    residual stream whose RMS norm is folded in.  With ``any_shape`` every shape it can compute is taken;
+    a shape it cannot raises."""
+    return _gemm_by_name("ms_gemm_stream", a, w, bias, epilogue, out_dtype, residual, norm_weight, eps, rows, any_shape)
+
+
+PANEL_MAX_ROWS = 64
+
+
+def gemm_panel(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, epilogue: int = EPI_STORE,
+               out_dtype: torch.dtype = torch.bfloat16, residual: Optional[torch.Tensor] = None,
+               norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0,
+               rows: Optional[torch.Tensor] = None, any_shape: bool = True) -> torch.Tensor:
+    """The kernel that keeps up to 64 rows of activations whole in LDS, called by name (``gemm_skinny`` and
+    ``gemm_skinny_norm`` go to it by themselves for more than 16 rows against a matrix of many rows).  Arguments
+    as for ``gemm_stream``; a shape it cannot compute (rows that do not fit LDS) raises."""
+    return _gemm_by_name("ms_gemm_panel", a, w, bias, epilogue, out_dtype, residual, norm_weight, eps, rows, any_shape)
 
 
 def qkv_rope_store_ok(x: torch.Tensor, w: torch.Tensor, head_dim: int, rot_dim: int) -> bool:

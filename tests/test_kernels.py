@@ -394,6 +394,71 @@ def test_gemm_stream_refuses_what_it_cannot_take(ops):
         ops.gemm_stream(torch.zeros(2, 64, dtype=torch.bfloat16, device=DEV), w, any_shape=False)
 
 
+@pytest.mark.parametrize("M", [17, 32, 41, 64])
+@pytest.mark.parametrize("N,K", [(7000, 96), (4100, 200), (330, 256), (48, 896), (16 * 256 * 17 + 6, 64), (1000, 1000)])
+def test_gemm_panel(ops, M, N, K):
+    """The kernel that holds the activations in LDS, at every shape it can compute: blocks of one tile, of a few
+    tiles whose k-steps several waves share, and of more tiles than waves; a last k-step that K fills in part;
+    rows of W that run out inside the last tile; every epilogue, the folded norm with gathered rows; a row's
+    numbers do not depend on the rest of the batch."""
+    g = torch.Generator().manual_seed(M * 1000 + N + K)
+    a = torch.randn(M, K, generator=g).bfloat16().to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16().to(DEV)
+    bias = torch.randn(N, generator=g).to(DEV)
+    want = a.double() @ w.double().T
+    out = ops.gemm_panel(a, w, bias)
+    torch.testing.assert_close(out.double(), want + bias.double(), **tol(torch.bfloat16))
+    f = ops.gemm_panel(a, w, None, out_dtype=torch.float32)
+    torch.testing.assert_close(f.double(), want, atol=3e-5, rtol=3e-5)
+    x = torch.randn(M, N, generator=g).to(DEV)
+    x0 = x.clone()
+    ops.gemm_panel(a, w, bias, ops.EPI_RESIDUAL, residual=x)
+    torch.testing.assert_close(x.double(), x0.double() + want + bias.double(), atol=3e-5, rtol=3e-5)
+    act = ops.gemm_panel(a, w, None, ops.EPI_SWIGLU)
+    torch.testing.assert_close(act.double(), torch.nn.functional.silu(want[:, 0::2]) * want[:, 1::2], **tol(torch.bfloat16))
+    assert torch.equal(ops.gemm_panel(a[M - 3:], w, bias), out[M - 3:])
+    # the folded norm over gathered rows of a taller residual stream
+    xs = torch.randn(M + 3, K, generator=g).to(DEV)
+    nw = (1 + 0.1 * torch.randn(K, generator=g)).to(DEV)
+    rows = torch.randperm(M + 3, generator=g)[:M].to(torch.int32).to(DEV)
+    xr = xs[rows.long()].double()
+    h = (xr * nw.double()).float().bfloat16().double() * torch.rsqrt((xr * xr).mean(-1, keepdim=True) + 1e-5)
+    got = ops.gemm_panel(xs, w, bias, out_dtype=torch.float32, norm_weight=nw, eps=1e-5, rows=rows)
+    torch.testing.assert_close(got.double(), h @ w.double().T + bias.double(), atol=2e-4, rtol=2e-4)
+    gated = ops.gemm_panel(xs, w, None, ops.EPI_SWIGLU, norm_weight=nw, eps=1e-5, rows=rows)
+    hw = h @ w.double().T
+    torch.testing.assert_close(gated.double(), torch.nn.functional.silu(hw[:, 0::2]) * hw[:, 1::2], **tol(torch.bfloat16))
+
+
+@pytest.mark.parametrize("M,N,K", [(20, 300, 1200), (33, 4100, 1528), (18, 500, 2040)])
+def test_gemm_panel_long_rows(ops, M, N, K):
+    """Rows of three and four 512-column parts (with three a quarter of the waves sit the loading out)."""
+    g = torch.Generator().manual_seed(K)
+    xs = torch.randn(M, K, generator=g).to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16().to(DEV)
+    nw = (1 + 0.1 * torch.randn(K, generator=g)).to(DEV)
+    h = (xs.double() * nw.double()).float().bfloat16().double() * torch.rsqrt((xs.double() ** 2).mean(-1, keepdim=True) + 1e-6)
+    got = ops.gemm_panel(xs, w, None, out_dtype=torch.float32, norm_weight=nw, eps=1e-6)
+    torch.testing.assert_close(got.double(), h @ w.double().T, atol=2e-4, rtol=2e-4)
+    a = xs.bfloat16()
+    plain = ops.gemm_panel(a, w, None, out_dtype=torch.float32)
+    torch.testing.assert_close(plain.double(), a.double() @ w.double().T, atol=3e-5, rtol=3e-5)
+
+
+def test_gemm_panel_refuses_what_it_cannot_take(ops):
+    w = torch.zeros(64, 64, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(RuntimeError, match="unsupported"):
+        ops.gemm_panel(torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV), w)             # more than 64 rows
+    with pytest.raises(RuntimeError, match="unsupported"):                                   # rows that do not fit LDS
+        ops.gemm_panel(torch.zeros(64, 1600, dtype=torch.bfloat16, device=DEV),
+                       torch.zeros(64, 1600, dtype=torch.bfloat16, device=DEV))
+    with pytest.raises(RuntimeError, match="unsupported"):
+        ops.gemm_panel(torch.zeros(20, 4096, dtype=torch.bfloat16, device=DEV),
+                       torch.zeros(64, 4096, dtype=torch.bfloat16, device=DEV))              # K beyond its loads
+    with pytest.raises(RuntimeError, match="unsupported"):                                   # not the shape it is for
+        ops.gemm_panel(torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV), w, any_shape=False)
+
+
 def test_gemm_skinny_refuses_what_it_cannot_take(ops):
     a = torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV)
     w = torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV)
