@@ -560,6 +560,21 @@ def test_paged_attention_mfma(ops, nh, nkv, d, page_size, window, shape):
     torch.testing.assert_close(out2.double().cpu(), want, **tol(torch.bfloat16))
 
 
+@pytest.mark.parametrize("R,nh,nkv,d,window", [(40, 6, 2, 64, None), (64, 4, 2, 32, None), (21, 8, 4, 128, 700)])
+def test_split_decode_attention_of_a_large_uneven_batch(ops, R, nh, nkv, d, window):
+    """Many requests whose contexts differ widely, some far beyond the length from which keys are split over
+    blocks: few splits per request (a number that is no power of two), short requests that use one of them."""
+    g = torch.Generator().manual_seed(R)
+    ctx = [int(v) for v in torch.randint(1, 1500, (R,), generator=g)]
+    ctx[3], ctx[R - 1] = 2300, 1
+    qlen = [1] * R
+    assert ops.attention_splits_keys(R, nkv, nh // nkv, 1, max(ctx))
+    c = _paged_case(g, torch.bfloat16, nh, nkv, d, 16, ctx, qlen, float("nan"))
+    want = torch.cat([attention_reference(q.double(), k.double(), v.double(), 1.0 / math.sqrt(d), window).transpose(0, 1).reshape(-1, nh * d)
+                      for q, k, v in zip(c["qs"], c["ks"], c["vs"])])
+    torch.testing.assert_close(_run_mfma(ops, c, nh, d, ctx, qlen, window), want, **tol(torch.bfloat16))
+
+
 def _run_mfma(ops, c, nh, d, ctx, qlen, window=None):
     N = c["q"].shape[0]
     out = torch.full((N, nh * d), float("nan"), dtype=torch.bfloat16, device=DEV)
