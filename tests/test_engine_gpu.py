@@ -247,6 +247,42 @@ def test_long_context_decode_splits_keys_and_matches_plain(eng, tmp_path):
             assert sorted(r.graphs.buckets) == [(2, False), (2, True)]   # it crossed from short to long on the way
 
 
+def test_large_uneven_decode_batch_matches_plain(eng, tmp_path):
+    """36 requests with contexts of 20 to 1,150 tokens decode together at the layer widths of the half-billion
+    model (two layers, a vocabulary of 4,128): the products for 17 to 64 tokens, attention over many requests of
+    which some pass the length from which keys are split over blocks, prompts in portions beside each other."""
+    from llm_infrence_engine_amd.config import config_from_dict
+    from llm_infrence_engine_amd.engine import StepEntry, load_runner
+
+    cfg = {"architectures": ["Qwen2ForCausalLM"], "num_hidden_layers": 2, "hidden_size": 896, "num_attention_heads": 14,
+           "num_key_value_heads": 2, "intermediate_size": 4864, "vocab_size": 4128, "rope_theta": 1000000.0,
+           "rms_norm_eps": 1e-6, "tie_word_embeddings": True}
+    d = tmp_path / "m"
+    eng.write_random_model(d, config_from_dict(cfg), seed=1, dtype="bfloat16", std=0.05)
+    pc, w = P.read_config(d), P.read_weights(d, torch.float64)
+    rng = np.random.default_rng(1)
+    R, tail = 36, 2
+    seqs = {f"r{i}": [int(t) for t in rng.integers(0, 4128, n)] for i, n in enumerate(rng.integers(20, 1151, R))}
+    seqs["r5"] = seqs["r5"] + seqs["r6"][:1150 - len(seqs["r5"])]   # one of them as long as it gets
+    exact = {r: P.forward(w, pc, t)[-tail:].numpy() for r, t in seqs.items()}
+    noise = {r: np.abs(P.forward(w, pc, t, act_dtype=torch.bfloat16)[-tail:].numpy() - exact[r]).max() for r, t in seqs.items()}
+    runner = load_runner(d, dtype="bfloat16", page_size=16, max_requests=R, max_len=1168)
+    done = {r: 0 for r in seqs}
+    while any(done[r] < len(seqs[r]) - tail for r in seqs):     # portions of up to 500 tokens, 2,048 to a step
+        entries, left = [], 2048
+        for r, t in seqs.items():
+            n = min(len(t) - tail - done[r], left, int(rng.integers(1, 500)))
+            if n > 0:
+                entries.append(StepEntry(r, t[done[r]:done[r] + n], []))
+                done[r] += n
+                left -= n
+        runner.step(entries)
+    for k in range(tail):
+        lg = runner.step([StepEntry(r, [t[len(t) - tail + k]], [0]) for r, t in seqs.items()]).float().cpu().numpy()
+        for row, r in zip(lg, seqs):
+            assert np.abs(row - exact[r][k]).max() < 3.0 * noise[r], (r, len(seqs[r]), k)
+
+
 def test_several_decode_steps_per_launch_change_nothing(tiny, eng):
     """Up to 8 decode steps queued in one graph launch (tokens fed back on the device): the same outputs as step
     by step, also when a stop id arrives in the middle of a launch, a request joins, or pages are scarce."""
