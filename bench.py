@@ -145,9 +145,13 @@ def run_serving(eng_mod, model, vocab, seed, n_requests=64, new_tokens=256, lo=1
     dt = time.perf_counter() - t0
     made = sum(len(r.output_ids) for r in reqs)
     mixed = sum(1 for rec in e.steps if rec.n_prefill_tokens and rec.decode_batch)
+    s = eng_mod.engine.summarize(reqs, e.steps, dt)
     return {"seconds": round(dt, 3), "requests": n_requests, "prompt_tokens": sum(lens), "new_tokens": made,
             "new_tokens_per_s": round(made / dt, 1), "all_tokens_per_s": round((sum(lens) + made) / dt, 1),
-            "launches": len(e.steps), "mixed_launches": mixed, "preemptions": e.preemptions}
+            "launches": len(e.steps), "mixed_launches": mixed, "preemptions": e.preemptions,
+            "ttft_p50_s": round(s["ttft_p50_s"], 4), "ttft_p95_s": round(s["ttft_p95_s"], 4),
+            "tpot_mean_ms": round(s["tpot_mean_ms"], 3), "mean_decode_batch": round(s["mean_decode_batch"], 1),
+            "wasted_row_fraction": round(s["wasted_row_fraction"], 4)}
 
 
 def main() -> int:

@@ -59,6 +59,32 @@ def test_greedy_generation_matches_plain(tiny, eng):
     assert len(r.step_times) == n_new - 1 and r.cache_bytes > 0
 
 
+def test_run_summary_of_continuous_batching(tiny, eng):
+    """Requests of very different lengths: no decode row is computed for nothing (tests/test_batching.py:108-113
+    of the reference); a launch of several steps that runs past a short request's end does waste rows."""
+    import time
+
+    from llm_infrence_engine_amd.engine import summarize
+
+    name, d, cfg, w = tiny
+    model = eng.load_model(d, "float32", "cuda:0")
+    prompts = prompts_for(name, cfg["vocab_size"])
+    lens = [3, 12, 5, 8][:len(prompts)]
+    for per_launch in (1, 4):
+        e = eng.Engine(model, block_size=8, max_len=64, max_seqs=4, hip_graphs=per_launch > 1,
+                       decode_steps_per_launch=per_launch)
+        reqs = [eng.Request(p, max_new_tokens=n) for p, n in zip(prompts, lens)]
+        t0 = time.perf_counter()
+        for r in reqs:
+            e.add_request(r)
+        e.run_until_idle()
+        s = summarize(reqs, e.steps, time.perf_counter() - t0)
+        assert s["requests"] == len(reqs) and s["output_tokens"] == sum(lens)
+        assert s["wasted_row_fraction"] == 0.0        # launches of several steps never run past a request's budget
+        assert 0 < s["ttft_p50_s"] <= s["ttft_p95_s"] <= s["e2e_p95_s"]
+        assert s["throughput_tok_s"] > 0 and 1.0 <= s["mean_decode_batch"] <= len(reqs)
+
+
 def test_stop_id_is_not_emitted(tiny, eng):
     name, d, cfg, w = tiny
     p = prompts_for(name, cfg["vocab_size"])[1]
