@@ -24,6 +24,7 @@ Only decisions and bookkeeping live here: no tensors, so it runs (and is tested)
 from __future__ import annotations
 
 import random
+import threading
 import time
 from collections import deque
 from typing import Callable, Deque, List, Optional
@@ -46,6 +47,9 @@ class Scheduler:
         self._next_id = 0
         self._admit_counter = 0
         self._seed_rng = random.Random()
+        # add_request and cancel may be called from another thread than the one that steps
+        # (src/miniserve/engine.py:136, 149): ids and the waiting queue change under this lock
+        self._lock = threading.Lock()
 
     # ------------------------------------------------------------------ public
     def add_request(self, req: Request) -> Request:
@@ -56,12 +60,13 @@ class Scheduler:
             raise ValueError(f"request needs {need} cache positions but max_len is {self.config.max_len}")
         if need > self.manager.num_pages * self.manager.page_size:
             raise ValueError("request can never fit in the page pool")
-        req.id = self._next_id
-        self._next_id += 1
-        req.arrival_time = self.clock()
-        req.state = "waiting"
-        req.sample_seed = req.seed if req.seed is not None else self._seed_rng.getrandbits(62)
-        self.waiting.append(req)
+        with self._lock:
+            req.id = self._next_id
+            self._next_id += 1
+            req.arrival_time = self.clock()
+            req.state = "waiting"
+            req.sample_seed = req.seed if req.seed is not None else self._seed_rng.getrandbits(62)
+            self.waiting.append(req)
         return req
 
     def has_work(self) -> bool:
@@ -191,8 +196,11 @@ class Scheduler:
 
     def _reap_cancelled(self) -> None:
         now = self.clock()
-        for r in [r for r in self.waiting if r.cancelled]:
-            self.waiting.remove(r)
+        with self._lock:
+            dropped = [r for r in self.waiting if r.cancelled]
+            for r in dropped:
+                self.waiting.remove(r)
+        for r in dropped:
             self._finish(r, "abort", now)
         for r in [r for r in self.running if r.cancelled]:
             self._finish(r, "abort", now)

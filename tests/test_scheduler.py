@@ -196,3 +196,43 @@ def test_random_arrivals_under_pressure(seed):
     drain(s, m)
     assert [r.output_ids for r in reqs] == want
     assert all(g.allocator.num_in_use() == 0 for g in m.groups)
+
+
+def test_requests_may_arrive_and_be_cancelled_from_other_threads():
+    """add_request and cancel from threads of their own while this one steps (the reference's server does so,
+    src/miniserve/engine.py:136-161): ids stay unique, nothing is lost, outputs are those of each request alone."""
+    import threading
+
+    s, m = make(num_pages=40, page_size=4, max_seqs=4, max_len=48, budget=16)
+    ps = prompts(3, [5, 9, 2, 14, 7, 3, 11, 6] * 5)
+    reqs, stop = [], threading.Event()
+    lock = threading.Lock()
+
+    def feed(mine):
+        for p in mine:
+            r = s.add_request(Request(p, max_new_tokens=6))
+            with lock:
+                reqs.append(r)
+
+    feeders = [threading.Thread(target=feed, args=(ps[i::4],)) for i in range(4)]
+    for t in feeders:
+        t.start()
+    steps = 0
+    while any(t.is_alive() for t in feeders) or s.has_work():
+        if s.has_work():
+            one_step(s, m)
+            steps += 1
+            if steps == 3:
+                with lock:
+                    victim = reqs[-1]
+                threading.Thread(target=s.cancel, args=(victim,)).start()
+        assert steps < 5000
+    for t in feeders:
+        t.join()
+    assert len(reqs) == len(ps) and sorted(r.id for r in reqs) == list(range(len(ps)))
+    for r in reqs:
+        if r.finish_reason == "abort":
+            assert r is victim
+        else:
+            assert r.output_ids == alone(r.prompt_ids, 6)
+    assert all(g.allocator.num_in_use() == 0 for g in m.groups)
