@@ -6,7 +6,9 @@ Default run: the layer sizes of the Qwen2.5-0.5B configuration with random weigh
 of 8 requests with 512-token prompts, K timed decode steps through the whole engine (scheduler, step
 function, sampler).  One JSON line is printed: ``value`` is decoded tokens a second; ``prefill`` is one
 2,048-token prompt in one step; ``roofline`` prices the decode step against HBM bandwidth (every weight it
-uses once plus the cache of the live requests); ``points`` holds decode throughput at batch 1 and 64.
+uses once plus the cache of the live requests); ``points`` holds decode throughput at batch 1 and 64;
+``launch`` says how many decode steps one graph launch holds and what it costs the host to enqueue it against
+the whole launch (a step bound by launching would show the two close together).
 """
 from __future__ import annotations
 
@@ -91,12 +93,20 @@ def run_decode(eng_mod, model, batch, steps, warmup, vocab, seed, prompt_len=PRO
 
     run(warmup)
     assert len(e.running) == batch and all(r.num_tokens - r.num_computed == 1 for r in e.running)
+    graphs = e.runner.graphs
     torch.cuda.synchronize()
+    q0, n0 = graphs.enqueue_seconds, graphs.launches
     t0 = time.perf_counter()
     run(steps)
     torch.cuda.synchronize()
-    dt = (time.perf_counter() - t0) / steps
+    total = time.perf_counter() - t0
+    dt = total / steps
     mean_context = prompt_len + warmup + (steps + 1) / 2
+    launches = graphs.launches - n0
+    # the host's share: filling the static buffers and enqueuing the graph, against the whole launch
+    run_decode.launch = {"steps_per_launch": round(steps / launches, 2),
+                         "enqueue_ms": round((graphs.enqueue_seconds - q0) / launches * 1e3, 4),
+                         "total_ms": round(total / launches * 1e3, 4)}
     return dt, mean_context
 
 
@@ -201,6 +211,7 @@ def main() -> int:
         return 0
 
     dt, ctx = run_decode(eng, model, a.batch, a.steps, a.warmup, vocab, seed=1, prompt_len=a.prompt_len)
+    launch = run_decode.launch
     value = a.batch / dt
     gbs = decode_bytes(cfg, a.batch, ctx) / dt / 1e9
     out = {
@@ -220,6 +231,7 @@ def main() -> int:
         },
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_GBS, 4)},
+        "launch": launch,
     }
     if not a.no_points:
         pt = run_prefill(eng, model, vocab, seed=2)

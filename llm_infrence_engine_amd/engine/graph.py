@@ -16,6 +16,7 @@ on the device, so the host is needed once per launch instead of once per step.
 """
 from __future__ import annotations
 
+import time
 from typing import Dict, List, Optional, Sequence
 
 import numpy as np
@@ -93,6 +94,10 @@ class DecodeGraphs:
         self.sizes = sorted(set(batch_sizes or default_batch_sizes(m.max_requests)))
         self.width = m.max_pages_per_request
         self.buckets: Dict[int, _Bucket] = {}
+        # what launching costs the host: seconds spent filling the buffers and enqueuing, and launches so far
+        # (the reference separates a launch-bound from a GPU-bound step the same way, benchmarks/diag_gpu_launch.py:1-8)
+        self.enqueue_seconds = 0.0
+        self.launches = 0
 
     @property
     def max_batch(self) -> int:
@@ -153,6 +158,7 @@ class DecodeGraphs:
         """``steps`` decode steps for ``entries`` (one token each, pages already grown for all the steps).
         Returns (logits [R, V] of the last step, greedy tokens int32 [steps, R]); both are views of static
         buffers that the next replay overwrites."""
+        t_begin = time.perf_counter()
         m = self.manager
         R = len(entries)
         rows = np.fromiter((m.row(e.req_id) for e in entries), dtype=np.int32, count=R)
@@ -182,4 +188,6 @@ class DecodeGraphs:
             a[bk.slots[g]][:R] = page * ps + pos % ps
         bk.dev.copy_(bk.host, non_blocking=True)
         bk.graph.replay()
+        self.enqueue_seconds += time.perf_counter() - t_begin
+        self.launches += 1
         return bk.logits[:R], bk.tokens[:, :R]
