@@ -239,6 +239,64 @@ def test_sample_greedy_and_vectors(ops):
     assert out.tolist() == big.argmax(-1).tolist()
 
 
+def test_argmax_in_two_stages(ops):
+    """Ties across and inside the slices of the first stage go to the smallest index; a row of -inf or NaN gives
+    index 0; vocabularies that are no multiple of the slice count."""
+    for V in (1000, 4097, 151936, 200003):
+        lg = torch.zeros(6, V, device=DEV)
+        lg[0, V - 1] = 1.0
+        lg[1, [V // 3, V // 3 + 1, V - 2]] = 2.0            # the first of three equal maxima
+        lg[2, :] = -5.0                                      # all equal: index 0
+        lg[3, :] = float("-inf")
+        lg[4, :] = float("nan")
+        lg[5, [7, V // 2]] = torch.tensor([3.0, 3.0], device=DEV)
+        out = torch.full((6,), -1, dtype=torch.int32, device=DEV)
+        ops.sample(lg, out)
+        assert out.tolist() == [V - 1, V // 3, 0, 0, 0, 7], V
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_bias_add_and_residual_add(ops, dtype):
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(7, 331, generator=g).to(dtype).to(DEV)
+    b = torch.randn(331, generator=g).to(DEV)
+    want = (x.double() + b.double())
+    ops.bias_add(x, b)
+    torch.testing.assert_close(x.double(), want, **tol(dtype))
+    stream = torch.randn(7, 331, generator=g).to(DEV)
+    delta = torch.randn(7, 331, generator=g).to(dtype).to(DEV)
+    want = stream.double() + delta.double()
+    ops.residual_add(stream, delta)
+    torch.testing.assert_close(stream.double(), want, atol=1e-6, rtol=1e-6)   # the sum itself is float
+
+
+@pytest.mark.parametrize("page_size", [4, 16, 48])
+def test_decode_advance(ops, page_size):
+    """Between two decode steps of one launch: live rows move on by one position, take the token just chosen and
+    get their slot from their block table (also across a page's edge, in every cache group); other rows stay."""
+    g = torch.Generator().manual_seed(page_size)
+    R, width, live = 9, 6, 6
+    pos = torch.tensor([0, page_size - 2, page_size - 1, 2 * page_size - 1, 3 * page_size + 1, 5, 7, 8, 9], dtype=torch.int32)
+    tables = [torch.randint(1, 500, (R, width), generator=g, dtype=torch.int32) for _ in range(2)]
+    prev = torch.randint(0, 1000, (R,), generator=g, dtype=torch.int32)
+    toks = torch.randint(0, 1000, (R,), generator=g, dtype=torch.int32)
+    ctx = pos + 1
+    slots = [torch.full((R,), -7, dtype=torch.int32) for _ in range(2)]
+    dev = lambda t: t.clone().to(DEV)
+    d_tok, d_pos, d_ctx, d_slots = dev(toks), dev(pos), dev(ctx), [dev(s_) for s_ in slots]
+    ops.decode_advance(dev(prev), d_tok, d_pos, d_ctx, torch.tensor([live], dtype=torch.int32, device=DEV),
+                       [dev(t) for t in tables], d_slots, page_size)
+    for r in range(R):
+        if r < live:
+            p = int(pos[r]) + 1
+            assert (int(d_pos[r]), int(d_ctx[r]), int(d_tok[r])) == (p, p + 1, int(prev[r]))
+            for t, s_ in zip(tables, d_slots):
+                assert int(s_[r]) == int(t[r, p // page_size]) * page_size + p % page_size
+        else:
+            assert (int(d_pos[r]), int(d_ctx[r]), int(d_tok[r])) == (int(pos[r]), int(ctx[r]), int(toks[r]))
+            assert all(int(s_[r]) == -7 for s_ in d_slots)
+
+
 def _draws(ops, logits, n, temperature=1.0, top_k=0, top_p=1.0, seed=0):
     M = n
     lg = logits.to(DEV).expand(M, -1).contiguous()
