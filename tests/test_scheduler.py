@@ -202,6 +202,7 @@ def test_requests_may_arrive_and_be_cancelled_from_other_threads():
     """add_request and cancel from threads of their own while this one steps (the reference's server does so,
     src/miniserve/engine.py:136-161): ids stay unique, nothing is lost, outputs are those of each request alone."""
     import threading
+    import time
 
     s, m = make(num_pages=40, page_size=4, max_seqs=4, max_len=48, budget=16)
     ps = prompts(3, [5, 9, 2, 14, 7, 3, 11, 6] * 5)
@@ -223,8 +224,12 @@ def test_requests_may_arrive_and_be_cancelled_from_other_threads():
             one_step(s, m)
             steps += 1
             if steps == 3:
-                with lock:
-                    victim = reqs[-1]
+                while True:     # a feeder may have been interrupted between add_request and its note of it
+                    with lock:
+                        if reqs:
+                            victim = reqs[-1]
+                            break
+                    time.sleep(0.001)
                 threading.Thread(target=s.cancel, args=(victim,)).start()
         assert steps < 5000
     for t in feeders:
