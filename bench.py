@@ -69,7 +69,8 @@ def prefill_flops(cfg, tokens):
 
 
 def run_decode(eng_mod, model, batch, steps, warmup, vocab, seed, prompt_len=PROMPT_LEN):
-    """Prefill ``batch`` prompts, then time ``steps`` decode steps of the engine.  Returns seconds per step."""
+    """Prefill ``batch`` prompts, then time ``steps`` decode steps of the engine.  Returns seconds per step, the
+    mean context length of the timed steps, and what a graph launch cost the host against the whole launch."""
     import numpy as np
     import torch
 
@@ -104,10 +105,10 @@ def run_decode(eng_mod, model, batch, steps, warmup, vocab, seed, prompt_len=PRO
     mean_context = prompt_len + warmup + (steps + 1) / 2
     launches = graphs.launches - n0
     # the host's share: filling the static buffers and enqueuing the graph, against the whole launch
-    run_decode.launch = {"steps_per_launch": round(steps / launches, 2),
-                         "enqueue_ms": round((graphs.enqueue_seconds - q0) / launches * 1e3, 4),
-                         "total_ms": round(total / launches * 1e3, 4)}
-    return dt, mean_context
+    launch = {"steps_per_launch": round(steps / launches, 2),
+              "enqueue_ms": round((graphs.enqueue_seconds - q0) / launches * 1e3, 4),
+              "total_ms": round(total / launches * 1e3, 4)}
+    return dt, mean_context, launch
 
 
 def run_prefill(eng_mod, model, vocab, seed, repeats=5):
@@ -210,8 +211,7 @@ def main() -> int:
         print(json.dumps({"serving": run_serving(eng, model, vocab, seed=5)}), flush=True)
         return 0
 
-    dt, ctx = run_decode(eng, model, a.batch, a.steps, a.warmup, vocab, seed=1, prompt_len=a.prompt_len)
-    launch = run_decode.launch
+    dt, ctx, launch = run_decode(eng, model, a.batch, a.steps, a.warmup, vocab, seed=1, prompt_len=a.prompt_len)
     value = a.batch / dt
     gbs = decode_bytes(cfg, a.batch, ctx) / dt / 1e9
     out = {
@@ -241,7 +241,7 @@ def main() -> int:
         points = {}
         for b in (1, 64):
             steps = min(a.steps, 128)
-            dtb, _ = run_decode(eng, model, b, steps, min(a.warmup, 8), vocab, seed=3 + b)
+            dtb, _, _ = run_decode(eng, model, b, steps, min(a.warmup, 8), vocab, seed=3 + b)
             points[f"decode_b{b}"] = round(b / dtb, 1)
         out["points"] = points
     print(json.dumps(out), flush=True)
