@@ -5,7 +5,7 @@ Same figures and names as the reference's summary (src/miniserve/metrics.py:10-4
 """
 from __future__ import annotations
 
-from typing import Dict, Iterable, List, Optional, Sequence
+from typing import Dict, List, Sequence
 
 from .request import Request, StepRecord
 
@@ -30,8 +30,9 @@ def _mean(values: List[float]) -> float:
     return sum(values) / len(values) if values else NAN
 
 
-def _known(values: Iterable[Optional[float]]) -> List[float]:
-    return [v for v in values if v is not None]
+def _timings(done: Sequence[Request], field: str) -> List[float]:
+    """One timing property of every finished request that has it."""
+    return [v for v in (getattr(r, field) for r in done) if v is not None]
 
 
 def summarize(requests: Sequence[Request], steps: Sequence[StepRecord], wall_time: float) -> Dict[str, float]:
@@ -41,27 +42,26 @@ def summarize(requests: Sequence[Request], steps: Sequence[StepRecord], wall_tim
     token: with continuous batching only the steps that a launch of several ran past a request's stop id).  A
     record that covers several decode steps of one launch counts its rows for each of them."""
     done = [r for r in requests if r.state == "finished"]
-    tokens = sum(len(r.output_ids) for r in done)
-    ttft, e2e = _known(r.ttft for r in done), _known(r.e2e for r in done)
-    tpot, wait = _known(r.tpot for r in done), _known(r.queue_wait for r in done)
-    decoding = [s for s in steps if s.decode_batch > 0]
-    launches = sum(max(1, s.decode_steps) for s in decoding)     # decode steps, several to a record at times
-    rows = sum(s.decode_batch * max(1, s.decode_steps) for s in decoding)
-    # a record's useful rows also count requests whose prompt ended in that step; those are no decode rows
-    useful = sum(min(s.useful_rows, s.decode_batch * max(1, s.decode_steps)) for s in decoding)
-    return {
-        "requests": len(done),
-        "output_tokens": tokens,
-        "wall_time_s": wall_time,
-        "throughput_tok_s": tokens / wall_time if wall_time > 0 else 0.0,
-        "ttft_mean_s": _mean(ttft),
-        "ttft_p50_s": percentile(ttft, 50),
-        "ttft_p95_s": percentile(ttft, 95),
-        "queue_wait_mean_s": _mean(wait),
-        "e2e_mean_s": _mean(e2e),
-        "e2e_p95_s": percentile(e2e, 95),
-        "tpot_mean_ms": 1000.0 * _mean(tpot),
-        "steps": len(steps),
-        "mean_decode_batch": rows / launches if launches else 0.0,
-        "wasted_row_fraction": 1.0 - useful / rows if rows else 0.0,
-    }
+    out: Dict[str, float] = {"requests": len(done), "output_tokens": sum(len(r.output_ids) for r in done),
+                             "wall_time_s": wall_time, "steps": len(steps)}
+    out["throughput_tok_s"] = out["output_tokens"] / wall_time if wall_time > 0 else 0.0
+
+    first = _timings(done, "ttft")
+    out.update(ttft_mean_s=_mean(first), ttft_p50_s=percentile(first, 50), ttft_p95_s=percentile(first, 95))
+    out["queue_wait_mean_s"] = _mean(_timings(done, "queue_wait"))
+    whole = _timings(done, "e2e")
+    out.update(e2e_mean_s=_mean(whole), e2e_p95_s=percentile(whole, 95))
+    out["tpot_mean_ms"] = 1000.0 * _mean(_timings(done, "tpot"))
+
+    n_steps = rows = useful = 0
+    for rec in steps:
+        if rec.decode_batch <= 0:
+            continue
+        k = max(1, rec.decode_steps)              # decode steps this record covers
+        n_steps += k
+        rows += rec.decode_batch * k
+        # a record's useful rows also count requests whose prompt ended in that step; those are no decode rows
+        useful += min(rec.useful_rows, rec.decode_batch * k)
+    out["mean_decode_batch"] = rows / n_steps if n_steps else 0.0
+    out["wasted_row_fraction"] = 1.0 - useful / rows if rows else 0.0
+    return out
