@@ -16,6 +16,7 @@ on the device, so the host is needed once per launch instead of once per step.
 """
 from __future__ import annotations
 
+import gc
 import time
 from typing import Dict, List, Optional, Sequence
 
@@ -145,13 +146,24 @@ class DecodeGraphs:
                 advance(1)
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
-        bk.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(bk.graph):
-            for k in range(bk.steps):
-                if k > 0:
-                    advance(k)
-                bk.logits = model.forward(ctx, caches)
-                ops.sample(bk.logits, bk.tokens[k])
+        # Nothing that owns device memory or graphs of its own (a runner that went out of use and waits in a
+        # reference cycle) may be finalised while the stream is capturing: giving device memory back is not
+        # allowed then, and the error, raised inside a destructor, ends the process.  So the collector runs
+        # now and stays off until the capture has ended.
+        gc.collect()
+        collecting = gc.isenabled()
+        gc.disable()
+        try:
+            bk.graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(bk.graph):
+                for k in range(bk.steps):
+                    if k > 0:
+                        advance(k)
+                    bk.logits = model.forward(ctx, caches)
+                    ops.sample(bk.logits, bk.tokens[k])
+        finally:
+            if collecting:
+                gc.enable()
         torch.cuda.synchronize()
 
     def run(self, entries: List[StepEntry], steps: int = 1):

@@ -246,6 +246,28 @@ def test_generation_with_hip_graphs(tiny, eng):
     assert llm.engine.runner.graphs.buckets
 
 
+def test_graph_capture_while_an_old_engine_waits_for_the_collector(tiny, eng):
+    """An engine with graphs of its own that went out of use inside a reference cycle is finalised before the
+    next capture starts, never during it (the collector is kept off while the stream captures)."""
+    import gc
+
+    name, d, cfg, w = tiny
+    prompts = prompts_for(name, cfg["vocab_size"])
+    want = eng.LLM(d, dtype="float32", block_size=8, max_len=64).generate(prompts, eng.SamplingParams(max_new_tokens=6))
+    old = gc.get_threshold()
+    try:
+        for _ in range(2):
+            llm = eng.LLM(d, dtype="float32", block_size=8, max_len=64, hip_graphs=True)
+            got = llm.generate(prompts, eng.SamplingParams(max_new_tokens=6))
+            assert [o.token_ids for o in got] == [o.token_ids for o in want]
+            llm.cycle = llm            # only the collector can free it and its graphs now
+            del llm, got
+            gc.set_threshold(50, 2, 2)   # the collector runs often from here on, the oldest generation too
+    finally:
+        gc.set_threshold(*old)
+        gc.collect()
+
+
 def test_long_context_decode_splits_keys_and_matches_plain(eng, tmp_path):
     """Past 2,048 keys a small decode batch spreads each request's keys over several blocks (and, with graphs,
     switches to the long-context graphs): logits still follow the plain implementation."""
