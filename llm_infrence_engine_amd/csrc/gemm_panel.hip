@@ -1,5 +1,5 @@
-// out[M,N] = A[M,K] . W[N,K]^T for 17 to 64 tokens (a decode step of a larger batch) and a W of many rows,
-// bfloat16 in, float accumulation on the matrix cores (v_mfma_f32_16x16x32_bf16).
+// out[M,N] = A[M,K] . W[N,K]^T for up to 64 tokens (a decode step; mostly of a larger batch) and a W of many
+// rows, bfloat16 in, float accumulation on the matrix cores (v_mfma_f32_16x16x32_bf16).
 //
 // With this many tokens the activations, not the weights, are most of what a block has to load when it reads
 // them as MFMA operands k-step by k-step: every 16-row tile of W needs all of A again, and what a CU can pull
@@ -252,6 +252,225 @@ gemm_panel_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restric
   }
 }
 
+// The same for rows of A that do not fit LDS whole: the panel holds KC columns at a time, and a wave keeps the
+// accumulators of all its tiles (up to NACC whole tiles and one shared tile) across the chunks.  Between two
+// chunks the block waits twice: for the panel to be complete, and for everybody to be done with it.
+template <int TT, int NACC, int EPI, typename TO, bool NORM>
+__global__ void __launch_bounds__(WAVES * MS_WAVE)
+gemm_panel_chunked_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restrict__ W, size_t ldw,
+                          const float* __restrict__ bias, TO* __restrict__ out, size_t ldo, int M, int N, int K,
+                          const float* __restrict__ norm_w, float eps, const int* __restrict__ rows, int q, int rem,
+                          int KC) {
+  // weight fragments a wave asks for before it multiplies them: what the 128 registers of a lane (16 waves on
+  // the CU) leave beside the accumulators, each fragment with its TT operands from the panel
+  constexpr int FREE = 104 - (NACC + 1) * TT * 4;
+  constexpr int PB = (NACC + 1) * TT * 4 >= 48 ? 2 : BATCH;   // panel loads in flight, by the same budget
+  constexpr int DEPTH = FREE / (4 * (1 + TT)) > 4 ? 4 : (FREE / (4 * (1 + TT)) < 1 ? 1 : FREE / (4 * (1 + TT)));
+  extern __shared__ u32x4 smem[];   // the panel [tokens][pitch] of one chunk; afterwards the waves' partial sums
+  __shared__ float ss_part[MAX_TOKENS * MAX_PARTS];
+  __shared__ float inv_rms[MAX_TOKENS];
+  const bf16* A = (const bf16*)Av;
+  const float* X = (const float*)Av;
+  const int lane = threadIdx.x & (MS_WAVE - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MS_WAVE);   // the same for the whole wave
+  const int col = lane & 15, kq = lane >> 4;
+  const int C8 = KC / 8;                    // pieces per row of a full chunk (KC is a multiple of 32)
+  const int pitch = C8 + 1;                 // odd, so that 16 rows read at one column hit 16 different banks
+  const int parts = (C8 + 63) / 64;         // loads of 64 lanes x 8 columns per row and chunk
+  u32x4* xst = smem;
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+
+  // this block's tiles of W, as in the kernel above
+  const int b = blockIdx.x;
+  const int T = q + (b < rem ? 1 : 0);
+  const int t0 = b * q + min(b, rem);
+  const int T_whole = T & ~(WAVES - 1), T_left = T - T_whole;
+  const int n_whole = T_whole / WAVES;      // whole tiles of every wave: wave, wave + 16, ...; at most NACC
+  const int g = T_left ? WAVES / T_left : 1;
+  int left_tile = 0, j = 0;
+  if (T_left) {
+    left_tile = small_div(wave, small_inverse(g));
+    j = wave - left_tile * g;
+  }
+  const bool shares = T_left && left_tile < T_left;
+
+  // the panel's loads of this wave: one 512-column part of the chunk, every (16 / parts2)-th token
+  const int parts2 = parts <= 1 ? 1 : (parts <= 2 ? 2 : 4);
+  const int part = wave & (parts2 - 1);
+  const int tok_step = WAVES / parts2;
+  const int c = part * 64 + lane;
+
+  int xrow[TT];   // idle columns repeat the last token; their results are not stored
+#pragma unroll
+  for (int tt = 0; tt < TT; ++tt) xrow[tt] = min(tt * 16 + col, M - 1) * pitch + kq;
+
+  f32x4 acc[NACC][TT], acc_left[TT];
+#pragma unroll
+  for (int tt = 0; tt < TT; ++tt) {
+    acc_left[tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < NACC; ++i) acc[i][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  for (int k0 = 0; k0 < K; k0 += KC) {
+    const int Kc8 = min(KC, K - k0) / 8;      // pieces per row of this chunk
+    const int S = (Kc8 + 3) / 4;              // its k-steps
+    // ---- the panel of columns k0 .. k0 + 8 * Kc8
+    {
+      const bool in = c < Kc8;
+      const int cc = k0 + min(c, Kc8 - 1) * 8;
+      f32x4 nwf[2];
+      if (NORM) {
+        nwf[0] = *reinterpret_cast<const f32x4*>(norm_w + cc);
+        nwf[1] = *reinterpret_cast<const f32x4*>(norm_w + cc + 4);
+      }
+      if (part < parts) {
+        for (int base = wave / parts2; base < M; base += tok_step * PB) {
+          u32x4 piece[NORM ? 1 : PB];
+          f32x4 xf[NORM ? PB : 1][2];
+#pragma unroll
+          for (int i = 0; i < PB; ++i) {
+            const int tok = base + i * tok_step;
+            if (tok >= M) break;   // the same for the whole wave
+            const size_t at = (size_t)(rows ? rows[tok] : tok) * lda + cc;
+            if (NORM) {
+              xf[i][0] = *reinterpret_cast<const f32x4*>(X + at);
+              xf[i][1] = *reinterpret_cast<const f32x4*>(X + at + 4);
+            } else {
+              piece[i] = *reinterpret_cast<const u32x4*>(A + at);
+            }
+          }
+#pragma unroll
+          for (int i = 0; i < PB; ++i) {
+            const int tok = base + i * tok_step;
+            if (tok >= M) break;
+            u32x4 pc;
+            if (NORM) {
+              bf16x8 h;
+              float ss = 0.f;
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                const float x0 = in ? xf[i][0][e] : 0.f, x1 = in ? xf[i][1][e] : 0.f;
+                ss = fmaf(x0, x0, ss);
+                ss = fmaf(x1, x1, ss);
+                h[e] = (__bf16)(x0 * nwf[0][e]);
+                h[4 + e] = (__bf16)(x1 * nwf[1][e]);
+              }
+              pc = __builtin_bit_cast(u32x4, h);
+              ss = wave_sum(ss);   // the lanes of a load in a fixed tree; a (token, part) is this wave's in every chunk
+              if (lane == 0) ss_part[tok * parts + part] = (k0 ? ss_part[tok * parts + part] : 0.f) + ss;
+            } else {
+              pc = piece[i];
+            }
+            if (in) xst[tok * pitch + c] = pc;
+          }
+        }
+      }
+      // a last k-step that the chunk fills only in part reads zeros for the rest
+      const int padn = S * 4 - Kc8;   // 0..3
+      for (int t = threadIdx.x; t < M * padn; t += WAVES * MS_WAVE) {
+        const int rr = t / padn;
+        xst[rr * pitch + Kc8 + t - rr * padn] = zero;
+      }
+    }
+    __syncthreads();
+
+    // ---- this chunk's k-steps of the wave's tiles
+    auto run = [&](int tile, int s_first, int step, f32x4* a) {
+      const bf16* wrow = W + (size_t)min((t0 + tile) * 16 + col, N - 1) * ldw + k0;   // rows past N repeat the last
+      for (int s0 = s_first; s0 < S; s0 += step * DEPTH) {
+        bf16x8 wa[DEPTH];
+#pragma unroll
+        for (int p = 0; p < DEPTH; ++p) {
+          const int s = s0 + p * step;
+          if (s >= S) break;   // the same for the whole wave
+          const int k = s * 32 + kq * 8;
+          wa[p] = *reinterpret_cast<const bf16x8*>(wrow + min(k, K - k0 - 8));   // a piece is in or out
+          if (k0 + k >= K) wa[p] = __builtin_bit_cast(bf16x8, zero);
+        }
+#pragma unroll
+        for (int p = 0; p < DEPTH; ++p) {
+          const int s = s0 + p * step;
+          if (s >= S) break;
+#pragma unroll
+          for (int tt = 0; tt < TT; ++tt) {
+            const bf16x8 xb = __builtin_bit_cast(bf16x8, xst[xrow[tt] + 4 * s]);
+            a[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[p], xb, a[tt], 0, 0, 0);
+          }
+        }
+      }
+    };
+#pragma unroll
+    for (int i = 0; i < NACC; ++i) {
+      if (i >= n_whole) break;
+      run(wave + i * WAVES, 0, 1, acc[i]);
+    }
+    if (shares) run(T_whole + left_tile, j, g, acc_left);
+    __syncthreads();   // the next chunk overwrites the panel
+  }
+
+  if (NORM) {
+    if (threadIdx.x < M) {   // a token's parts in order (each the sum of its chunks in order)
+      float total = 0.f;
+      for (int p = 0; p < parts; ++p) total += ss_part[threadIdx.x * parts + p];
+      inv_rms[threadIdx.x] = 1.0f / sqrtf(total / (float)K + eps);
+    }
+    __syncthreads();
+  }
+
+  // what a lane holds of a finished tile: out[token tt * 16 + col][n0 + kq * 4 + (0..3)]
+  auto finish = [&](int tl, f32x4* sum) {
+    const int nb = (t0 + tl) * 16 + kq * 4;
+    f32x4 bv = {0.f, 0.f, 0.f, 0.f};
+    if (bias && EPI != EPI_SWIGLU) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) if (nb + r < N) bv[r] = bias[nb + r];
+    }
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) {
+      const int m = tt * 16 + col;
+      if (m >= M) continue;
+      f32x4 v = sum[tt];
+      if (NORM) v *= inv_rms[m];
+      if (EPI == EPI_SWIGLU) {
+#pragma unroll
+        for (int p = 0; p < 2; ++p)
+          if (nb + 2 * p + 1 < N) out[(size_t)m * ldo + nb / 2 + p] = from_float<TO>(fast_silu(v[2 * p]) * v[2 * p + 1]);
+      } else {
+        TO* o = out + (size_t)m * ldo + nb;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          if (nb + r >= N) continue;
+          if (EPI == EPI_RESIDUAL) o[r] = from_float<TO>(to_float(o[r]) + v[r] + bv[r]);
+          else o[r] = from_float<TO>(v[r] + bv[r]);
+        }
+      }
+    }
+  };
+#pragma unroll
+  for (int i = 0; i < NACC; ++i) {
+    if (i >= n_whole) break;
+    finish(wave + i * WAVES, acc[i]);
+  }
+  if (!T_left) return;   // the same for the whole block
+
+  // the first wave of a shared tile adds the others' accumulators in wave order (the panel is free: the loop
+  // ended with a wait)
+  f32x4* red = reinterpret_cast<f32x4*>(smem);   // [WAVES][TT][64]
+  if (shares && j > 0) {
+#pragma unroll
+    for (int tt = 0; tt < TT; ++tt) red[(wave * TT + tt) * MS_WAVE + lane] = acc_left[tt];
+  }
+  __syncthreads();
+  if (shares && j == 0) {
+    for (int w = 1; w < g; ++w) {
+#pragma unroll
+      for (int tt = 0; tt < TT; ++tt) acc_left[tt] += red[((wave + w) * TT + tt) * MS_WAVE + lane];
+    }
+    finish(T_whole + left_tile, acc_left);
+  }
+}
+
 constexpr int LDS_BUDGET = 144 * 1024;   // of the CU's 160 KB, for the panel
 
 template <int TT, int EPI, typename TO, bool NORM>
@@ -270,25 +489,60 @@ int launch(const void* A, size_t lda, const bf16* W, size_t ldw, const float* bi
   return ms_launch_status();
 }
 
+template <int TT, int NACC, int EPI, typename TO, bool NORM>
+int launch_chunked(const void* A, size_t lda, const bf16* W, size_t ldw, const float* bias, TO* out, size_t ldo, int M,
+                   int N, int K, const float* norm_w, float eps, const int* rows, int blocks, int q, int rem, int KC,
+                   size_t lds, hipStream_t stream) {
+  static bool raised = false;
+  if (!raised) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_panel_chunked_kernel<TT, NACC, EPI, TO, NORM>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BUDGET) != hipSuccess)
+      return MS_LAUNCH_FAILED;
+    raised = true;
+  }
+  gemm_panel_chunked_kernel<TT, NACC, EPI, TO, NORM><<<dim3(blocks), dim3(WAVES * MS_WAVE), lds, stream>>>(
+      A, lda, W, ldw, bias, out, ldo, M, N, K, norm_w, eps, rows, q, rem, KC);
+  return ms_launch_status();
+}
+
 template <int EPI, typename TO, bool NORM>
 int plan(const void* A, size_t lda, const bf16* W, size_t ldw, const float* bias, TO* out, size_t ldo, int M, int N,
          int K, const float* norm_w, float eps, const int* rows, bool any_shape, hipStream_t stream) {
   const int cus = ms_compute_units();
   const int tiles = (N + 15) / 16;
-  // Where this kernel wins over ms_gemm_skinny, by measurement: more than 16 tokens and at least a tile of W
-  // for every CU (with fewer blocks than CUs the panel, which every block loads whole, costs more than it saves).
-  if (!any_shape && (M <= 16 || tiles < cus)) return MS_UNSUPPORTED;
+  // Where this kernel wins over ms_gemm_skinny, by measurement.  More than 16 tokens: from 7/8 of a tile of W
+  // for every CU on (the 7B shape's down projection, 224 tiles: 81 against 101 us at 64 tokens; with 96 or 128
+  // tiles the panel, which every block loads whole, costs more than it saves).  Up to 16 tokens: a W of at least
+  // four tiles per CU with long rows (gate/up and head of the 7B shape at 8 tokens: 54 against 66 us, 212 against
+  // 248; at the 0.5B shape the two kernels are equal or this one slower).
+  if (!any_shape && (M > 16 ? tiles * 8 < cus * 7 : (tiles < 4 * cus || K < 2048))) return MS_UNSUPPORTED;
   const int tt = (M + 15) / 16;
   const int S = (K + 31) / 32;
-  if ((K / 8 + 63) / 64 > MAX_PARTS) return MS_UNSUPPORTED;
-  size_t lds = (size_t)M * (S * 4 + 1) * 16;
-  if (lds > (size_t)LDS_BUDGET) return MS_UNSUPPORTED;   // the panel has to fit whole
-  const size_t red = (size_t)WAVES * tt * MS_WAVE * 16;
-  if (lds < red) lds = red;
   const int blocks = tiles < cus ? tiles : cus;
   const int q = tiles / blocks, rem = tiles % blocks;
+  const size_t red = (size_t)WAVES * tt * MS_WAVE * 16;
+  size_t lds = (size_t)M * (S * 4 + 1) * 16;
+  if (lds <= (size_t)LDS_BUDGET && (K / 8 + 63) / 64 <= MAX_PARTS) {   // the rows fit whole
+    if (lds < red) lds = red;
 #define GO(TTV) if (tt == TTV) return launch<TTV, EPI, TO, NORM>(A, lda, W, ldw, bias, out, ldo, M, N, K, norm_w, eps, rows, blocks, q, rem, lds, stream)
-  GO(1); GO(2); GO(3); GO(4);
+    GO(1); GO(2); GO(3); GO(4);
+#undef GO
+    return MS_UNSUPPORTED;
+  }
+  // in chunks of KC columns: the widest of 2048, 1536, 1024, 512 that fits
+  int KC = 0;
+  for (int kc = 2048; kc >= 512; kc -= 512) {
+    if ((size_t)M * (kc / 8 + 1) * 16 <= (size_t)LDS_BUDGET) { KC = kc; break; }
+  }
+  if (!KC) return MS_UNSUPPORTED;
+  lds = (size_t)M * (KC / 8 + 1) * 16;
+  if (lds < red) lds = red;
+  const int nacc = (q + (rem ? 1 : 0)) / WAVES;   // whole tiles a wave keeps accumulators for
+  if (nacc > 3 || (tt == 4 && nacc > 2)) return MS_UNSUPPORTED;   // what a lane's registers hold
+#define GO(TTV, NA) if (tt == TTV && (nacc < 1 ? 1 : nacc) == NA) return launch_chunked<TTV, NA, EPI, TO, NORM>(A, lda, W, ldw, bias, out, ldo, M, N, K, norm_w, eps, rows, blocks, q, rem, KC, lds, stream)
+  GO(1, 1); GO(2, 1); GO(3, 1); GO(4, 1);
+  GO(1, 2); GO(2, 2); GO(3, 2); GO(4, 2);
+  GO(1, 3); GO(2, 3); GO(3, 3);
 #undef GO
   return MS_UNSUPPORTED;
 }
@@ -303,7 +557,7 @@ int plan(const void* A, size_t lda, const bf16* W, size_t ldw, const float* bias
 // epilogue 3: out[M,N] float += product + bias (not with norm)
 // MS_UNSUPPORTED for shapes it does not take (the caller then uses ms_gemm_skinny): with any_shape = 0 all but
 // those it is the faster kernel for; with any_shape = 1 (tests, measurements) only those it cannot compute
-// (rows that do not fit LDS whole: M * (K + 40) * 2 bytes over 144 KB, or K over 2048).
+// (more than 63 tiles of W to a block, 47 with more than 48 rows, when the rows have to go through LDS in chunks).
 extern "C" int ms_gemm_panel(const void* A, long long lda, const int* rows, const float* norm_w, float eps,
                              const void* W, long long ldw, const float* bias, void* out, long long ldo, int M, int N,
                              int K, int epilogue, int out_dtype, int norm, int any_shape, hipStream_t stream) {

@@ -258,7 +258,7 @@ extern "C" int ms_gemm_skinny(const void* A, long long lda, const void* W, long 
     const int rc = ms_gemm_stream(A, lda, nullptr, nullptr, 0.f, W, ldw, bias, out, ldo, M, N, K, epilogue, out_dtype, 0, 0, stream);
     if (rc != MS_UNSUPPORTED) return rc;
   }
-  if (M > 16 && !forced()) {    // several: the kernel that holds the activations in LDS, where it takes the shape
+  if (!forced()) {    // the kernel that holds the activations in LDS, where it takes the shape
     const int rc = ms_gemm_panel(A, lda, nullptr, nullptr, 0.f, W, ldw, bias, out, ldo, M, N, K, epilogue, out_dtype, 0, 0, stream);
     if (rc != MS_UNSUPPORTED) return rc;
   }
@@ -294,7 +294,7 @@ extern "C" int ms_gemm_skinny_norm(const float* x, long long ldx, const int* row
     const int rc = ms_gemm_stream(x, ldx, rows, norm_w, eps, W, ldw, bias, out, ldo, M, N, K, epilogue, out_dtype, 1, 0, stream);
     if (rc != MS_UNSUPPORTED) return rc;
   }
-  if (M > 16 && !forced()) {
+  if (!forced()) {
     const int rc = ms_gemm_panel(x, ldx, rows, norm_w, eps, W, ldw, bias, out, ldo, M, N, K, epilogue, out_dtype, 1, 0, stream);
     if (rc != MS_UNSUPPORTED) return rc;
   }

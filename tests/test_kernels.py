@@ -488,9 +488,13 @@ def test_gemm_panel(ops, M, N, K):
     torch.testing.assert_close(gated.double(), torch.nn.functional.silu(hw[:, 0::2]) * hw[:, 1::2], **tol(torch.bfloat16))
 
 
-@pytest.mark.parametrize("M,N,K", [(20, 300, 1200), (33, 4100, 1528), (18, 500, 2040)])
+@pytest.mark.parametrize("M,N,K", [(20, 300, 1200), (33, 4100, 1528), (18, 500, 2040),
+                                   (64, 4300, 3584), (40, 700, 5120), (64, 4096 + 16 * 256 * 2, 2600), (17, 90, 4872),
+                                   (50, 16 * 256 * 33 + 40, 2400), (40, 16 * 256 * 50, 1840)])
 def test_gemm_panel_long_rows(ops, M, N, K):
-    """Rows of three and four 512-column parts (with three a quarter of the waves sit the loading out)."""
+    """Rows of three and four 512-column parts (with three a quarter of the waves sit the loading out), and rows
+    that do not fit LDS whole and go through it in chunks: a last chunk that is shorter, blocks with whole and
+    shared tiles, two and three whole tiles to a wave."""
     g = torch.Generator().manual_seed(K)
     xs = torch.randn(M, K, generator=g).to(DEV)
     w = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16().to(DEV)
@@ -507,12 +511,9 @@ def test_gemm_panel_refuses_what_it_cannot_take(ops):
     w = torch.zeros(64, 64, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(RuntimeError, match="unsupported"):
         ops.gemm_panel(torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV), w)             # more than 64 rows
-    with pytest.raises(RuntimeError, match="unsupported"):                                   # rows that do not fit LDS
-        ops.gemm_panel(torch.zeros(64, 1600, dtype=torch.bfloat16, device=DEV),
-                       torch.zeros(64, 1600, dtype=torch.bfloat16, device=DEV))
-    with pytest.raises(RuntimeError, match="unsupported"):
-        ops.gemm_panel(torch.zeros(20, 4096, dtype=torch.bfloat16, device=DEV),
-                       torch.zeros(64, 4096, dtype=torch.bfloat16, device=DEV))              # K beyond its loads
+    with pytest.raises(RuntimeError, match="unsupported"):           # in chunks, and too many tiles to a block
+        ops.gemm_panel(torch.zeros(64, 2400, dtype=torch.bfloat16, device=DEV),
+                       torch.zeros(16 * 256 * 48, 2400, dtype=torch.bfloat16, device=DEV))
     with pytest.raises(RuntimeError, match="unsupported"):                                   # not the shape it is for
         ops.gemm_panel(torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV), w, any_shape=False)
 
