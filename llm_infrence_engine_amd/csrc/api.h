@@ -44,6 +44,11 @@ int ms_gemm_panel(const void* A, long long lda, const int* rows, const float* no
                    long long ldw, const float* bias, void* out, long long ldo, int M, int N, int K, int epilogue,
                    int out_dtype, int norm, int any_shape, hipStream_t stream);
 
+int ms_gemm_panel_splitk_parts(int M, int N, int K);
+int ms_gemm_panel_splitk(const void* A, long long lda, const void* W, long long ldw, const float* bias, void* out,
+                         long long ldo, int M, int N, int K, int epilogue, int out_dtype, void* partial, int parts,
+                         hipStream_t stream);
+
 int ms_gemm_skinny_norm(const float* x, long long ldx, const int* rows, const float* norm_w, float eps, const void* W,
                         long long ldw, const float* bias, void* out, long long ldo, int M, int N, int K, int epilogue,
                         int out_dtype, hipStream_t stream);

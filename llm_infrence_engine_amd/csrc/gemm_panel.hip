@@ -260,12 +260,12 @@ __global__ void __launch_bounds__(WAVES * MS_WAVE)
 gemm_panel_chunked_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restrict__ W, size_t ldw,
                           const float* __restrict__ bias, TO* __restrict__ out, size_t ldo, int M, int N, int K,
                           const float* __restrict__ norm_w, float eps, const int* __restrict__ rows, int q, int rem,
-                          int KC) {
+                          int KC, int row_blocks, int k_per) {
   // weight fragments a wave asks for before it multiplies them: what the 128 registers of a lane (16 waves on
   // the CU) leave beside the accumulators, each fragment with its TT operands from the panel
-  constexpr int FREE = 104 - (NACC + 1) * TT * 4;
+  constexpr int FREE = (NACC >= 3 ? 88 : 96) - (NACC + 1) * TT * 4;
   constexpr int PB = (NACC + 1) * TT * 4 >= 48 ? 2 : BATCH;   // panel loads in flight, by the same budget
-  constexpr int DEPTH = FREE / (4 * (1 + TT)) > 4 ? 4 : (FREE / (4 * (1 + TT)) < 1 ? 1 : FREE / (4 * (1 + TT)));
+  constexpr int DEPTH = FREE / (4 * (1 + TT)) > 8 ? 8 : (FREE / (4 * (1 + TT)) < 1 ? 1 : FREE / (4 * (1 + TT)));
   extern __shared__ u32x4 smem[];   // the panel [tokens][pitch] of one chunk; afterwards the waves' partial sums
   __shared__ float ss_part[MAX_TOKENS * MAX_PARTS];
   __shared__ float inv_rms[MAX_TOKENS];
@@ -280,8 +280,13 @@ gemm_panel_chunked_kernel(const void* __restrict__ Av, size_t lda, const bf16* _
   u32x4* xst = smem;
   const u32x4 zero = {0u, 0u, 0u, 0u};
 
-  // this block's tiles of W, as in the kernel above
-  const int b = blockIdx.x;
+  // this block's tiles of W, as in the kernel above.  When the columns are split as well (k_per < K: block ids
+  // beyond row_blocks take the next k_per columns of the same tiles), a block's result is a partial sum that
+  // goes to its own [M, ldo] slice of `out`, to be added up by splitk_reduce_kernel.
+  const int k_part = blockIdx.x / row_blocks;
+  const int b = blockIdx.x - k_part * row_blocks;
+  const int k_begin = k_part * k_per, k_end = min(K, k_begin + k_per);
+  out += (size_t)k_part * M * ldo;
   const int T = q + (b < rem ? 1 : 0);
   const int t0 = b * q + min(b, rem);
   const int T_whole = T & ~(WAVES - 1), T_left = T - T_whole;
@@ -312,8 +317,8 @@ gemm_panel_chunked_kernel(const void* __restrict__ Av, size_t lda, const bf16* _
     for (int i = 0; i < NACC; ++i) acc[i][tt] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  for (int k0 = 0; k0 < K; k0 += KC) {
-    const int Kc8 = min(KC, K - k0) / 8;      // pieces per row of this chunk
+  for (int k0 = k_begin; k0 < k_end; k0 += KC) {
+    const int Kc8 = min(KC, k_end - k0) / 8;  // pieces per row of this chunk
     const int S = (Kc8 + 3) / 4;              // its k-steps
     // ---- the panel of columns k0 .. k0 + 8 * Kc8
     {
@@ -358,7 +363,7 @@ gemm_panel_chunked_kernel(const void* __restrict__ Av, size_t lda, const bf16* _
               }
               pc = __builtin_bit_cast(u32x4, h);
               ss = wave_sum(ss);   // the lanes of a load in a fixed tree; a (token, part) is this wave's in every chunk
-              if (lane == 0) ss_part[tok * parts + part] = (k0 ? ss_part[tok * parts + part] : 0.f) + ss;
+              if (lane == 0) ss_part[tok * parts + part] = (k0 != k_begin ? ss_part[tok * parts + part] : 0.f) + ss;
             } else {
               pc = piece[i];
             }
@@ -385,8 +390,8 @@ gemm_panel_chunked_kernel(const void* __restrict__ Av, size_t lda, const bf16* _
           const int s = s0 + p * step;
           if (s >= S) break;   // the same for the whole wave
           const int k = s * 32 + kq * 8;
-          wa[p] = *reinterpret_cast<const bf16x8*>(wrow + min(k, K - k0 - 8));   // a piece is in or out
-          if (k0 + k >= K) wa[p] = __builtin_bit_cast(bf16x8, zero);
+          wa[p] = *reinterpret_cast<const bf16x8*>(wrow + min(k, k_end - k0 - 8));   // a piece is in or out
+          if (k0 + k >= k_end) wa[p] = __builtin_bit_cast(bf16x8, zero);
         }
 #pragma unroll
         for (int p = 0; p < DEPTH; ++p) {
@@ -471,6 +476,36 @@ gemm_panel_chunked_kernel(const void* __restrict__ Av, size_t lda, const bf16* _
   }
 }
 
+// out[m, n] (=, +=) sum over the column parts of partial[part][m][n], in part order, + bias.
+template <int EPI, typename TO>
+__global__ void __launch_bounds__(256)
+splitk_reduce_kernel(const float* __restrict__ partial, int parts, const float* __restrict__ bias, TO* __restrict__ out,
+                     size_t ldo, int M, int N) {
+  const int quads = (N + 3) / 4;
+  const int id = blockIdx.x * blockDim.x + threadIdx.x;
+  if (id >= M * quads) return;
+  const int m = id / quads, n = (id - m * quads) * 4;
+  float sum[4] = {0.f, 0.f, 0.f, 0.f};
+  const size_t slice = (size_t)M * N;
+  const bool whole = n + 3 < N && N % 4 == 0;   // rows of the partial sums are 16-byte aligned then
+  for (int p = 0; p < parts; ++p) {
+    const float* src = partial + p * slice + (size_t)m * N + n;
+    if (whole) {
+      const f32x4 v = *reinterpret_cast<const f32x4*>(src);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) sum[r] += v[r];
+    } else {
+      for (int r = 0; r < 4 && n + r < N; ++r) sum[r] += src[r];
+    }
+  }
+  TO* o = out + (size_t)m * ldo + n;
+  for (int r = 0; r < 4 && n + r < N; ++r) {
+    const float v = sum[r] + (bias ? bias[n + r] : 0.f);
+    if (EPI == EPI_RESIDUAL) o[r] = from_float<TO>(to_float(o[r]) + v);
+    else o[r] = from_float<TO>(v);
+  }
+}
+
 constexpr int LDS_BUDGET = 144 * 1024;   // of the CU's 160 KB, for the panel
 
 template <int TT, int EPI, typename TO, bool NORM>
@@ -492,7 +527,7 @@ int launch(const void* A, size_t lda, const bf16* W, size_t ldw, const float* bi
 template <int TT, int NACC, int EPI, typename TO, bool NORM>
 int launch_chunked(const void* A, size_t lda, const bf16* W, size_t ldw, const float* bias, TO* out, size_t ldo, int M,
                    int N, int K, const float* norm_w, float eps, const int* rows, int blocks, int q, int rem, int KC,
-                   size_t lds, hipStream_t stream) {
+                   size_t lds, hipStream_t stream, int k_parts = 1, int k_per = 0) {
   static bool raised = false;
   if (!raised) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_panel_chunked_kernel<TT, NACC, EPI, TO, NORM>),
@@ -500,8 +535,8 @@ int launch_chunked(const void* A, size_t lda, const bf16* W, size_t ldw, const f
       return MS_LAUNCH_FAILED;
     raised = true;
   }
-  gemm_panel_chunked_kernel<TT, NACC, EPI, TO, NORM><<<dim3(blocks), dim3(WAVES * MS_WAVE), lds, stream>>>(
-      A, lda, W, ldw, bias, out, ldo, M, N, K, norm_w, eps, rows, q, rem, KC);
+  gemm_panel_chunked_kernel<TT, NACC, EPI, TO, NORM><<<dim3(blocks * k_parts), dim3(WAVES * MS_WAVE), lds, stream>>>(
+      A, lda, W, ldw, bias, out, ldo, M, N, K, norm_w, eps, rows, q, rem, KC, blocks, k_parts > 1 ? k_per : K);
   return ms_launch_status();
 }
 
@@ -547,6 +582,54 @@ int plan(const void* A, size_t lda, const bf16* W, size_t ldw, const float* bias
   return MS_UNSUPPORTED;
 }
 
+// Columns split over blocks as well, for a W with long rows and too few tiles to give every CU a share of
+// whole rows that is worth its loads of the activations (down projections): the number of column parts, 0 if
+// the shape is not one for it.  Every block then takes at most 16 tiles (one round of its waves).
+int splitk_parts(int M, int N, int K) {
+  const int cus = ms_compute_units();
+  const int tiles = (N + 15) / 16;
+  if (M <= 0 || M > MAX_TOKENS || K < 8192 || K % 8 || tiles > 2 * cus) return 0;
+  // up to 16 tokens a W with a tile for (nearly) every CU and no more is served as well unsplit (7B shape's down
+  // projection, 224 tiles, at 8 tokens: 34 us unsplit, 39 split; 320 tiles of the 14B and 32B shapes: 47 -> 39
+  // and 93 -> 64 us split, for the second round of blocks that unsplit they need)
+  if (M <= 16 && tiles <= cus) return 0;
+  int best = 0;
+  for (int parts = 2; parts <= 16; parts *= 2) {
+    const int row_blocks = cus / parts;
+    if (row_blocks < 1 || (tiles + row_blocks - 1) / row_blocks > WAVES) continue;
+    if (K / parts < 1024) break;
+    best = parts;
+  }
+  return best;
+}
+
+template <int EPI, typename TO>
+int run_splitk(const bf16* A, size_t lda, const bf16* W, size_t ldw, const float* bias, TO* out, size_t ldo, int M, int N,
+               int K, float* partial, int parts, hipStream_t stream) {
+  const int cus = ms_compute_units();
+  const int tiles = (N + 15) / 16;
+  const int row_blocks = tiles < cus / parts ? tiles : cus / parts;
+  const int q = tiles / row_blocks, rem = tiles % row_blocks;
+  const int k_per = ((K + parts - 1) / parts + 31) / 32 * 32;
+  const int tt = (M + 15) / 16;
+  int KC = 0;
+  for (int kc = 2048; kc >= 512; kc -= 512) {
+    if ((size_t)M * (kc / 8 + 1) * 16 <= (size_t)LDS_BUDGET) { KC = kc; break; }
+  }
+  if (!KC) return MS_UNSUPPORTED;
+  size_t lds = (size_t)M * (KC / 8 + 1) * 16;
+  const size_t red = (size_t)WAVES * tt * MS_WAVE * 16;
+  if (lds < red) lds = red;
+  int rc = MS_UNSUPPORTED;
+#define GO(TTV) if (tt == TTV) rc = launch_chunked<TTV, 1, EPI_STORE, float, false>(A, lda, W, ldw, nullptr, partial, (size_t)N, M, N, K, nullptr, 0.f, nullptr, row_blocks, q, rem, KC, lds, stream, parts, k_per)
+  GO(1); GO(2); GO(3); GO(4);
+#undef GO
+  if (rc != MS_OK) return rc;
+  const int threads = M * ((N + 3) / 4);
+  splitk_reduce_kernel<EPI, TO><<<dim3((threads + 255) / 256), dim3(256), 0, stream>>>(partial, parts, bias, out, ldo, M, N);
+  return ms_launch_status();
+}
+
 }  // namespace
 
 // The product of up to 64 rows with W[N,K]^T, the rows held whole in LDS.  norm = 0: A is bfloat16 [M, lda];
@@ -583,5 +666,30 @@ extern "C" int ms_gemm_panel(const void* A, long long lda, const int* rows, cons
     RUN(EPI_RESIDUAL, float, false);
   }
 #undef RUN
+  return MS_BAD_ARG;
+}
+
+// Column parts that ms_gemm_panel_splitk uses for this shape (the caller sizes `partial` by it); 0: not a
+// shape for it.
+extern "C" int ms_gemm_panel_splitk_parts(int M, int N, int K) { return splitk_parts(M, N, K); }
+
+// The product with the columns of W split over blocks too: partial sums float [parts, M, N] in `partial`, then
+// added up in part order into out with epilogue 0 (out_dtype float or bfloat16, + bias) or 3 (out float += ).
+// A bfloat16 [M, lda], no folded norm.
+extern "C" int ms_gemm_panel_splitk(const void* A, long long lda, const void* W, long long ldw, const float* bias,
+                                    void* out, long long ldo, int M, int N, int K, int epilogue, int out_dtype,
+                                    void* partial, int parts, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return MS_OK;
+  if (parts <= 1 || parts != splitk_parts(M, N, K) || !partial) return MS_BAD_ARG;
+  if (ldw % 8 || lda < K || ldw < K || lda % 8 || ldo < N) return MS_UNSUPPORTED;
+  if (((uintptr_t)A | (uintptr_t)W | (uintptr_t)partial) % 16) return MS_UNSUPPORTED;
+  const bf16* a = (const bf16*)A;
+  const bf16* w = (const bf16*)W;
+  if (epilogue == EPI_STORE && out_dtype == MS_BF16)
+    return run_splitk<EPI_STORE, bf16>(a, lda, w, ldw, bias, (bf16*)out, ldo, M, N, K, (float*)partial, parts, stream);
+  if (epilogue == EPI_STORE && out_dtype == MS_F32)
+    return run_splitk<EPI_STORE, float>(a, lda, w, ldw, bias, (float*)out, ldo, M, N, K, (float*)partial, parts, stream);
+  if (epilogue == EPI_RESIDUAL && out_dtype == MS_F32)
+    return run_splitk<EPI_RESIDUAL, float>(a, lda, w, ldw, bias, (float*)out, ldo, M, N, K, (float*)partial, parts, stream);
   return MS_BAD_ARG;
 }

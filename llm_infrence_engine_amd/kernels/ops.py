@@ -34,6 +34,9 @@ _SIGNATURES = {
                        _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "ms_gemm_panel": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int,
                       _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "ms_gemm_panel_splitk_parts": [_c_int, _c_int, _c_int],
+    "ms_gemm_panel_splitk": [_c_ptr, _c_ll, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int,
+                             _c_ptr, _c_int, _c_ptr],
     "ms_residual_add": [_c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr],
     "ms_silu_mul": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "ms_rope_store": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int,
@@ -264,7 +267,8 @@ def skinny_ok(a: torch.Tensor, w: torch.Tensor) -> bool:
 
 
 def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, epilogue: int = EPI_STORE,
-                out_dtype: torch.dtype = torch.bfloat16, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+                out_dtype: torch.dtype = torch.bfloat16, residual: Optional[torch.Tensor] = None,
+                split_columns: bool = True) -> torch.Tensor:
     """a [M <= 64, K] @ w [N, K].T on the matrix cores, bfloat16 in.  Epilogues: EPI_STORE -> [M, N] (+ bias);
     EPI_SWIGLU -> [M, N / 2] = silu(even rows' products) * odd rows' products; EPI_RESIDUAL -> ``residual``
     (float [M, N]) += product + bias, in place."""
@@ -291,7 +295,17 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] =
         out, ldo, out_dtype = residual, N, torch.float32
     else:
         raise ValueError(f"unknown epilogue {epilogue}")
-    _call("ms_gemm_skinny", a.data_ptr(), a.stride(0) if M > 1 else K, w.data_ptr(), K, _ptr(bias), out.data_ptr(), ldo,
+    lda = a.stride(0) if M > 1 else K
+    if epilogue != EPI_SWIGLU and split_columns:
+        # long rows against few of them (a down projection): the columns are split over blocks too, and the
+        # partial sums are added up in a fixed order by a second kernel
+        parts = _get("ms_gemm_panel_splitk_parts")(M, N, K)
+        if parts > 1:
+            partial = torch.empty((parts, M, N), dtype=torch.float32, device=a.device)
+            _call("ms_gemm_panel_splitk", a.data_ptr(), lda, w.data_ptr(), K, _ptr(bias), out.data_ptr(), ldo, M, N, K,
+                  epilogue, _code(out_dtype), partial.data_ptr(), parts, _stream())
+            return out
+    _call("ms_gemm_skinny", a.data_ptr(), lda, w.data_ptr(), K, _ptr(bias), out.data_ptr(), ldo,
           M, N, K, epilogue, _code(out_dtype), _stream())
     return out
 

@@ -507,6 +507,42 @@ def test_gemm_panel_long_rows(ops, M, N, K):
     torch.testing.assert_close(plain.double(), a.double() @ w.double().T, atol=3e-5, rtol=3e-5)
 
 
+@pytest.mark.parametrize("M,N,K", [(8, 5120, 13824), (64, 3584, 18944), (33, 5120, 27648), (17, 900, 8200), (64, 16, 9000),
+                                   (5, 8192, 16384)])
+def test_gemm_with_the_columns_split_over_blocks(ops, M, N, K):
+    """Long rows against few of them: blocks take parts of the columns, a second kernel adds the partial sums in
+    order.  Every epilogue that has no gate; a row's numbers do not depend on the rest of the batch; parts of
+    uneven length, a vocabulary-free odd N, one tile only."""
+    from llm_infrence_engine_amd.kernels import build
+    assert build.load().ms_gemm_panel_splitk_parts(M, N, K) > 1
+    g = torch.Generator().manual_seed(M + N + K)
+    a = torch.randn(M, K, generator=g).bfloat16().to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16().to(DEV)
+    bias = torch.randn(N, generator=g).to(DEV)
+    want = a.double() @ w.double().T
+    out = ops.gemm_skinny(a, w, bias)
+    torch.testing.assert_close(out.double(), want + bias.double(), **tol(torch.bfloat16))
+    f = ops.gemm_skinny(a, w, None, out_dtype=torch.float32)
+    torch.testing.assert_close(f.double(), want, atol=5e-5, rtol=5e-5)
+    x = torch.randn(M, N, generator=g).to(DEV)
+    x0 = x.clone()
+    ops.gemm_skinny(a, w, bias, ops.EPI_RESIDUAL, residual=x)
+    torch.testing.assert_close(x.double(), x0.double() + want + bias.double(), atol=5e-5, rtol=5e-5)
+    assert torch.equal(ops.gemm_skinny(a[M - 1:], w, bias), out[M - 1:]) or M > 16   # the same kernel for one row
+    unsplit = ops.gemm_skinny(a, w, None, out_dtype=torch.float32, split_columns=False)
+    torch.testing.assert_close(unsplit.double(), want, atol=5e-5, rtol=5e-5)
+
+
+def test_columns_are_split_only_where_it_pays(ops):
+    from llm_infrence_engine_amd.kernels import build
+    parts = build.load().ms_gemm_panel_splitk_parts
+    assert parts(8, 896, 4864) == 0          # rows too short
+    assert parts(8, 3584, 18944) == 0        # few tokens and a tile for nearly every CU: as well unsplit
+    assert parts(8, 37888, 3584) == 0        # and here, with tiles enough for every CU besides
+    assert parts(65, 3584, 18944) == 0       # too many tokens
+    assert parts(8, 16384, 18944) == 0       # more than two tiles per CU
+
+
 def test_gemm_panel_refuses_what_it_cannot_take(ops):
     w = torch.zeros(64, 64, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(RuntimeError, match="unsupported"):
