@@ -331,6 +331,32 @@ def test_large_uneven_decode_batch_matches_plain(eng, tmp_path):
             assert np.abs(row - exact[r][k]).max() < 3.0 * noise[r], (r, len(seqs[r]), k)
 
 
+def test_decode_batch_at_the_widths_of_the_seven_billion_model(eng, tmp_path):
+    """22 requests decode together at the layer widths of Qwen2.5-7B (two layers, a vocabulary of 4,100): rows too
+    long to lie in LDS whole go through it in chunks, the down projection splits its columns over blocks, head
+    size 128 with seven query heads to a key/value head."""
+    from llm_infrence_engine_amd.config import config_from_dict
+    from llm_infrence_engine_amd.engine import StepEntry, load_runner
+
+    cfg = {"architectures": ["Qwen2ForCausalLM"], "num_hidden_layers": 2, "hidden_size": 3584, "num_attention_heads": 28,
+           "num_key_value_heads": 4, "intermediate_size": 18944, "vocab_size": 4100, "rope_theta": 1000000.0,
+           "rms_norm_eps": 1e-6, "tie_word_embeddings": False}
+    d = tmp_path / "m"
+    eng.write_random_model(d, config_from_dict(cfg), seed=7, dtype="bfloat16", std=0.02)
+    pc, w = P.read_config(d), P.read_weights(d, torch.float64)
+    rng = np.random.default_rng(7)
+    R, tail = 22, 2
+    seqs = {f"r{i}": [int(t) for t in rng.integers(0, 4100, n)] for i, n in enumerate(rng.integers(20, 121, R))}
+    exact = {r: P.forward(w, pc, t)[-tail:].numpy() for r, t in seqs.items()}
+    noise = {r: np.abs(P.forward(w, pc, t, act_dtype=torch.bfloat16)[-tail:].numpy() - exact[r]).max() for r, t in seqs.items()}
+    runner = load_runner(d, dtype="bfloat16", page_size=16, max_requests=R, max_len=128)
+    runner.step([StepEntry(r, t[:-tail], []) for r, t in seqs.items()])
+    for k in range(tail):
+        lg = runner.step([StepEntry(r, [t[len(t) - tail + k]], [0]) for r, t in seqs.items()]).float().cpu().numpy()
+        for row, r in zip(lg, seqs):
+            assert np.abs(row - exact[r][k]).max() < 3.0 * noise[r], (r, len(seqs[r]), k)
+
+
 def test_several_decode_steps_per_launch_change_nothing(tiny, eng):
     """Up to 8 decode steps queued in one graph launch (tokens fed back on the device): the same outputs as step
     by step, also when a stop id arrives in the middle of a launch, a request joins, or pages are scarce."""
