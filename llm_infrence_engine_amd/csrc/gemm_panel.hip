@@ -39,6 +39,122 @@ constexpr int MAX_PARTS = 4;    // 64-piece (512-column) loads per row of A at m
 __device__ __forceinline__ int small_inverse(int parts) { return (65536 + parts - 1) / parts; }
 __device__ __forceinline__ int small_div(int id, int inverse) { return (id * inverse) >> 16; }
 
+// One chunk of the panel: columns k0 .. k0 + 8 * Kc8 of the M rows of A go to LDS as bfloat16 pieces
+// xst[token * pitch + piece], the S * 4 - Kc8 pieces that a last k-step lacks as zeros.  A wave keeps to one
+// 512-column part of the chunk (so it loads that part of the norm weights once) and takes every
+// (16 / parts2)-th token, PB of them in flight.  With NORM the rows are float and are multiplied by the norm
+// weights on the way; their squares are summed per (token, part): the lanes of a load in the fixed tree of
+// wave_sum, a (token, part)'s chunks in order (the same wave has it in every chunk).
+template <bool NORM, int PB>
+__device__ __forceinline__ void load_panel(const void* __restrict__ Av, size_t lda, const float* __restrict__ norm_w,
+                                           const int* __restrict__ rows, int M, int k0, int Kc8, int S, int parts,
+                                           int pitch, bool first_chunk, u32x4* xst, float* ss_part, int wave, int lane) {
+  const bf16* A = (const bf16*)Av;
+  const float* X = (const float*)Av;
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+  const int parts2 = parts <= 1 ? 1 : (parts <= 2 ? 2 : 4);
+  const int part = wave & (parts2 - 1);
+  const int tok_step = WAVES / parts2;
+  const int c = part * 64 + lane;
+  const bool in = c < Kc8;   // lanes past the chunk's end (and whole waves, when parts is 3) load nothing new
+  const int cc = k0 + min(c, Kc8 - 1) * 8;
+  f32x4 nwf[2];
+  if (NORM) {
+    nwf[0] = *reinterpret_cast<const f32x4*>(norm_w + cc);
+    nwf[1] = *reinterpret_cast<const f32x4*>(norm_w + cc + 4);
+  }
+  if (part < parts) {
+    for (int base = wave / parts2; base < M; base += tok_step * PB) {
+      u32x4 piece[NORM ? 1 : PB];
+      f32x4 xf[NORM ? PB : 1][2];
+#pragma unroll
+      for (int i = 0; i < PB; ++i) {
+        const int tok = base + i * tok_step;
+        if (tok >= M) break;   // the same for the whole wave
+        const size_t at = (size_t)(rows ? rows[tok] : tok) * lda + cc;
+        if (NORM) {
+          xf[i][0] = *reinterpret_cast<const f32x4*>(X + at);
+          xf[i][1] = *reinterpret_cast<const f32x4*>(X + at + 4);
+        } else {
+          piece[i] = *reinterpret_cast<const u32x4*>(A + at);
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < PB; ++i) {
+        const int tok = base + i * tok_step;
+        if (tok >= M) break;
+        u32x4 pc;
+        if (NORM) {
+          bf16x8 h;
+          float ss = 0.f;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float x0 = in ? xf[i][0][e] : 0.f, x1 = in ? xf[i][1][e] : 0.f;
+            ss = fmaf(x0, x0, ss);
+            ss = fmaf(x1, x1, ss);
+            h[e] = (__bf16)(x0 * nwf[0][e]);
+            h[4 + e] = (__bf16)(x1 * nwf[1][e]);
+          }
+          pc = __builtin_bit_cast(u32x4, h);
+          ss = wave_sum(ss);
+          if (lane == 0) ss_part[tok * parts + part] = (first_chunk ? 0.f : ss_part[tok * parts + part]) + ss;
+        } else {
+          pc = piece[i];
+        }
+        if (in) xst[tok * pitch + c] = pc;
+      }
+    }
+  }
+  const int padn = S * 4 - Kc8;   // 0..3
+  for (int t = threadIdx.x; t < M * padn; t += WAVES * MS_WAVE) {
+    const int rr = t / padn;
+    xst[rr * pitch + Kc8 + t - rr * padn] = zero;
+  }
+}
+
+// After the last chunk: every token's rsqrt(mean(x^2) + eps) from its parts' sums, in part order.
+__device__ __forceinline__ void finish_norm(const float* ss_part, float* inv_rms, int M, int K, int parts, float eps) {
+  if (threadIdx.x < M) {
+    float total = 0.f;
+    for (int p = 0; p < parts; ++p) total += ss_part[threadIdx.x * parts + p];
+    inv_rms[threadIdx.x] = 1.0f / sqrtf(total / (float)K + eps);
+  }
+  __syncthreads();
+}
+
+// A finished tile: lane (col, kq) holds out[token tt * 16 + col][n0 + kq * 4 + (0..3)] of the 16 features from n0.
+template <int TT, int EPI, typename TO, bool NORM>
+__device__ __forceinline__ void finish_tile(const f32x4* sum, int n0, int M, int N, const float* __restrict__ bias,
+                                            TO* __restrict__ out, size_t ldo, const float* inv_rms, int col, int kq) {
+  const int nb = n0 + kq * 4;
+  f32x4 bv = {0.f, 0.f, 0.f, 0.f};
+  if (bias && EPI != EPI_SWIGLU) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) if (nb + r < N) bv[r] = bias[nb + r];
+  }
+#pragma unroll
+  for (int tt = 0; tt < TT; ++tt) {
+    const int m = tt * 16 + col;
+    if (m >= M) continue;
+    f32x4 v = sum[tt];
+    if (NORM) v *= inv_rms[m];
+    if (EPI == EPI_SWIGLU) {
+      // rows nb, nb+1 are (gate, up) of feature nb/2; rows nb+2, nb+3 of feature nb/2 + 1
+#pragma unroll
+      for (int p = 0; p < 2; ++p)
+        if (nb + 2 * p + 1 < N) out[(size_t)m * ldo + nb / 2 + p] = from_float<TO>(fast_silu(v[2 * p]) * v[2 * p + 1]);
+    } else {
+      TO* o = out + (size_t)m * ldo + nb;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        if (nb + r >= N) continue;
+        if (EPI == EPI_RESIDUAL) o[r] = from_float<TO>(to_float(o[r]) + v[r] + bv[r]);
+        else o[r] = from_float<TO>(v[r] + bv[r]);
+      }
+    }
+  }
+}
+
 template <int TT, int EPI, typename TO, bool NORM>
 __global__ void __launch_bounds__(WAVES * MS_WAVE)
 gemm_panel_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restrict__ W, size_t ldw,
@@ -50,8 +166,6 @@ gemm_panel_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restric
   extern __shared__ u32x4 smem[];   // the panel [tokens][pitch]; afterwards the waves' partial sums
   __shared__ float ss_part[MAX_TOKENS * MAX_PARTS];
   __shared__ float inv_rms[MAX_TOKENS];
-  const bf16* A = (const bf16*)Av;
-  const float* X = (const float*)Av;
   const int lane = threadIdx.x & (MS_WAVE - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MS_WAVE);   // the same for the whole wave
   const int col = lane & 15, kq = lane >> 4;
@@ -93,112 +207,16 @@ gemm_panel_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restric
   if (T_whole) fetch(wave, 0, 1);
   else if (shares) fetch(left_tile, j, g);
 
-  // ---- the panel.  A wave keeps to one 512-column part of the rows (so it loads that part of the norm weights
-  // once) and takes every (16 / parts2)-th token, BATCH of them in flight.
-  {
-    const int parts2 = parts <= 1 ? 1 : (parts <= 2 ? 2 : 4);
-    const int part = wave & (parts2 - 1);
-    const int tok_step = WAVES / parts2;
-    const int c = part * 64 + lane;
-    const bool in = c < K8;   // lanes past the row's end (and whole waves, when parts is 3) load nothing new
-    const int cc = min(c, K8 - 1) * 8;
-    f32x4 nwf[2];
-    if (NORM) {
-      nwf[0] = *reinterpret_cast<const f32x4*>(norm_w + cc);
-      nwf[1] = *reinterpret_cast<const f32x4*>(norm_w + cc + 4);
-    }
-    if (part < parts) {
-      for (int base = wave / parts2; base < M; base += tok_step * BATCH) {
-        u32x4 piece[NORM ? 1 : BATCH];
-        f32x4 xf[NORM ? BATCH : 1][2];
-#pragma unroll
-        for (int i = 0; i < BATCH; ++i) {
-          const int tok = base + i * tok_step;
-          if (tok >= M) break;   // the same for the whole wave
-          const size_t at = (size_t)(rows ? rows[tok] : tok) * lda + cc;
-          if (NORM) {
-            xf[i][0] = *reinterpret_cast<const f32x4*>(X + at);
-            xf[i][1] = *reinterpret_cast<const f32x4*>(X + at + 4);
-          } else {
-            piece[i] = *reinterpret_cast<const u32x4*>(A + at);
-          }
-        }
-#pragma unroll
-        for (int i = 0; i < BATCH; ++i) {
-          const int tok = base + i * tok_step;
-          if (tok >= M) break;
-          u32x4 pc;
-          if (NORM) {
-            bf16x8 h;
-            float ss = 0.f;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const float x0 = in ? xf[i][0][e] : 0.f, x1 = in ? xf[i][1][e] : 0.f;
-              ss = fmaf(x0, x0, ss);
-              ss = fmaf(x1, x1, ss);
-              h[e] = (__bf16)(x0 * nwf[0][e]);
-              h[4 + e] = (__bf16)(x1 * nwf[1][e]);
-            }
-            pc = __builtin_bit_cast(u32x4, h);
-            ss = wave_sum(ss);   // the lanes of a load in a fixed tree
-            if (lane == 0) ss_part[tok * parts + part] = ss;
-          } else {
-            pc = piece[i];
-          }
-          if (in) xst[tok * pitch + c] = pc;
-        }
-      }
-    }
-    // a last k-step that K fills only in part reads zeros for the rest
-    const int padn = S * 4 - K8;   // 0..3
-    for (int t = threadIdx.x; t < M * padn; t += WAVES * MS_WAVE) {
-      const int rr = t / padn;
-      xst[rr * pitch + K8 + t - rr * padn] = zero;
-    }
-  }
+  load_panel<NORM, BATCH>(Av, lda, norm_w, rows, M, 0, K8, S, parts, pitch, true, xst, ss_part, wave, lane);
   __syncthreads();
-  if (NORM) {
-    if (threadIdx.x < M) {   // a token's parts in order
-      float total = 0.f;
-      for (int p = 0; p < parts; ++p) total += ss_part[threadIdx.x * parts + p];
-      inv_rms[threadIdx.x] = 1.0f / sqrtf(total / (float)K + eps);
-    }
-    __syncthreads();
-  }
+  if (NORM) finish_norm(ss_part, inv_rms, M, K, parts, eps);
 
   int xrow[TT];   // idle columns repeat the last token; their results are not stored
 #pragma unroll
   for (int tt = 0; tt < TT; ++tt) xrow[tt] = min(tt * 16 + col, M - 1) * pitch + kq;
 
-  // what a lane holds of a finished tile: out[token tt * 16 + col][n0 + kq * 4 + (0..3)]
   auto finish = [&](int tl, f32x4* sum) {
-    const int nb = (t0 + tl) * 16 + kq * 4;
-    f32x4 bv = {0.f, 0.f, 0.f, 0.f};
-    if (bias && EPI != EPI_SWIGLU) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r) if (nb + r < N) bv[r] = bias[nb + r];
-    }
-#pragma unroll
-    for (int tt = 0; tt < TT; ++tt) {
-      const int m = tt * 16 + col;
-      if (m >= M) continue;
-      f32x4 v = sum[tt];
-      if (NORM) v *= inv_rms[m];
-      if (EPI == EPI_SWIGLU) {
-        // rows nb, nb+1 are (gate, up) of feature nb/2; rows nb+2, nb+3 of feature nb/2 + 1
-#pragma unroll
-        for (int p = 0; p < 2; ++p)
-          if (nb + 2 * p + 1 < N) out[(size_t)m * ldo + nb / 2 + p] = from_float<TO>(fast_silu(v[2 * p]) * v[2 * p + 1]);
-      } else {
-        TO* o = out + (size_t)m * ldo + nb;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          if (nb + r >= N) continue;
-          if (EPI == EPI_RESIDUAL) o[r] = from_float<TO>(to_float(o[r]) + v[r] + bv[r]);
-          else o[r] = from_float<TO>(v[r] + bv[r]);
-        }
-      }
-    }
+    finish_tile<TT, EPI, TO, NORM>(sum, (t0 + tl) * 16, M, N, bias, out, ldo, inv_rms, col, kq);
   };
 
   f32x4 acc[TT];
@@ -269,8 +287,6 @@ gemm_panel_chunked_kernel(const void* __restrict__ Av, size_t lda, const bf16* _
   extern __shared__ u32x4 smem[];   // the panel [tokens][pitch] of one chunk; afterwards the waves' partial sums
   __shared__ float ss_part[MAX_TOKENS * MAX_PARTS];
   __shared__ float inv_rms[MAX_TOKENS];
-  const bf16* A = (const bf16*)Av;
-  const float* X = (const float*)Av;
   const int lane = threadIdx.x & (MS_WAVE - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MS_WAVE);   // the same for the whole wave
   const int col = lane & 15, kq = lane >> 4;
@@ -299,12 +315,6 @@ gemm_panel_chunked_kernel(const void* __restrict__ Av, size_t lda, const bf16* _
   }
   const bool shares = T_left && left_tile < T_left;
 
-  // the panel's loads of this wave: one 512-column part of the chunk, every (16 / parts2)-th token
-  const int parts2 = parts <= 1 ? 1 : (parts <= 2 ? 2 : 4);
-  const int part = wave & (parts2 - 1);
-  const int tok_step = WAVES / parts2;
-  const int c = part * 64 + lane;
-
   int xrow[TT];   // idle columns repeat the last token; their results are not stored
 #pragma unroll
   for (int tt = 0; tt < TT; ++tt) xrow[tt] = min(tt * 16 + col, M - 1) * pitch + kq;
@@ -320,64 +330,7 @@ gemm_panel_chunked_kernel(const void* __restrict__ Av, size_t lda, const bf16* _
   for (int k0 = k_begin; k0 < k_end; k0 += KC) {
     const int Kc8 = min(KC, k_end - k0) / 8;  // pieces per row of this chunk
     const int S = (Kc8 + 3) / 4;              // its k-steps
-    // ---- the panel of columns k0 .. k0 + 8 * Kc8
-    {
-      const bool in = c < Kc8;
-      const int cc = k0 + min(c, Kc8 - 1) * 8;
-      f32x4 nwf[2];
-      if (NORM) {
-        nwf[0] = *reinterpret_cast<const f32x4*>(norm_w + cc);
-        nwf[1] = *reinterpret_cast<const f32x4*>(norm_w + cc + 4);
-      }
-      if (part < parts) {
-        for (int base = wave / parts2; base < M; base += tok_step * PB) {
-          u32x4 piece[NORM ? 1 : PB];
-          f32x4 xf[NORM ? PB : 1][2];
-#pragma unroll
-          for (int i = 0; i < PB; ++i) {
-            const int tok = base + i * tok_step;
-            if (tok >= M) break;   // the same for the whole wave
-            const size_t at = (size_t)(rows ? rows[tok] : tok) * lda + cc;
-            if (NORM) {
-              xf[i][0] = *reinterpret_cast<const f32x4*>(X + at);
-              xf[i][1] = *reinterpret_cast<const f32x4*>(X + at + 4);
-            } else {
-              piece[i] = *reinterpret_cast<const u32x4*>(A + at);
-            }
-          }
-#pragma unroll
-          for (int i = 0; i < PB; ++i) {
-            const int tok = base + i * tok_step;
-            if (tok >= M) break;
-            u32x4 pc;
-            if (NORM) {
-              bf16x8 h;
-              float ss = 0.f;
-#pragma unroll
-              for (int e = 0; e < 4; ++e) {
-                const float x0 = in ? xf[i][0][e] : 0.f, x1 = in ? xf[i][1][e] : 0.f;
-                ss = fmaf(x0, x0, ss);
-                ss = fmaf(x1, x1, ss);
-                h[e] = (__bf16)(x0 * nwf[0][e]);
-                h[4 + e] = (__bf16)(x1 * nwf[1][e]);
-              }
-              pc = __builtin_bit_cast(u32x4, h);
-              ss = wave_sum(ss);   // the lanes of a load in a fixed tree; a (token, part) is this wave's in every chunk
-              if (lane == 0) ss_part[tok * parts + part] = (k0 != k_begin ? ss_part[tok * parts + part] : 0.f) + ss;
-            } else {
-              pc = piece[i];
-            }
-            if (in) xst[tok * pitch + c] = pc;
-          }
-        }
-      }
-      // a last k-step that the chunk fills only in part reads zeros for the rest
-      const int padn = S * 4 - Kc8;   // 0..3
-      for (int t = threadIdx.x; t < M * padn; t += WAVES * MS_WAVE) {
-        const int rr = t / padn;
-        xst[rr * pitch + Kc8 + t - rr * padn] = zero;
-      }
-    }
+    load_panel<NORM, PB>(Av, lda, norm_w, rows, M, k0, Kc8, S, parts, pitch, k0 == k_begin, xst, ss_part, wave, lane);
     __syncthreads();
 
     // ---- this chunk's k-steps of the wave's tiles
@@ -414,43 +367,10 @@ gemm_panel_chunked_kernel(const void* __restrict__ Av, size_t lda, const bf16* _
     __syncthreads();   // the next chunk overwrites the panel
   }
 
-  if (NORM) {
-    if (threadIdx.x < M) {   // a token's parts in order (each the sum of its chunks in order)
-      float total = 0.f;
-      for (int p = 0; p < parts; ++p) total += ss_part[threadIdx.x * parts + p];
-      inv_rms[threadIdx.x] = 1.0f / sqrtf(total / (float)K + eps);
-    }
-    __syncthreads();
-  }
+  if (NORM) finish_norm(ss_part, inv_rms, M, K, parts, eps);
 
-  // what a lane holds of a finished tile: out[token tt * 16 + col][n0 + kq * 4 + (0..3)]
   auto finish = [&](int tl, f32x4* sum) {
-    const int nb = (t0 + tl) * 16 + kq * 4;
-    f32x4 bv = {0.f, 0.f, 0.f, 0.f};
-    if (bias && EPI != EPI_SWIGLU) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r) if (nb + r < N) bv[r] = bias[nb + r];
-    }
-#pragma unroll
-    for (int tt = 0; tt < TT; ++tt) {
-      const int m = tt * 16 + col;
-      if (m >= M) continue;
-      f32x4 v = sum[tt];
-      if (NORM) v *= inv_rms[m];
-      if (EPI == EPI_SWIGLU) {
-#pragma unroll
-        for (int p = 0; p < 2; ++p)
-          if (nb + 2 * p + 1 < N) out[(size_t)m * ldo + nb / 2 + p] = from_float<TO>(fast_silu(v[2 * p]) * v[2 * p + 1]);
-      } else {
-        TO* o = out + (size_t)m * ldo + nb;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          if (nb + r >= N) continue;
-          if (EPI == EPI_RESIDUAL) o[r] = from_float<TO>(to_float(o[r]) + v[r] + bv[r]);
-          else o[r] = from_float<TO>(v[r] + bv[r]);
-        }
-      }
-    }
+    finish_tile<TT, EPI, TO, NORM>(sum, (t0 + tl) * 16, M, N, bias, out, ldo, inv_rms, col, kq);
   };
 #pragma unroll
   for (int i = 0; i < NACC; ++i) {
