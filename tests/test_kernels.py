@@ -670,6 +670,19 @@ def test_split_decode_attention_of_a_large_uneven_batch(ops, R, nh, nkv, d, wind
     torch.testing.assert_close(_run_mfma(ops, c, nh, d, ctx, qlen, window), want, **tol(torch.bfloat16))
 
 
+@pytest.mark.parametrize("longest,splits_window", [(17000, None), (70000, None), (70000, 30000)])
+def test_split_decode_attention_of_very_long_contexts(ops, longest, splits_window):
+    """Tens of thousands of keys: more splits than at a few thousand (32 and 64), beside a short request that
+    uses one of them."""
+    nh, nkv, d = 4, 2, 64
+    g = torch.Generator().manual_seed(longest)
+    ctx, qlen = [longest, 40], [1, 1]
+    c = _paged_case(g, torch.bfloat16, nh, nkv, d, 16, ctx, qlen, float("nan"))
+    want = torch.cat([attention_reference(q.double(), k.double(), v.double(), 1.0 / math.sqrt(d), splits_window).transpose(0, 1).reshape(-1, nh * d)
+                      for q, k, v in zip(c["qs"], c["ks"], c["vs"])])
+    torch.testing.assert_close(_run_mfma(ops, c, nh, d, ctx, qlen, splits_window), want, **tol(torch.bfloat16))
+
+
 def _run_mfma(ops, c, nh, d, ctx, qlen, window=None):
     N = c["q"].shape[0]
     out = torch.full((N, nh * d), float("nan"), dtype=torch.bfloat16, device=DEV)
