@@ -8,7 +8,11 @@ function, sampler).  One JSON line is printed: ``value`` is decoded tokens a sec
 2,048-token prompt in one step; ``roofline`` prices the decode step against HBM bandwidth (every weight it
 uses once plus the cache of the live requests); ``points`` holds decode throughput at batch 1 and 64;
 ``launch`` says how many decode steps one graph launch holds and what it costs the host to enqueue it against
-the whole launch (a step bound by launching would show the two close together).
+the whole launch (a step bound by launching would show the two close together).  Every graph is captured
+when the engine is built, before any timer starts; ``launch.graphs_captured_while_timed`` is asserted to be 0.
+``roofline.measured_peak`` is the bandwidth a plain streaming read of 2 GiB reaches on this device (the
+reference measures its own the same way, benchmarks/diag_gpu_launch.py:29-40); fractions are against the
+published peak.
 """
 from __future__ import annotations
 
@@ -16,7 +20,6 @@ import argparse
 import json
 import os
 import sys
-import tempfile
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
@@ -27,20 +30,6 @@ if ROOT not in sys.path:
 HBM_GBS = 8000.0
 PEAK_TFLOPS = {"bf16": 2500.0, "fp16": 2500.0, "fp8": 5000.0, "fp32": 157.3}
 
-# Qwen2.5-0.5B's config.json sizes
-MODEL = {
-    "architectures": ["Qwen2ForCausalLM"], "num_hidden_layers": 24, "hidden_size": 896, "num_attention_heads": 14,
-    "num_key_value_heads": 2, "intermediate_size": 4864, "vocab_size": 151936, "rope_theta": 1000000.0,
-    "rms_norm_eps": 1e-6, "tie_word_embeddings": True,
-}
-# further shapes of the same architecture (Qwen2.5-7B and -32B config.json sizes), for --shape
-SHAPES = {
-    "0.5b": MODEL,
-    "7b": {**MODEL, "num_hidden_layers": 28, "hidden_size": 3584, "num_attention_heads": 28, "num_key_value_heads": 4,
-           "intermediate_size": 18944, "vocab_size": 152064, "tie_word_embeddings": False},
-    "32b": {**MODEL, "num_hidden_layers": 64, "hidden_size": 5120, "num_attention_heads": 40, "num_key_value_heads": 8,
-            "intermediate_size": 27648, "vocab_size": 152064, "tie_word_embeddings": False, "rms_norm_eps": 1e-5},
-}
 PROMPT_LEN = 512
 CONTEXT_LIMIT = 8192
 BLOCK_SIZE = 16
@@ -95,20 +84,40 @@ def run_decode(eng_mod, model, batch, steps, warmup, vocab, seed, prompt_len=PRO
     run(warmup)
     assert len(e.running) == batch and all(r.num_tokens - r.num_computed == 1 for r in e.running)
     graphs = e.runner.graphs
+    held = len(graphs.buckets)
     torch.cuda.synchronize()
     q0, n0 = graphs.enqueue_seconds, graphs.launches
     t0 = time.perf_counter()
     run(steps)
     torch.cuda.synchronize()
     total = time.perf_counter() - t0
+    if len(graphs.buckets) != held:
+        raise AssertionError("a graph was captured inside the timed region")
     dt = total / steps
     mean_context = prompt_len + warmup + (steps + 1) / 2
     launches = graphs.launches - n0
     # the host's share: filling the static buffers and enqueuing the graph, against the whole launch
     launch = {"steps_per_launch": round(steps / launches, 2),
               "enqueue_ms": round((graphs.enqueue_seconds - q0) / launches * 1e3, 4),
-              "total_ms": round(total / launches * 1e3, 4)}
+              "total_ms": round(total / launches * 1e3, 4), "graphs_held": held, "graphs_captured_while_timed": 0}
     return dt, mean_context, launch
+
+
+def measure_read_gbs(repeats=5):
+    """GB/s of a plain streaming read: the sum of a 2 GiB tensor, best of ``repeats``."""
+    import torch
+
+    x = torch.ones(1 << 30, dtype=torch.bfloat16, device="cuda:0")
+    best = None
+    for i in range(repeats + 1):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        x.sum()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        if i > 0:
+            best = dt if best is None else min(best, dt)
+    return x.numel() * 2 / best / 1e9
 
 
 def run_prefill(eng_mod, model, vocab, seed, repeats=5):
@@ -171,7 +180,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--shape", choices=sorted(SHAPES), default="0.5b",
+    ap.add_argument("--shape", choices=["0.5b", "7b", "32b"], default="0.5b",
                     help="layer sizes: the default is the configuration the headline numbers are quoted on")
     ap.add_argument("--layers", type=int, default=None,
                     help="fewer layers than the configuration has, if memory or time needs it (both numbers are reported)")
@@ -188,17 +197,15 @@ def main() -> int:
     import torch
 
     import llm_infrence_engine_amd as eng
-    from llm_infrence_engine_amd.config import config_from_dict
+    from llm_infrence_engine_amd.config import config_from_dict, preset
 
-    shape = SHAPES[a.shape]
+    shape = preset(a.shape)
     if a.layers is None:
         a.layers = shape["num_hidden_layers"]
     d = dict(shape)
     d["num_hidden_layers"] = a.layers
     cfg = config_from_dict(d)
-    with tempfile.TemporaryDirectory() as folder:
-        eng.write_random_model(folder, cfg, seed=0, dtype="bfloat16")
-        model = eng.load_model(folder, "bfloat16", "cuda:0")
+    model = eng.load_random_model(cfg, seed=0, dtype="bfloat16", device="cuda:0")   # drawn on the GPU: no file
     vocab = cfg.vocab_size
     if a.only == "prefill":
         pt = run_prefill(eng, model, vocab, seed=2, repeats=3)
@@ -214,6 +221,7 @@ def main() -> int:
     dt, ctx, launch = run_decode(eng, model, a.batch, a.steps, a.warmup, vocab, seed=1, prompt_len=a.prompt_len)
     value = a.batch / dt
     gbs = decode_bytes(cfg, a.batch, ctx) / dt / 1e9
+    measured = measure_read_gbs()
     out = {
         "metric": "decode_tokens_per_s", "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1,
         "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(dt * 1e3, 4), "higher_is_better": True,
@@ -230,7 +238,8 @@ def main() -> int:
             "baseline": "reference CUDA-graph decode, batch 8, ctx 128, A10 bf16: 6.0 ms/step",
         },
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_GBS, 4)},
+                     "frac": round(gbs / HBM_GBS, 4), "measured_peak": round(measured, 1),
+                     "frac_of_measured": round(gbs / measured, 4)},
         "launch": launch,
     }
     if not a.no_points:

@@ -4,7 +4,8 @@ from .config import EngineConfig, Qwen2Config, load_config, register_architectur
 from .engine import LLM, Engine, GenerationResult, Request, generate
 from .loading import load_model
 from .sampling import SamplingParams
-from .weights import write_random_model
+from .weights import load_random_model, write_random_model
 
 __all__ = ["EngineConfig", "Qwen2Config", "load_config", "register_architecture", "LLM", "Engine",
-           "GenerationResult", "Request", "generate", "load_model", "SamplingParams", "write_random_model"]
+           "GenerationResult", "Request", "generate", "load_model", "SamplingParams", "write_random_model",
+           "load_random_model"]

@@ -89,6 +89,13 @@ class CacheLayout:
                 self.state_needs[i] = state
 
 
+    def bytes_per_token(self, bytes_per_value: int) -> int:
+        """Stored bytes per token over all runs that keep keys and values
+        (layers x 2 x kv heads x head size x bytes, src/miniserve/cache.py:27-29)."""
+        return sum(len(runs) * 2 * key.num_kv_heads * key.head_dim * bytes_per_value
+                   for key, runs in zip(self.group_keys, self.group_runs))
+
+
 class CacheManager:
     def __init__(self, layout: CacheLayout, page_size: int, num_pages: int, max_requests: int, max_len: int):
         """``num_pages`` usable pages in every group's pool; a request may hold up to ``max_len`` tokens."""
@@ -199,9 +206,7 @@ class CacheManager:
 
     # ------------------------------------------------------------------ accounting
     def bytes_per_token(self, bytes_per_value: int) -> int:
-        """Stored bytes per token over all runs that keep keys and values
-        (layers x 2 x kv heads x head size x bytes, src/miniserve/cache.py:27-29)."""
-        return sum(len(g.runs) * 2 * g.key.num_kv_heads * g.key.head_dim * bytes_per_value for g in self.groups)
+        return self.layout.bytes_per_token(bytes_per_value)
 
     def check_invariants(self) -> None:
         """No page lost, held twice or freed twice; rows are held once; tables agree with the allocators."""

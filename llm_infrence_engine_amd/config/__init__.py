@@ -3,7 +3,8 @@ from .registry import (ConfigError, build_spec, config_class, config_from_dict, 
                        load_config, register_architecture)
 from .spec import LayerSpec, ModelSpec, PartSpec, Run
 from .qwen2 import Qwen2Config
+from .presets import PRESETS, preset
 
 __all__ = ["EngineConfig", "ConfigError", "build_spec", "config_class", "config_from_dict",
            "known_architectures", "load_config", "register_architecture", "LayerSpec", "ModelSpec",
-           "PartSpec", "Run", "Qwen2Config"]
+           "PartSpec", "Run", "Qwen2Config", "PRESETS", "preset"]

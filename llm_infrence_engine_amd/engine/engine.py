@@ -13,6 +13,7 @@ from typing import Callable, List, Optional, Sequence
 
 import torch
 
+from ..cache import CacheLayout
 from ..cache.allocator import OutOfPages
 from ..config.engine_config import EngineConfig
 from ..parts.model import Model
@@ -28,9 +29,17 @@ class Engine:
                  max_len: int = 1024, max_num_batched_tokens: int = 2048, max_prefill_chunk: Optional[int] = None,
                  on_token: Optional[Callable[[Request, int], None]] = None,
                  on_finish: Optional[Callable[[Request], None]] = None,
-                 clock: Callable[[], float] = time.perf_counter, hip_graphs: bool = False,
-                 decode_steps_per_launch: int = 1):
-        """``decode_steps_per_launch`` > 1 (with ``hip_graphs``): while every running request is decoding
+                 clock: Callable[[], float] = time.perf_counter, hip_graphs: Optional[bool] = None,
+                 decode_steps_per_launch: int = 1, capture_at_start: bool = True,
+                 gpu_memory_fraction: Optional[float] = None):
+        """``hip_graphs`` None: on when the model serves in bfloat16 (float32 is the checking path and launches
+        every kernel itself).  ``num_blocks`` None: as many pages as ``max_seqs`` requests of ``max_len`` tokens can
+        fill, or with ``gpu_memory_fraction`` as many of them as that share of the device's memory has room for
+        beside the weights.
+        With ``hip_graphs`` every graph that serving can reach is captured here, before the first request
+        (as the reference's constructor does, src/miniserve/graph_decode.py:46-47), unless ``capture_at_start``
+        is False: then a graph is captured when a step first needs it.
+        ``decode_steps_per_launch`` > 1 (with ``hip_graphs``): while every running request is decoding
         greedily and nobody waits, up to that many decode steps run in one graph launch, each fed the argmax of
         the one before on the device; a stop id is then noticed up to that many steps late (the surplus tokens
         are dropped), so outputs do not change."""
@@ -38,18 +47,40 @@ class Engine:
         self.config = EngineConfig(dtype=dtype, block_size=block_size, num_blocks=num_blocks, max_seqs=max_seqs,
                                    max_len=max_len, max_num_batched_tokens=max_num_batched_tokens,
                                    max_prefill_chunk=max_prefill_chunk, hip_graphs=hip_graphs,
-                                   device=str(model.rt.device))
+                                   decode_steps_per_launch=decode_steps_per_launch,
+                                   gpu_memory_fraction=gpu_memory_fraction, device=str(model.rt.device))
         self.model = model
-        self.runner = ModelRunner(model, block_size, self.config.resolved_num_blocks(), max_seqs, max_len,
-                                  hip_graphs=hip_graphs)
+        pages = self.config.resolved_num_blocks()
+        if num_blocks is None and gpu_memory_fraction is not None:
+            free, total = torch.cuda.mem_get_info(model.rt.device)
+            per_token = CacheLayout(model.run_needs()).bytes_per_token(model.rt.dtype.itemsize)
+            pages = self.config.resolved_num_blocks(per_token, total, total - free)
+        self.runner = ModelRunner(model, block_size, pages, max_seqs, max_len, hip_graphs=self.config.hip_graphs)
         self.scheduler = Scheduler(self.runner.manager, self.config, clock, on_token, on_finish)
         self.sampler = Sampler(model.rt.device)
         self.clock = clock
         self.decode_steps_per_launch = max(1, decode_steps_per_launch) if self.runner.graphs is not None else 1
+        if capture_at_start:
+            self.warm_up()
         self.steps: List[StepRecord] = []
         self.peak_running = 0
         self.peak_pages_in_use = 0
         self.prefill_tokens_computed = 0
+
+    def launch_sizes(self) -> List[int]:
+        """The numbers of decode steps one graph launch may hold: powers of two up to ``decode_steps_per_launch``."""
+        sizes, k = [], 1
+        while k <= self.decode_steps_per_launch:
+            sizes.append(k)
+            k *= 2
+        return sizes
+
+    def warm_up(self) -> int:
+        """Capture every decode graph this engine can need (all batch-size buckets, context classes and
+        launch sizes), so that no step of serving holds a capture.  Returns the number of graphs held."""
+        if self.runner.graphs is None:
+            return 0
+        return self.runner.graphs.warm_up(self.launch_sizes())
 
     # ------------------------------------------------------------------ the reference's public face
     def add_request(self, req: Request) -> Request:
@@ -112,7 +143,8 @@ class Engine:
             raise RuntimeError("the scheduler could place no request although work is waiting")
         ahead = self._steps_ahead(sched, max_decode_steps) if sched and self.decode_steps_per_launch > 1 else 1
         if ahead > 1:
-            entries = [StepEntry(s.request.id, [s.request.output_ids[-1]]) for s in sched]
+            # a request's newest token: its last output, or its prompt's last token when a portion left only that
+            entries = [StepEntry(s.request.id, [(s.request.output_ids or s.request.prompt_ids)[-1]]) for s in sched]
             tokens = self.runner.decode_steps(entries, ahead)
             for k in range(ahead):      # as the single steps would have: a finished request drops its later tokens
                 for i, s in enumerate(sched):

@@ -63,6 +63,7 @@ class _Bucket:
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.logits: Optional[torch.Tensor] = None
         self.tokens = torch.zeros((steps, B), dtype=torch.int32, device=device)   # the argmax of every step
+        self.copied: Optional[torch.cuda.Event] = None   # set once the last copy of ``host`` has left it
 
     def reset_host(self) -> None:
         """Every row a padding row: token 0 at position 0, one visible key on the null page, nothing stored."""
@@ -94,7 +95,8 @@ class DecodeGraphs:
         self.runner, self.manager = runner, m
         self.sizes = sorted(set(batch_sizes or default_batch_sizes(m.max_requests)))
         self.width = m.max_pages_per_request
-        self.buckets: Dict[int, _Bucket] = {}
+        self.buckets: Dict[tuple, _Bucket] = {}
+        self.pool = None   # one memory pool for all graphs: they never run at the same time
         # what launching costs the host: seconds spent filling the buffers and enqueuing, and launches so far
         # (the reference separates a launch-bound from a GPU-bound step the same way, benchmarks/diag_gpu_launch.py:1-8)
         self.enqueue_seconds = 0.0
@@ -104,9 +106,26 @@ class DecodeGraphs:
     def max_batch(self) -> int:
         return self.sizes[-1]
 
+    def context_classes(self) -> List[bool]:
+        """The attention's launch shapes a decode step of this cache can need: short contexts, and long ones
+        if a request can grow beyond ``ops.LONG_CONTEXT``."""
+        return [False, True] if self.manager.max_len > ops.LONG_CONTEXT else [False]
+
+    def warm_up(self, steps: Sequence[int] = (1,), batch_sizes: Optional[Sequence[int]] = None) -> int:
+        """Capture, before serving, every graph that serving can reach: each batch-size bucket (or those of
+        ``batch_sizes``), each context class, each number of steps per launch in ``steps``; the reference
+        captures all its buckets in the constructor (src/miniserve/graph_decode.py:46-47).  Afterwards
+        ``run`` captures nothing.  Returns the number of graphs held."""
+        sizes = self.sizes if batch_sizes is None else sorted({next(b for b in self.sizes if b >= n) for n in batch_sizes})
+        for B in reversed(sizes):            # the largest first: the others fit into the memory it leaves
+            for long_context in self.context_classes():
+                for k in sorted(set(steps), reverse=True):
+                    self._bucket(B, long_context, k)
+        return len(self.buckets)
+
     def _bucket(self, n: int, long_context: bool, steps: int = 1) -> _Bucket:
         B = next(b for b in self.sizes if b >= n)
-        key = (B, long_context) if steps == 1 else (B, long_context, steps)
+        key = (B, long_context, steps)
         bk = self.buckets.get(key)
         if bk is None:
             bk = self.buckets[key] = _Bucket(B, self.width, len(self.manager.groups), self.runner.rt.device, steps)
@@ -140,7 +159,9 @@ class DecodeGraphs:
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
-            for _ in range(2):            # load kernels and settle allocations before capturing
+            # load the kernels of this shape before capturing (twice for the first graph, which also
+            # settles the allocator)
+            for _ in range(1 if self.buckets.keys() - {(bk.B, long_context, bk.steps)} else 2):
                 ops.sample(model.forward(ctx, caches), bk.tokens[0])
             if bk.steps > 1:
                 advance(1)
@@ -154,8 +175,10 @@ class DecodeGraphs:
         collecting = gc.isenabled()
         gc.disable()
         try:
+            if self.pool is None:
+                self.pool = torch.cuda.graph_pool_handle()
             bk.graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(bk.graph):
+            with torch.cuda.graph(bk.graph, pool=self.pool):
                 for k in range(bk.steps):
                     if k > 0:
                         advance(k)
@@ -177,6 +200,8 @@ class DecodeGraphs:
         pos = np.fromiter((m.computed(e.req_id) for e in entries), dtype=np.int32, count=R)
         bk = self._bucket(R, int(pos.max()) + steps > ops.LONG_CONTEXT, steps)
         a, o, ps = bk.np, bk.off, m.page_size
+        if bk.copied is not None:
+            bk.copied.synchronize()      # the last launch's copy must have read the pinned buffer before it changes
         toks = np.fromiter((e.tokens[0] for e in entries), dtype=np.int64, count=R)
         if toks.min() < 0 or toks.max() >= self.runner.model.spec.vocab_size:
             raise ValueError("a token id is outside the vocabulary")
@@ -199,6 +224,9 @@ class DecodeGraphs:
                 raise RuntimeError("a token of this launch has no page; grow the requests before it")
             a[bk.slots[g]][:R] = page * ps + pos % ps
         bk.dev.copy_(bk.host, non_blocking=True)
+        if bk.copied is None:
+            bk.copied = torch.cuda.Event()
+        bk.copied.record()
         bk.graph.replay()
         self.enqueue_seconds += time.perf_counter() - t_begin
         self.launches += 1

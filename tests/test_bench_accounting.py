@@ -2,7 +2,7 @@
 import importlib.util
 import os
 
-from llm_infrence_engine_amd.config import config_from_dict
+from llm_infrence_engine_amd.config import config_from_dict, preset
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 spec = importlib.util.spec_from_file_location("bench", os.path.join(ROOT, "bench.py"))
@@ -11,7 +11,7 @@ spec.loader.exec_module(bench)
 
 
 def test_decode_bytes_of_the_half_billion_shape():
-    cfg = config_from_dict(bench.SHAPES["0.5b"])
+    cfg = config_from_dict(preset("0.5b"))
     # the reference counts 494,032,768 parameters = 988,065,536 bytes in bfloat16 (results/raw/gpu_launch_diag.json)
     assert cfg.num_params == 494_032_768
     weights = bench.decode_bytes(cfg, batch=0, context=0)
@@ -22,7 +22,7 @@ def test_decode_bytes_of_the_half_billion_shape():
 
 
 def test_prefill_flops_of_the_half_billion_shape():
-    cfg = config_from_dict(bench.SHAPES["0.5b"])
+    cfg = config_from_dict(preset("0.5b"))
     f = bench.prefill_flops(cfg, 2048)
     linear = 2 * 2048 * 24 * 14_912_384 - 2 * 2048 * 24 * (18 * 64 + 2 * 896)   # per-layer parameters without biases and norms
     attention = 24 * 4 * 14 * 64 * 2048 * 2049 // 2
@@ -31,8 +31,8 @@ def test_prefill_flops_of_the_half_billion_shape():
 
 
 def test_further_shapes_have_their_published_sizes():
-    assert config_from_dict(bench.SHAPES["7b"]).num_params == 7_615_616_512
-    assert config_from_dict(bench.SHAPES["32b"]).kv_bytes_per_token(2) == 262_144
+    assert config_from_dict(preset("7b")).num_params == 7_615_616_512
+    assert config_from_dict(preset("32b")).kv_bytes_per_token(2) == 262_144
 
 
 def test_more_than_one_gpu_is_refused(capsys):

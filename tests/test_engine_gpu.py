@@ -229,11 +229,12 @@ def test_hip_graph_decode_equals_eager(tiny, eng, dtype):
             out.append(r.step([StepEntry(2, [seqs[2][34 + p]], [0]), StepEntry(0, [seqs[0][37 + p]], [0])]).cpu())
         runs[graphs] = out
         if graphs:
-            assert sorted(r.graphs.buckets) == [(1, False), (2, False), (4, False)]
+            assert sorted(r.graphs.buckets) == [(1, False, 1), (2, False, 1), (4, False, 1)]
     for a, b in zip(runs[False], runs[True]):
         assert torch.equal(a, b)
     exact = P.forward(w, cfg, seqs[2]).numpy()
-    assert np.abs(runs[True][-1][0].numpy() - exact[36]).max() < (1e-3 if dtype == "float32" else 0.5)
+    noise = np.abs(P.forward(w, cfg, seqs[2], act_dtype=torch.bfloat16).numpy() - exact).max()
+    assert np.abs(runs[True][-1][0].numpy() - exact[36]).max() < (1e-3 if dtype == "float32" else 3.0 * noise)
 
 
 def test_generation_with_hip_graphs(tiny, eng):
@@ -292,7 +293,7 @@ def test_long_context_decode_splits_keys_and_matches_plain(eng, tmp_path):
             for row, q in zip(lg, ("a", "b")):
                 assert np.abs(row - exact[q][cut[q] + i]).max() < 3.0 * noise[q], (graphs, q, i)
         if graphs:
-            assert sorted(r.graphs.buckets) == [(2, False), (2, True)]   # it crossed from short to long on the way
+            assert sorted(r.graphs.buckets) == [(2, False, 1), (2, True, 1)]   # it crossed from short to long on the way
 
 
 def test_large_uneven_decode_batch_matches_plain(eng, tmp_path):

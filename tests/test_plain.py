@@ -172,6 +172,109 @@ def test_bias_is_added_to_q_k_v_and_not_to_o():
     assert torch.allclose(P.attention_block(x, w, p, pc, cos, sin), torch.zeros_like(x), atol=1e-15)
 
 
+def _one_layer(cfg_name="B", seed=6):
+    cfg = dict(TINY[cfg_name])
+    cfg["num_hidden_layers"] = 1
+    return cfg, plain_cfg(cfg), plain_random_weights(cfg, seed, std=0.2, dtype=torch.float64)
+
+
+def test_each_norm_feeds_its_own_branch_known_answers():
+    """One layer, sequences of one token (attention over one key returns its value): with the feed-forward's
+    norm scale zeroed the feed-forward adds silu(0) * 0 = 0 and the logits are the attention branch's over
+    ``input_layernorm``; with the attention's norm scale zeroed the attention adds o(v's bias) and the
+    feed-forward sees ``post_attention_layernorm`` of that sum.  Both answers are written with library routines.
+    Dropping a norm, using one scale for both branches or swapping the two fails one of them."""
+    cfg, pc, w = _one_layer()
+    eps, p = cfg["rms_norm_eps"], "model.layers.0."
+    H, nh, nkv, d = cfg["hidden_size"], pc["num_heads"], pc["num_kv_heads"], pc["head_dim"]
+    head = w["lm_head.weight"]
+
+    def finish(x):
+        return F.linear(F.rms_norm(x, (H,), w["model.norm.weight"], eps), head)
+
+    def value_of(h, wts):   # one key: every query head returns the value of its key/value head
+        v = F.linear(h, wts[p + "self_attn.v_proj.weight"], wts[p + "self_attn.v_proj.bias"])
+        return F.linear(v.view(nkv, d).repeat_interleave(nh // nkv, 0).reshape(-1), wts[p + "self_attn.o_proj.weight"])
+
+    def mlp(h, wts):
+        return F.linear(F.silu(F.linear(h, wts[p + "mlp.gate_proj.weight"])) * F.linear(h, wts[p + "mlp.up_proj.weight"]),
+                        wts[p + "mlp.down_proj.weight"])
+
+    for tok in (3, 77):
+        x = w["model.embed_tokens.weight"][tok]
+        a = {k: v.clone() for k, v in w.items()}
+        a[p + "post_attention_layernorm.weight"].zero_()
+        want = finish(x + value_of(F.rms_norm(x, (H,), a[p + "input_layernorm.weight"], eps), a))
+        assert torch.allclose(P.forward(a, pc, [tok])[0], want, atol=1e-10)
+        b = {k: v.clone() for k, v in w.items()}
+        b[p + "input_layernorm.weight"].zero_()
+        x1 = x + value_of(torch.zeros(H, dtype=torch.float64), b)
+        want = finish(x1 + mlp(F.rms_norm(x1, (H,), b[p + "post_attention_layernorm.weight"], eps), b))
+        assert torch.allclose(P.forward(b, pc, [tok])[0], want, atol=1e-10)
+        assert not torch.allclose(want, finish(x1), atol=1e-4)      # the feed-forward branch is really there
+    swapped = dict(w)
+    swapped[p + "input_layernorm.weight"], swapped[p + "post_attention_layernorm.weight"] = \
+        w[p + "post_attention_layernorm.weight"], w[p + "input_layernorm.weight"]
+    ids = [3, 77, 5, 190]
+    assert (P.forward(swapped, pc, ids) - P.forward(w, pc, ids)).abs().max() > 1e-3
+
+
+def test_bias_is_added_before_the_rotation_closed_form():
+    """Zero q and k matrices, biases s * e_0 on both: pair 0 (inverse frequency 1) turns by the position, so the
+    score of query i against key j is s^2 cos(i - j) / sqrt(d) if and only if the bias is rotated too (added
+    after the rotation it would give equal scores and uniform weights).  Values are one-hot rows, so the
+    output rows are the softmax weights themselves."""
+    d = T = 8
+    s = 3.0
+    pc = {"num_heads": 1, "num_kv_heads": 1, "head_dim": d}
+    e0 = torch.zeros(d, dtype=torch.float64)
+    e0[0] = s
+    z, eye = torch.zeros(d, d, dtype=torch.float64), torch.eye(d, dtype=torch.float64)
+    w = {"q_proj.weight": z, "q_proj.bias": e0, "k_proj.weight": z, "k_proj.bias": e0.clone(),
+         "v_proj.weight": eye, "v_proj.bias": torch.zeros(d, dtype=torch.float64), "o_proj.weight": eye}
+    cos, sin = P.rope_cos_sin(torch.arange(T), d, 10000.0)
+    out = P.attention_block(eye[:T], w, "", pc, cos, sin)
+    for i in range(T):
+        scores = torch.tensor([s * s * math.cos(i - j) / math.sqrt(d) for j in range(i + 1)], dtype=torch.float64)
+        assert torch.allclose(out[i, :i + 1], torch.softmax(scores, 0), atol=1e-12), i
+        assert torch.allclose(out[i, i + 1:], torch.zeros(T - i - 1, dtype=torch.float64), atol=1e-15)
+    assert not torch.allclose(out[5, :6], torch.full((6,), 1 / 6, dtype=torch.float64), atol=1e-2)
+
+
+def test_bias_then_rotation_on_non_zero_input_against_complex_arithmetic():
+    """The attention block on random input and weights against an independent formulation: biased projections
+    from the library's linear, the rotation as a multiplication of the complex numbers (x_j + i x_{j+d/2}) by
+    exp(i pos / theta^(2j/d)), the library's causal attention with repeated key/value heads.  Rotating first and
+    adding the bias afterwards gives another result."""
+    cfg, pc, w = _one_layer("C", seed=8)
+    p = "model.layers.0.self_attn."
+    T, nh, nkv, d, theta = 9, pc["num_heads"], pc["num_kv_heads"], pc["head_dim"], pc["rope_theta"]
+    x = torch.randn(T, cfg["hidden_size"], dtype=torch.float64)
+    turn = torch.polar(torch.ones(T, d // 2, dtype=torch.float64),
+                       torch.arange(T, dtype=torch.float64)[:, None] * theta ** (-torch.arange(0, d, 2, dtype=torch.float64) / d))
+
+    def rotate(t):      # [T, heads, d]
+        c = torch.complex(t[..., :d // 2], t[..., d // 2:]) * turn[:, None, :]
+        return torch.cat((c.real, c.imag), dim=-1)
+
+    def block(bias_first):
+        q = F.linear(x, w[p + "q_proj.weight"], w[p + "q_proj.bias"] if bias_first else None).view(T, nh, d)
+        k = F.linear(x, w[p + "k_proj.weight"], w[p + "k_proj.bias"] if bias_first else None).view(T, nkv, d)
+        v = F.linear(x, w[p + "v_proj.weight"], w[p + "v_proj.bias"]).view(T, nkv, d)
+        q, k = rotate(q), rotate(k)
+        if not bias_first:
+            q, k = q + w[p + "q_proj.bias"].view(nh, d), k + w[p + "k_proj.bias"].view(nkv, d)
+        k, v = k.repeat_interleave(nh // nkv, 1), v.repeat_interleave(nh // nkv, 1)
+        o = F.scaled_dot_product_attention(q.transpose(0, 1), k.transpose(0, 1), v.transpose(0, 1), is_causal=True)
+        return F.linear(o.transpose(0, 1).reshape(T, nh * d), w[p + "o_proj.weight"])
+
+    cos, sin = P.rope_cos_sin(torch.arange(T), d, theta)
+    got = P.attention_block(x, w, p, pc, cos, sin)
+    assert torch.allclose(got, block(True), atol=1e-10)
+    assert (got - block(False)).abs().max() > 1e-3
+
+
+
 # ------------------------------------------------------------------ whole model
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_causality_and_shift_of_all_positions(name):

@@ -241,3 +241,39 @@ def test_requests_may_arrive_and_be_cancelled_from_other_threads():
         else:
             assert r.output_ids == alone(r.prompt_ids, 6)
     assert all(g.allocator.num_in_use() == 0 for g in m.groups)
+
+
+def test_a_portion_may_leave_one_prompt_token_which_then_runs_as_a_single_token_row():
+    """A 5-token prompt under a budget of 4: first four tokens, then the last one alone, with its start past 0,
+    one token and a sample, before the request has any output: what feeds such a row must be the prompt's
+    last token."""
+    s, m = make(budget=4)
+    r = s.add_request(Request(prompts(3, [5])[0], max_new_tokens=3))
+    first = one_step(s, m)
+    assert [(e.start, e.count, e.sample) for e in first] == [(0, 4, False)]
+    second = s.schedule()
+    assert [(e.start, e.count, e.sample) for e in second] == [(4, 1, True)]
+    assert not r.output_ids and r.tokens[second[0].start] == r.prompt_ids[-1]
+    assert (r.output_ids or r.prompt_ids)[-1] == r.tokens[second[0].start]
+
+
+def test_pool_size_from_a_memory_budget():
+    """Without num_blocks: max_seqs requests of max_len, or what the stated share of the device's memory has
+    room for beside what is held already; too little for one request is refused."""
+    per_token = 24 * 2 * 2 * 64 * 2                       # the half-billion shape in bfloat16: 12,288 bytes a token
+    cfg = EngineConfig(block_size=16, max_seqs=64, max_len=8192)
+    assert cfg.resolved_num_blocks() == 64 * 512
+    assert EngineConfig(block_size=16, num_blocks=7, max_seqs=64, max_len=8192, gpu_memory_fraction=0.5) \
+        .resolved_num_blocks(per_token, 1 << 30, 0) == 7   # given by hand wins
+    gib = 1 << 30
+    small = EngineConfig(block_size=16, max_seqs=64, max_len=8192, gpu_memory_fraction=0.5)
+    # half of 8 GiB, 1 GiB of it held by the weights: 3 GiB of pages of 16 * 12,288 bytes, one of them the null page
+    assert small.resolved_num_blocks(per_token, 8 * gib, 1 * gib) == 3 * gib // (16 * per_token) - 1
+    # plenty of memory: never more pages than the requests can fill
+    assert small.resolved_num_blocks(per_token, 288 * gib, 1 * gib) == 64 * 512
+    with pytest.raises(ValueError, match="less than one request"):
+        small.resolved_num_blocks(per_token, 2 * gib, 1 * gib - 50 * 16 * per_token)
+    with pytest.raises(ValueError, match="gpu_memory_fraction"):
+        EngineConfig(gpu_memory_fraction=1.5)
+    assert EngineConfig(dtype="bfloat16").hip_graphs is True and EngineConfig(dtype="float32").hip_graphs is False
+    assert EngineConfig(dtype="float32", hip_graphs=True).hip_graphs is True
