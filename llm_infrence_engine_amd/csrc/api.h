@@ -81,6 +81,21 @@ int ms_paged_attention_mfma_decode(const void* q, long long q_stride, const void
 int ms_argmax(const float* logits, long long ld, int n_rows, int vocab, float* scratch_val, int* scratch_idx,
               int n_chunks, int* out, hipStream_t stream);
 
+// The one entry point that allocates nothing.  It has no counterpart in the reference; it is for callers that
+// cannot allocate device memory: code under HIP graph capture, tight serving loops, harnesses that forbid
+// hipMalloc.  Same result as ms_argmax, but the stage-1 results live in a static device array of the library
+// (256 KB on every GPU the library runs on, held until the process ends) instead of scratch_val / scratch_idx.
+// The caller still passes logits and out; `stream` must belong to the current device.  Limits: n_rows <= 256
+// and n_chunks <= 128 (ms_argmax_static_limits reports them); beyond them the call returns MS_UNSUPPORTED (2)
+// and launches nothing.  All calls on one GPU share that GPU's array: calls that overlap on one GPU (different
+// streams or threads) race; calls on one stream, or ordered by events, do not.  Nothing in the array needs
+// clearing between calls.  The array's address is looked up once per device, at the first call there or by
+// ms_argmax_static_init() with that device current (call it before a stream capture starts).
+int ms_argmax_static_init();
+void ms_argmax_static_limits(int* max_rows, int* max_chunks);
+int ms_argmax_static(const float* logits, long long ld, int n_rows, int vocab, int n_chunks, int* out,
+                     hipStream_t stream);
+
 int ms_sample(const float* logits, long long ld, int n_rows, int vocab, const float* temperature, const int* top_k,
               const float* top_p, const unsigned long long* seeds, const int* draw_index, int* out,
               hipStream_t stream);

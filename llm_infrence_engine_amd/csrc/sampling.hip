@@ -8,6 +8,7 @@
 // uniform number of a draw is Philox4x32-10(seed, draw index): the same seed and index give the same token.
 #include "common.h"
 #include "api.h"
+#include <mutex>
 
 namespace {
 
@@ -192,6 +193,28 @@ argmax_final_kernel(const float* __restrict__ val, const int* __restrict__ idx, 
 
 }  // namespace
 
+// ---- the stage-1 results of ms_argmax_static: values first, then indices.  A file-scope array: every GPU the
+// library runs on holds its own copy (256 KB) at its own address until the process ends.
+constexpr int STATIC_MAX_ROWS = 256, STATIC_MAX_CHUNKS = 128, STATIC_MAX_DEVICES = 64;
+static __device__ __align__(256) unsigned char scratch[(size_t)STATIC_MAX_ROWS * STATIC_MAX_CHUNKS * (sizeof(float) + sizeof(int))];
+// In host code `scratch` is only a handle for the symbol; what kernels may dereference is the address
+// that hipGetSymbolAddress returns for the current device, looked up once per device and kept here.
+static void* scratch_addr[STATIC_MAX_DEVICES] = {};
+static std::mutex scratch_mutex;
+
+// Device address of `scratch` on the current device (nullptr: the lookup failed or the device index is too large).
+static void* scratch_of_current_device() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= STATIC_MAX_DEVICES) return nullptr;
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (scratch_addr[dev] == nullptr) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess) return nullptr;
+    scratch_addr[dev] = p;
+  }
+  return scratch_addr[dev];
+}
+
 // out[r] = first index of the maximum of logits[r, :].  scratch_val / scratch_idx: [n_rows, n_chunks].
 extern "C" int ms_argmax(const float* logits, long long ld, int n_rows, int vocab, float* scratch_val,
                          int* scratch_idx, int n_chunks, int* out, hipStream_t stream) {
@@ -200,6 +223,30 @@ extern "C" int ms_argmax(const float* logits, long long ld, int n_rows, int voca
   argmax_chunks_kernel<<<dim3(n_chunks, n_rows), dim3(256), 0, stream>>>(logits, (size_t)ld, vocab, n_chunks,
                                                                           scratch_val, scratch_idx);
   argmax_final_kernel<<<dim3(n_rows), dim3(MS_WAVE), 0, stream>>>(scratch_val, scratch_idx, n_chunks, out);
+  return ms_launch_status();
+}
+
+extern "C" int ms_argmax_static_init() { return scratch_of_current_device() ? MS_OK : MS_LAUNCH_FAILED; }
+
+extern "C" void ms_argmax_static_limits(int* max_rows, int* max_chunks) {
+  if (max_rows) *max_rows = STATIC_MAX_ROWS;
+  if (max_chunks) *max_chunks = STATIC_MAX_CHUNKS;
+}
+
+// ms_argmax with the stage-1 results in the library's own static device array instead of caller-provided
+// buffers: nothing is allocated or freed here.  Nothing in the array has to start at zero (stage 2 reads only
+// what stage 1 of the same call wrote, with this call's row stride), so the last call's contents are harmless.
+extern "C" int ms_argmax_static(const float* logits, long long ld, int n_rows, int vocab, int n_chunks, int* out,
+                                hipStream_t stream) {
+  if (n_rows <= 0) return MS_OK;
+  if (vocab <= 0 || ld < vocab || n_chunks <= 0 || logits == nullptr || out == nullptr) return MS_BAD_ARG;
+  if (n_rows > STATIC_MAX_ROWS || n_chunks > STATIC_MAX_CHUNKS) return MS_UNSUPPORTED;
+  unsigned char* base = (unsigned char*)scratch_of_current_device();
+  if (base == nullptr) return MS_LAUNCH_FAILED;
+  float* val = (float*)base;
+  int* idx = (int*)(base + (size_t)STATIC_MAX_ROWS * STATIC_MAX_CHUNKS * sizeof(float));
+  argmax_chunks_kernel<<<dim3(n_chunks, n_rows), dim3(256), 0, stream>>>(logits, (size_t)ld, vocab, n_chunks, val, idx);
+  argmax_final_kernel<<<dim3(n_rows), dim3(MS_WAVE), 0, stream>>>(val, idx, n_chunks, out);
   return ms_launch_status();
 }
 
