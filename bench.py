@@ -69,7 +69,11 @@ def run_decode(eng_mod, model, batch, steps, warmup, vocab, seed, prompt_len=PRO
     need = prompt_len + warmup + steps + extra
     pages = batch * (-(-need // BLOCK_SIZE) + 1)
     e = eng_mod.Engine(model, num_blocks=pages, block_size=BLOCK_SIZE, max_seqs=batch, max_len=CONTEXT_LIMIT,
-                       max_num_batched_tokens=budget, hip_graphs=True, decode_steps_per_launch=DECODE_STEPS_PER_LAUNCH)
+                       max_num_batched_tokens=budget, hip_graphs=True, decode_steps_per_launch=DECODE_STEPS_PER_LAUNCH,
+                       capture_at_start=False)
+    # every graph this run can reach, before any timer: all requests stay alive, so the one bucket of ``batch``
+    # rows, in both context classes and every launch size (an engine that serves captures all buckets itself)
+    e.runner.graphs.warm_up(e.launch_sizes(), batch_sizes=[batch])
     for _ in range(batch):
         e.add_request(eng_mod.Request([int(t) for t in rng.integers(0, vocab, prompt_len)],
                                       max_new_tokens=warmup + steps + extra))
@@ -104,15 +108,17 @@ def run_decode(eng_mod, model, batch, steps, warmup, vocab, seed, prompt_len=PRO
 
 
 def measure_read_gbs(repeats=5):
-    """GB/s of a plain streaming read: the sum of a 2 GiB tensor, best of ``repeats``."""
+    """GB/s of a plain streaming read of 2 GiB by a kernel that does nothing else, best of ``repeats``."""
     import torch
+
+    from llm_infrence_engine_amd.kernels import ops
 
     x = torch.ones(1 << 30, dtype=torch.bfloat16, device="cuda:0")
     best = None
     for i in range(repeats + 1):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        x.sum()
+        ops.read_probe(x)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         if i > 0:

@@ -19,6 +19,10 @@ int ms_decode_advance(const int* prev_tokens, int* token_ids, int* positions, in
                       const int* const* tables, int* const* slots, int n_groups, int table_stride, int page_size,
                       int n_rows, hipStream_t stream);
 
+// A plain streaming read of `bytes` for bandwidth measurements; sink: unsigned [ms_read_probe_blocks()].
+int ms_read_probe_blocks();
+int ms_read_probe(const void* base, long long bytes, unsigned* sink, hipStream_t stream);
+
 int ms_residual_add(float* x, const void* delta, long long total, int dtype, hipStream_t stream);
 
 int ms_silu_mul(const void* gate_up, void* out, int n_tokens, int intermediate, int dtype, hipStream_t stream);

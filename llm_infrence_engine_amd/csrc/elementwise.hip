@@ -419,3 +419,38 @@ extern "C" int ms_decode_advance(const int* prev_tokens, int* token_ids, int* po
   decode_advance_kernel<<<dim3((n_rows + 63) / 64), dim3(64), 0, stream>>>(a);
   return ms_launch_status();
 }
+
+// ------------------------------------------------------------------------------------------------
+// A plain streaming read of `bytes` (a multiple of 16, 16-byte aligned), for measuring what bandwidth this
+// device gives a kernel that does nothing else: every wave asks for 1 KB at a time, four requests in flight,
+// the blocks dealt contiguous shares.  The exclusive-or of everything read goes to sink[block] so that the
+// loads cannot be dropped.
+__global__ void __launch_bounds__(1024)
+read_probe_kernel(const uint4* __restrict__ base, size_t n16, unsigned* __restrict__ sink) {
+  const size_t per_block = (n16 + gridDim.x - 1) / gridDim.x;
+  const size_t begin = (size_t)blockIdx.x * per_block, end = begin + per_block < n16 ? begin + per_block : n16;
+  uint4 acc = {0u, 0u, 0u, 0u};
+  for (size_t i = begin + threadIdx.x; i < end; i += (size_t)4 * blockDim.x) {
+    uint4 v[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const size_t k = i + (size_t)j * blockDim.x;
+      v[j] = k < end ? base[k] : uint4{0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { acc.x ^= v[j].x; acc.y ^= v[j].y; acc.z ^= v[j].z; acc.w ^= v[j].w; }
+  }
+  unsigned r = acc.x ^ acc.y ^ acc.z ^ acc.w;
+  for (int o = MS_WAVE / 2; o > 0; o >>= 1) r ^= __shfl_xor(r, o, MS_WAVE);
+  if ((threadIdx.x & (MS_WAVE - 1)) == 0) atomicXor(&sink[blockIdx.x], r);
+}
+
+// sink: unsigned [n_blocks], n_blocks = 8 blocks per compute unit (ms_read_probe_blocks).
+extern "C" int ms_read_probe_blocks() { return 8 * ms_compute_units(); }
+
+extern "C" int ms_read_probe(const void* base, long long bytes, unsigned* sink, hipStream_t stream) {
+  if (bytes <= 0) return MS_OK;
+  if (bytes % 16 || (uintptr_t)base % 16) return MS_BAD_ARG;
+  read_probe_kernel<<<dim3(ms_read_probe_blocks()), dim3(1024), 0, stream>>>((const uint4*)base, (size_t)bytes / 16, sink);
+  return ms_launch_status();
+}

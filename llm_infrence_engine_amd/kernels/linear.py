@@ -18,6 +18,21 @@ from . import ops
 
 _mm_out_dtype_ok = None  # whether torch.mm can write float from bfloat16 inputs (found out at first use)
 
+# Products that a few-rows kernel turned down (no block shape for the sizes) and that went to the vector-ALU
+# kernel instead: correct, slower.  (shape, epilogue) -> times.  Zero for every shape the kernels are tuned for.
+fallbacks = {}
+
+
+def _fell_back(M: int, N: int, K: int, what: str) -> None:
+    key = (M, N, K, what)
+    fallbacks[key] = fallbacks.get(key, 0) + 1
+    ops._say_once(("linear", N, K, what), f"no few-rows kernel for {what} of {M} x {K} by {N} x {K}; "
+                                          f"the vector-ALU kernel runs it")
+
+
+def fallback_count() -> int:
+    return sum(fallbacks.values())
+
 
 class LazyNorm:
     """Rows of the float residual stream that are still to be RMS-normalised.  The product that consumes them
@@ -70,12 +85,18 @@ def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None
     """[M, K] x [N, K] -> [M, N] in ``out_dtype`` (default: a's type).  ``a`` may be a ``LazyNorm``."""
     if isinstance(a, LazyNorm):
         if ops.skinny_norm_ok(a.x, w, a.num_rows):
-            return ops.gemm_skinny_norm(a.x, a.weight, a.eps, w, bias, ops.EPI_STORE, out_dtype or a.out_dtype, a.rows)
+            try:
+                return ops.gemm_skinny_norm(a.x, a.weight, a.eps, w, bias, ops.EPI_STORE, out_dtype or a.out_dtype, a.rows)
+            except ops.UnsupportedShape:
+                _fell_back(a.num_rows, w.shape[0], w.shape[1], "norm + product")
         a = a.materialize()
     out_dtype = out_dtype or a.dtype
     if a.dtype == torch.bfloat16:
         if ops.skinny_ok(a, w):
-            return ops.gemm_skinny(a, w, bias, ops.EPI_STORE, out_dtype=out_dtype)
+            try:
+                return ops.gemm_skinny(a, w, bias, ops.EPI_STORE, out_dtype=out_dtype)
+            except ops.UnsupportedShape:
+                _fell_back(a.shape[0], w.shape[0], w.shape[1], "product")
         if a.shape[0] > ops.SKINNY_MAX_ROWS and a.is_contiguous():
             out = _library_mm(a, w, out_dtype)
             if out is not None:
@@ -90,8 +111,13 @@ def linear_residual(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tenso
     ``residual`` itself (each element by one lane, no atomics) and None is returned; otherwise the product
     [M, N] is returned for the next norm to add."""
     if residual is not None and a.dtype == torch.bfloat16 and ops.skinny_ok(a, w):
-        ops.gemm_skinny(a, w, bias, ops.EPI_RESIDUAL, residual=residual)
-        return None
+        try:
+            ops.gemm_skinny(a, w, bias, ops.EPI_RESIDUAL, residual=residual)
+            return None
+        except ops.UnsupportedShape:
+            _fell_back(a.shape[0], w.shape[0], w.shape[1], "product + residual")
+            out = torch.empty((a.shape[0], w.shape[0]), dtype=a.dtype, device=a.device)
+            return ops.gemm_generic(a, w, out, bias=bias)
     return linear(a, w, bias)
 
 
@@ -100,10 +126,16 @@ def linear_swiglu(a: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
     ``LazyNorm``."""
     if isinstance(a, LazyNorm):
         if ops.skinny_norm_ok(a.x, w_gate_up, a.num_rows):
-            return ops.gemm_skinny_norm(a.x, a.weight, a.eps, w_gate_up, None, ops.EPI_SWIGLU, rows=a.rows)
+            try:
+                return ops.gemm_skinny_norm(a.x, a.weight, a.eps, w_gate_up, None, ops.EPI_SWIGLU, rows=a.rows)
+            except ops.UnsupportedShape:
+                _fell_back(a.num_rows, w_gate_up.shape[0], w_gate_up.shape[1], "norm + gated product")
         a = a.materialize()
     if a.dtype == torch.bfloat16 and ops.skinny_ok(a, w_gate_up):
-        return ops.gemm_skinny(a, w_gate_up, None, ops.EPI_SWIGLU)
+        try:
+            return ops.gemm_skinny(a, w_gate_up, None, ops.EPI_SWIGLU)
+        except ops.UnsupportedShape:
+            _fell_back(a.shape[0], w_gate_up.shape[0], w_gate_up.shape[1], "gated product")
     gu = linear(a, w_gate_up)
     act = torch.empty((a.shape[0], w_gate_up.shape[0] // 2), dtype=a.dtype, device=a.device)
     return ops.silu_mul(gu, act)

@@ -7,6 +7,7 @@ missing library, raises.
 from __future__ import annotations
 
 import ctypes
+import sys
 from typing import Optional
 
 import torch
@@ -37,6 +38,8 @@ _SIGNATURES = {
     "ms_gemm_panel_splitk_parts": [_c_int, _c_int, _c_int],
     "ms_gemm_panel_splitk": [_c_ptr, _c_ll, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int,
                              _c_ptr, _c_int, _c_ptr],
+    "ms_read_probe_blocks": [],
+    "ms_read_probe": [_c_ptr, _c_ll, _c_ptr, _c_ptr],
     "ms_residual_add": [_c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr],
     "ms_silu_mul": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "ms_rope_store": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int,
@@ -74,10 +77,26 @@ def _get(name):
     return f
 
 
+class UnsupportedShape(RuntimeError):
+    """A kernel has no variant for the sizes it was given (it launched nothing); another kernel may."""
+
+
 def _call(name, *args):
     rc = _get(name)(*args)
+    if rc == 2:
+        raise UnsupportedShape(f"{name} refused its arguments: unsupported size (it has no variant for these sizes)")
     if rc != 0:
         raise RuntimeError(f"{name} refused its arguments: {_CODES.get(rc, rc)}")
+
+
+_said = set()
+
+
+def _say_once(key, message: str) -> None:
+    """A notice on stderr, once per process and key: a slower kernel than one might expect is in use."""
+    if key not in _said:
+        _said.add(key)
+        print(f"[llm_infrence_engine_amd] {message}", file=sys.stderr, flush=True)
 
 
 def _stream():
@@ -179,6 +198,18 @@ def decode_advance(prev_tokens: torch.Tensor, token_ids: torch.Tensor, positions
     _call("ms_decode_advance", prev_tokens.data_ptr(), token_ids.data_ptr(), positions.data_ptr(),
           context_lens.data_ptr(), n_live.data_ptr(), ctypes.cast(tp, ctypes.c_void_p), ctypes.cast(sp, ctypes.c_void_p),
           len(tables), width, page_size, R, _stream())
+
+
+def read_probe(t: torch.Tensor) -> torch.Tensor:
+    """Stream ``t`` once from memory with a kernel that does nothing else (for bandwidth measurements).
+    Returns the exclusive-or of its 32-bit words per block."""
+    _check(t, "t")
+    nbytes = t.numel() * t.element_size()
+    if nbytes % 16:
+        raise ValueError("the probe reads multiples of 16 bytes")
+    sink = torch.zeros(_get("ms_read_probe_blocks")(), dtype=torch.int32, device=t.device)
+    _call("ms_read_probe", t.data_ptr(), nbytes, sink.data_ptr(), _stream())
+    return sink
 
 
 def residual_add(x: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
@@ -565,6 +596,10 @@ def paged_attention(q: torch.Tensor, kv, ctx, out: torch.Tensor, num_heads: int,
     bfloat16 with transposed value pages and a head size the matrix-core kernel has goes there; everything
     else (float32, other head sizes, small pages) goes to the generic kernel."""
     d, page_size = kv.k_pages.shape[3], kv.k_pages.shape[2]
+    if q.dtype == torch.bfloat16 and not (kv.v_transposed and attention_mfma_supported(d, page_size)):
+        _say_once(("attention", d, page_size),
+                  f"bfloat16 attention with head size {d} and pages of {page_size} tokens runs on the vector-ALU kernel: "
+                  f"the matrix-core kernel takes head sizes 32, 64 and 128 with pages of a multiple of 16")
     if (q.dtype == torch.bfloat16 and kv.v_transposed and attention_mfma_supported(d, page_size)
             and q.data_ptr() % 16 == 0 and (q.shape[0] == 1 or q.stride(0) % 8 == 0)):
         return paged_attention_mfma(q, kv.k_pages, kv.v_pages, kv.block_table, ctx.q_start, ctx.context_lens, out,

@@ -814,3 +814,79 @@ def test_qkv_rope_store_fused_equals_the_separate_kernels(ops, M, nh, nkv, d, K,
     untouched = torch.ones(pages * page_size, dtype=torch.bool)
     untouched[slots[slots >= 0].long().cpu()] = False
     assert (kp1.permute(0, 2, 1, 3).reshape(pages * page_size, -1)[untouched.to(DEV)] == 0).all()
+
+
+# the products of a decode step at the shapes of the published checkpoints: (rows of W, columns) of the packed
+# q/k/v, o, interleaved gate/up, down and head matrices
+MODEL_PRODUCTS = {
+    "0.5b": [(1152, 896), (896, 896), (9728, 896), (896, 4864), (151936, 896)],
+    "7b": [(4608, 3584), (3584, 3584), (37888, 3584), (3584, 18944), (152064, 3584)],
+    "32b": [(7168, 5120), (5120, 5120), (55296, 5120), (5120, 27648)],
+}
+
+
+@pytest.mark.parametrize("shape", sorted(MODEL_PRODUCTS))
+def test_every_row_count_of_the_model_products_has_a_kernel(ops, shape):
+    """1 to 64 rows against every product of the three model shapes, through ``kernels.linear`` as the parts call it:
+    right against a double-precision product, and never by falling back to the vector-ALU kernel."""
+    from llm_infrence_engine_amd.kernels import linear
+
+    g = torch.Generator(device=DEV).manual_seed(len(shape))
+    before = linear.fallback_count()
+    for N, K in MODEL_PRODUCTS[shape]:
+        w = (torch.randn(N, K, generator=g, device=DEV) / math.sqrt(K)).bfloat16()
+        a = torch.randn(64, K, generator=g, device=DEV).bfloat16()
+        want = a.double() @ w.double().T                                    # rows are independent: one reference for all M
+        x = torch.randn(64, N, generator=g, device=DEV) if N < 100000 else None
+        rows = (range(1, 65) if N < 100000 else (1, 2, 7, 8, 9, 16, 17, 31, 32, 33, 48, 63, 64))
+        for M in rows:
+            got = linear.linear(a[:M], w, out_dtype=torch.float32)
+            err = (got.double() - want[:M]).abs().max().item()
+            assert err < 5e-5 * max(1.0, want[:M].abs().max().item()) + 2e-5, (shape, "store", M, N, K, err)
+            if x is not None:
+                r = x[:M].clone()
+                assert linear.linear_residual(a[:M], w, None, r) is None
+                err = (r.double() - x[:M].double() - want[:M]).abs().max().item()
+                assert err < 1e-4, (shape, "residual", M, N, K, err)
+            if N % 2 == 0 and N > K and x is not None:                      # the gated product of gate/up
+                act = linear.linear_swiglu(a[:M], w)
+                ref = torch.nn.functional.silu(want[:M, 0::2]) * want[:M, 1::2]
+                assert (act.double() - ref).abs().max().item() < 0.02 * max(1.0, ref.abs().max().item()), (shape, "gated", M, N, K)
+        del w, a, want
+    assert linear.fallback_count() == before, linear.fallbacks
+
+
+def test_random_product_shapes_are_right_whatever_kernel_takes_them(ops):
+    """A few hundred random shapes of up to 64 rows: ``kernels.linear`` finds a kernel for each (falling back to the
+    vector-ALU kernel where the few-rows kernels have no variant, which is counted, not an error)."""
+    from llm_infrence_engine_amd.kernels import linear
+
+    rng = np.random.default_rng(17)
+    g = torch.Generator(device=DEV).manual_seed(17)
+    for case in range(300):
+        M = int(rng.integers(1, 65))
+        N = int(rng.choice([rng.integers(1, 64), rng.integers(64, 5000), rng.integers(5000, 40000)]))
+        K = int(rng.choice([rng.integers(1, 40), rng.integers(40, 2000), rng.integers(2000, 12000)]))
+        if rng.random() < 0.7:
+            K = max(8, K // 8 * 8)
+        a = torch.randn(M, K, generator=g, device=DEV).bfloat16()
+        w = (torch.randn(N, K, generator=g, device=DEV) / math.sqrt(K)).bfloat16()
+        b = torch.randn(N, generator=g, device=DEV) if rng.random() < 0.5 else None
+        want = a.double() @ w.double().T + (b.double() if b is not None else 0.0)
+        got = linear.linear(a, w, b, out_dtype=torch.float32)
+        err = (got.double() - want).abs().max().item()
+        assert err < 5e-5 * max(1.0, want.abs().max().item()) + 2e-5, (case, M, N, K, err)
+        x = torch.randn(M, N, generator=g, device=DEV)
+        r = x.clone()
+        d = linear.linear_residual(a, w, b, r)
+        total = r.double() if d is None else x.double() + d.double()
+        assert (total - x.double() - want).abs().max().item() < (1e-4 if d is None else 0.05), (case, M, N, K)
+
+
+def test_read_probe_reads_everything_once(ops):
+    t = torch.randint(-2 ** 31, 2 ** 31 - 1, (1 << 20,), dtype=torch.int32, device=DEV)
+    for n in (1 << 20, 4 * 1000, 4):
+        got = np.bitwise_xor.reduce(ops.read_probe(t[:n]).cpu().numpy().view(np.uint32))
+        assert got == np.bitwise_xor.reduce(t[:n].cpu().numpy().view(np.uint32))
+    with pytest.raises(ValueError, match="16 bytes"):
+        ops.read_probe(t[:3])
