@@ -26,9 +26,13 @@ from .allocator import NULL_PAGE, OutOfPages, PageAllocator
 
 @dataclass(frozen=True)
 class GroupKey:
-    num_kv_heads: int
-    head_dim: int
+    """What the pages of a group hold (a tuple of ``parts.base.PageTensor``) and for how long."""
+
+    tensors: tuple
     window: Optional[int]
+
+    def values_per_token(self) -> int:
+        return sum(t.heads * t.width for t in self.tensors)
 
 
 @dataclass
@@ -63,15 +67,15 @@ class CacheLayout:
                 if kv is None:
                     raise ValueError(f"run {i} reads the cache of run {cache_of} but its mixer keeps no keys and values")
                 src_kv = run_needs[cache_of][0]
-                if src_kv is None or (src_kv.num_kv_heads, src_kv.head_dim) != (kv.num_kv_heads, kv.head_dim):
-                    raise ValueError(f"run {i} cannot read the cache of run {cache_of}: their key/value shapes differ")
+                if src_kv is None or src_kv.tensors != kv.tensors:
+                    raise ValueError(f"run {i} cannot read the cache of run {cache_of}: their pages hold different tensors")
                 if src_kv.window is not None and (kv.window is None or kv.window > src_kv.window):
                     raise ValueError(f"run {i} looks further back than run {cache_of}, whose cache it reads, keeps keys")
                 self.run_group.append(self.run_group[cache_of])
                 self.run_entry.append(self.run_entry[cache_of])
                 self.run_stores.append(False)
             elif kv is not None:
-                key = GroupKey(kv.num_kv_heads, kv.head_dim, kv.window)
+                key = GroupKey(tuple(kv.tensors), kv.window)
                 if key not in self.group_keys:
                     self.group_keys.append(key)
                     self.group_runs.append([])
@@ -86,13 +90,13 @@ class CacheLayout:
                 self.run_stores.append(False)
             if state is not None:
                 self.state_runs.append(i)
-                self.state_needs[i] = state
+                self.state_needs[i] = tuple(state) if isinstance(state, (tuple, list)) else state
 
 
     def bytes_per_token(self, bytes_per_value: int) -> int:
-        """Stored bytes per token over all runs that keep keys and values
-        (layers x 2 x kv heads x head size x bytes, src/miniserve/cache.py:27-29)."""
-        return sum(len(runs) * 2 * key.num_kv_heads * key.head_dim * bytes_per_value
+        """Stored bytes per token over all runs that keep a cache (for keys and values: layers x 2 x kv heads
+        x head size x bytes, src/miniserve/cache.py:27-29)."""
+        return sum(len(runs) * key.values_per_token() * bytes_per_value
                    for key, runs in zip(self.group_keys, self.group_runs))
 
 

@@ -15,7 +15,7 @@ import math
 from dataclasses import asdict, dataclass
 
 from .registry import ConfigError, register_architecture, require
-from .spec import LayerSpec, ModelSpec, PartSpec, Run
+from .spec import ModelSpec, PartSpec, Run, layer
 
 
 @dataclass(frozen=True)
@@ -102,8 +102,8 @@ class Qwen2Config:
         layers = []
         for i in range(self.num_hidden_layers):
             p = f"model.layers.{i}."
-            layers.append(LayerSpec(
-                block="pre_norm_residual",
+            layers.append(layer(
+                "pre_norm_residual",
                 mixer=PartSpec("gqa_attention", p + "self_attn.", {
                     "hidden_size": H, "num_heads": self.num_attention_heads,
                     "num_kv_heads": self.num_key_value_heads, "head_dim": self.head_dim,

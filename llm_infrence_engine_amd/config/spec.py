@@ -23,15 +23,23 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """One layer: which arrangement (``block``) puts which mixer and feed-forward behind which
-    norms.  The position encoding belongs to the mixer (``position`` may be None)."""
+    """One layer: an arrangement (``block``, a name in the block registry) and the parts it is given, by the
+    names the arrangement takes.  ``pre_norm_residual`` takes ``mixer``, ``feed_forward``, ``mixer_norm``,
+    ``feed_forward_norm`` and optionally ``position`` (the mixer's position encoding); another arrangement
+    may take other parts (more norms, no feed-forward, two mixers)."""
 
     block: str
-    mixer: PartSpec
-    feed_forward: PartSpec
-    mixer_norm: PartSpec
-    feed_forward_norm: PartSpec
-    position: Optional[PartSpec] = None
+    parts: Mapping[str, PartSpec]
+
+    def __getattr__(self, name):      # layer.mixer, layer.position, ...: the named part, None if it has none
+        if name.startswith("__") or name in ("block", "parts"):
+            raise AttributeError(name)
+        return self.parts.get(name)
+
+
+def layer(block: str, **parts: Optional[PartSpec]) -> LayerSpec:
+    """``LayerSpec`` from keyword parts; a part given as None is left out."""
+    return LayerSpec(block, {k: v for k, v in parts.items() if v is not None})
 
 
 @dataclass(frozen=True)

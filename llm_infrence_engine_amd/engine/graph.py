@@ -40,8 +40,8 @@ def default_batch_sizes(max_batch: int) -> List[int]:
 
 
 class _Bucket:
-    def __init__(self, B: int, width: int, n_groups: int, device, steps: int = 1):
-        self.B, self.width, self.steps = B, width, steps
+    def __init__(self, B: int, width: int, n_groups: int, device, steps: int = 1, null_state_slot: int = 0):
+        self.B, self.width, self.steps, self.null_state_slot = B, width, steps, null_state_slot
         # layout of the static int32 buffer
         self.off: Dict[str, slice] = {}
         o = 0
@@ -74,6 +74,7 @@ class _Bucket:
         a[self.off["context_lens"]] = 1
         a[self.off["logit_rows"]] = np.arange(B)
         a[self.off["n_live"]] = 0
+        a[self.off["state_slots"]] = self.null_state_slot      # nobody's slot
         for s in self.slots:
             a[s] = -1
 
@@ -84,14 +85,15 @@ class _Bucket:
             token_req=d[o["token_req"]], q_start=d[o["q_start"]], context_lens=d[o["context_lens"]],
             state_slots=d[o["state_slots"]], logit_rows=d[o["logit_rows"]], max_q_len=1,
             max_context_len=self.width, q_lens_host=[1] * self.B, start_pos_host=[0] * self.B,
-            state_slots_host=[0] * self.B)
+            state_slots_host=[self.null_state_slot] * self.B)
 
 
 class DecodeGraphs:
     def __init__(self, runner, batch_sizes: Optional[Sequence[int]] = None):
         m = runner.manager
-        if runner.layout.state_runs:
-            raise ValueError("HIP graphs are not used for models whose mixers keep per-request state on the host side")
+        if not runner.model.graph_safe():
+            raise ValueError("HIP graphs are not used for this model: one of its parts says it cannot be captured "
+                             "(Part.graph_safe)")
         self.runner, self.manager = runner, m
         self.sizes = sorted(set(batch_sizes or default_batch_sizes(m.max_requests)))
         self.width = m.max_pages_per_request
@@ -128,7 +130,8 @@ class DecodeGraphs:
         key = (B, long_context, steps)
         bk = self.buckets.get(key)
         if bk is None:
-            bk = self.buckets[key] = _Bucket(B, self.width, len(self.manager.groups), self.runner.rt.device, steps)
+            bk = self.buckets[key] = _Bucket(B, self.width, len(self.manager.groups), self.runner.rt.device, steps,
+                                             self.runner.pools.null_state_slot)
             self._capture(bk, long_context)
         return bk
 
@@ -140,7 +143,8 @@ class DecodeGraphs:
             kv = None
             if g is not None:
                 kv = r.pools.kv_view(i, bk.dev[bk.tables[g]].view(bk.B, bk.width), bk.dev[bk.slots[g]])
-            caches.append(RunCache(kv, None))
+            state = r.pools.state_view(i) if i in r.layout.state_needs else None
+            caches.append(RunCache(kv, state))
         return caches
 
     def _capture(self, bk: _Bucket, long_context: bool) -> None:
@@ -210,6 +214,8 @@ class DecodeGraphs:
         if R < bk.last_rows:
             bk.reset_host()
         bk.last_rows = R
+        if self.runner.layout.state_runs and (pos == 0).any():
+            self.runner.pools.zero_state([int(r) for r in rows[pos == 0]])      # a first token starts from zero state
         a[o["token_ids"]][:R] = toks
         a[o["positions"]][:R] = pos
         a[o["context_lens"]][:R] = pos + 1

@@ -28,7 +28,9 @@ class ModelRunner:
         self.pools = CachePools(self.layout, page_size, num_pages, max_requests, self.rt)
         self.builder = BatchBuilder(self.manager, model.spec.vocab_size, self.rt.device)
         self.graphs = None
-        if hip_graphs and not self.layout.state_runs:
+        # a part that cannot be captured (it walks the requests on the host, as a mixer with state usually does)
+        # keeps the whole model out of graphs
+        if hip_graphs and model.graph_safe():
             from .graph import DecodeGraphs
 
             self.graphs = DecodeGraphs(self)

@@ -61,7 +61,11 @@ class GQAttention(Mixer):
 
     # ---- cache
     def cache_need(self):
-        return KVNeed(self.num_kv_heads, self.head_dim, self.window)
+        # in bfloat16 the matrix-core attention reads value pages as an operand as they lie, transposed, which it
+        # can for pages of a multiple of 16 tokens
+        rt = getattr(self, "rt", None)
+        at = 16 if rt is not None and rt.dtype == torch.bfloat16 else None
+        return KVNeed(self.num_kv_heads, self.head_dim, self.window, transpose_values_at=at)
 
     # ---- step
     def forward(self, h, ctx, kv, state):

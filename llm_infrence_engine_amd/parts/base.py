@@ -9,7 +9,7 @@ it is in.  Five kinds are chosen layer by layer:
 ``FeedForward``       forward(h, ctx) -> [N, hidden]
                       (both also forward_residual(..., x): add into the residual stream x and return None,
                       or return the addend; the default returns forward's result)
-``Block``             forward(x, pending, ctx, kv, state) -> pending             (the arrangement of the four)
+``Block``             forward(x, pending, ctx, kv, state) -> pending             (the arrangement; it names the parts it takes)
 
 plus ``Embedding`` and ``Head`` at the model's ends.  Every part lists the checkpoint tensors it wants
 (``tensor_specs``) and takes them in ``load``.
@@ -37,19 +37,48 @@ class Runtime:
 
 
 @dataclass(frozen=True)
-class KVNeed:
-    """A mixer that keeps keys and values: pages of [num_kv_heads, page_size, head_dim], all keys of a
-    request (``window`` None) or the last ``window`` of them."""
+class PageTensor:
+    """One tensor of a cache page: ``heads`` x ``width`` values per token, kept as [heads, page_size, width].
+    With ``transpose_at`` = n the pool keeps it as [heads, width, page_size] instead whenever the page size is
+    a multiple of n (a mixer asks for that when its kernels read the tensor as a matrix operand as it lies)."""
 
-    num_kv_heads: int
-    head_dim: int
+    name: str
+    heads: int
+    width: int
+    transpose_at: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class CacheNeed:
+    """What a mixer keeps per token in pages: one or more tensors, for all tokens of a request (``window``
+    None) or the last ``window`` of them.  Runs with equal needs share a group of the cache manager."""
+
+    tensors: Tuple[PageTensor, ...]
     window: Optional[int] = None
+
+    def __post_init__(self):
+        names = [t.name for t in self.tensors]
+        if not names or len(set(names)) != len(names):
+            raise ValueError("a cache need names at least one page tensor, each name once")
+        if self.window is not None and self.window <= 0:
+            raise ValueError("window must be positive")
+
+    def values_per_token(self) -> int:
+        return sum(t.heads * t.width for t in self.tensors)
+
+
+def KVNeed(num_kv_heads: int, head_dim: int, window: Optional[int] = None,
+           transpose_values_at: Optional[int] = None) -> CacheNeed:
+    """The usual need of attention: keys "k" and values "v", [num_kv_heads, head_dim] each."""
+    return CacheNeed((PageTensor("k", num_kv_heads, head_dim), PageTensor("v", num_kv_heads, head_dim, transpose_values_at)),
+                     window)
 
 
 @dataclass(frozen=True)
 class StateNeed:
-    """A mixer that keeps state of fixed size per request: one tensor of ``shape`` and ``dtype`` in a slot
-    that the request holds from admission to its end.  The slot is zero when the request's first portion runs."""
+    """State of fixed size per request: one tensor of ``shape`` and ``dtype`` in a slot that the request holds
+    from admission to its end.  The slot is zero when the request's first portion runs.  A mixer that keeps
+    several such tensors returns a tuple of these."""
 
     shape: Tuple[int, ...]
     dtype: torch.dtype = torch.float32
@@ -59,20 +88,34 @@ class StateNeed:
 class KVView:
     """One run's pages of its cache group, with the group's tables for the step's requests."""
 
-    k_pages: torch.Tensor      # [pages, nkv, page_size, d]
-    v_pages: torch.Tensor      # the same, or [pages, nkv, d, page_size] if v_transposed
-    block_table: torch.Tensor  # int32 [R, max pages]
-    slot_mapping: torch.Tensor  # int32 [N]: page * page_size + offset of each token
-    store: bool = True         # False: the run reads another run's cache and writes nothing
+    pages: Dict[str, torch.Tensor]       # name -> [pages, heads, page_size, width], or [pages, heads, width, page_size]
+    transposed: Dict[str, bool]          # name -> which of the two
+    block_table: torch.Tensor            # int32 [R, max pages]
+    slot_mapping: torch.Tensor           # int32 [N]: page * page_size + offset of each token
+    store: bool = True                   # False: the run reads another run's cache and writes nothing
     window: Optional[int] = None
-    v_transposed: bool = False
+
+    # the usual pair of attention
+    @property
+    def k_pages(self) -> torch.Tensor:
+        return self.pages["k"]
+
+    @property
+    def v_pages(self) -> torch.Tensor:
+        return self.pages["v"]
+
+    @property
+    def v_transposed(self) -> bool:
+        return self.transposed["v"]
 
 
 @dataclass
 class StateView:
-    """One run's state slots: ``slots[state_slots[r]]`` belongs to request row r of the step."""
+    """One run's state slots: ``slots[state_slots[r]]`` belongs to request row r of the step.  ``slots`` is one
+    tensor [num_slots, *shape], or a tuple of them when the mixer asked for several; the last slot is nobody's
+    (rows that pad a batch point there)."""
 
-    slots: torch.Tensor        # [num_slots, *shape]
+    slots: object
 
 
 @dataclass
@@ -107,6 +150,12 @@ Getter = Callable[[TensorSpec], torch.Tensor]
 
 
 class Part:
+    # Whether a decode step that runs this part may be captured into a graph and replayed: the part reads the
+    # step's batch from the device tensors of its StepContext only (never from the host copies), does not wait
+    # for the device and launches the same work whatever those tensors hold.  A model with a part that says
+    # False steps without graphs.
+    graph_safe = True
+
     def tensor_specs(self) -> List[TensorSpec]:
         return []
 
@@ -148,10 +197,17 @@ class PositionEncoding(Part):
 class Mixer(Part):
     accepts_lazy_norm = False   # True: h may be a LazyNorm that the part hands to kernels.linear
 
-    def cache_need(self) -> Optional[KVNeed]:
+    @property
+    def graph_safe(self) -> bool:
+        """A mixer with per-request state is taken to walk its requests on the host unless its class says
+        ``graph_safe = True``."""
+        return self.state_need() is None
+
+    def cache_need(self) -> Optional[CacheNeed]:
         return None
 
-    def state_need(self) -> Optional[StateNeed]:
+    def state_need(self):
+        """None, a ``StateNeed``, or a tuple of them."""
         return None
 
     def forward(self, h: torch.Tensor, ctx: StepContext, kv: Optional[KVView],
@@ -177,15 +233,75 @@ class FeedForward(Part):
 
 
 class Block(Part):
-    """The arrangement of a layer's parts.  ``pending`` is an addend of the residual stream that the
+    """The arrangement of a layer's parts.  A block class names the parts it takes and their categories in
+    ``takes`` (in the order their tensors are listed); ``LayerSpec.parts`` gives a ``PartSpec`` for each by
+    name, those in ``optional`` may be missing.  A position encoding belongs to the mixer that is built after
+    it (the mixer lists and loads its tensors).  ``pending`` is an addend of the residual stream that the
     previous layer left unsummed so that the next norm can fuse the sum; a block returns its own."""
 
-    def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm, feed_forward_norm: Norm):
-        self.mixer, self.feed_forward = mixer, feed_forward
-        self.mixer_norm, self.feed_forward_norm = mixer_norm, feed_forward_norm
+    takes: Dict[str, str] = {}
+    optional: Tuple[str, ...] = ()
+
+    def __init__(self, **built):
+        unknown = set(built) - set(self.takes)
+        if unknown:
+            raise TypeError(f"{type(self).__name__} takes {sorted(self.takes)}, not {sorted(unknown)}")
+        self.built: Dict[str, Optional[Part]] = {}
+        for name in self.takes:
+            part = built.get(name)
+            if part is None and name not in self.optional:
+                raise TypeError(f"{type(self).__name__} needs a part named {name!r}")
+            self.built[name] = part
+            setattr(self, name, part)
+
+    @classmethod
+    def build(cls, specs) -> "Block":
+        """Build every named part from its ``PartSpec`` and put them together."""
+        unknown = set(specs) - set(cls.takes)
+        if unknown:
+            raise KeyError(f"the {cls.__name__} arrangement takes the parts {sorted(cls.takes)}; it has no {sorted(unknown)}")
+        built: Dict[str, Optional[Part]] = {}
+        position = None
+        for name, category in cls.takes.items():
+            spec = specs.get(name)
+            if spec is None:
+                if name not in cls.optional:
+                    raise KeyError(f"the {cls.__name__} arrangement needs a part named {name!r}")
+                built[name] = None
+                continue
+            extra = {"position": position} if category == "mixer" else {}
+            built[name] = build_part(category, spec, **extra)
+            if category == "position":
+                position = built[name]
+            elif category == "mixer":
+                position = None
+        return cls(**built)
 
     def parts(self) -> List[Part]:
-        return [self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward]
+        """The parts whose tensors the block lists and loads itself (position encodings go with their mixers)."""
+        return [p for name, p in self.built.items() if p is not None and self.takes[name] != "position"]
+
+    def mixers(self) -> List[Mixer]:
+        return [p for p in self.built.values() if isinstance(p, Mixer)]
+
+    def cache_need(self) -> Optional[CacheNeed]:
+        needs = [n for n in (m.cache_need() for m in self.mixers()) if n is not None]
+        if len(needs) > 1:
+            raise ValueError("a run of a layer has one cache; a block with two caching mixers must merge their needs itself")
+        return needs[0] if needs else None
+
+    def state_need(self):
+        needs = []
+        for m in self.mixers():
+            n = m.state_need()
+            if n is not None:
+                needs.extend(n if isinstance(n, (tuple, list)) else [n])
+        if not needs:
+            return None
+        return needs[0] if len(needs) == 1 else tuple(needs)
+
+    def graph_safe(self) -> bool:
+        return all(p.graph_safe for p in self.built.values() if p is not None)
 
     def tensor_specs(self) -> List[TensorSpec]:
         return [s for p in self.parts() for s in p.tensor_specs()]

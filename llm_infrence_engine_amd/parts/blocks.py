@@ -10,6 +10,10 @@ from .base import Block, register_part
 
 
 class PreNormResidual(Block):
+    takes = {"position": "position", "mixer_norm": "norm", "mixer": "mixer", "feed_forward_norm": "norm",
+             "feed_forward": "feed_forward"}
+    optional = ("position",)
+
     def forward(self, x, pending, ctx, kv, state):
         norm = self.mixer_norm.lazy if self.mixer.accepts_lazy_norm else self.mixer_norm.forward
         a = self.mixer.forward_residual(norm(x, delta=pending), ctx, kv, state, x)

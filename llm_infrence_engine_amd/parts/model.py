@@ -31,12 +31,7 @@ class Model:
         self.embedding = build_part("embedding", spec.embedding)
         self.layers = []
         for ls in spec.layers:
-            position = build_part("position", ls.position) if ls.position is not None else None
-            mixer = build_part("mixer", ls.mixer, position=position)
-            ff = build_part("feed_forward", ls.feed_forward)
-            n1 = build_part("norm", ls.mixer_norm)
-            n2 = build_part("norm", ls.feed_forward_norm)
-            self.layers.append(part_class("block", ls.block)(mixer, ff, n1, n2))
+            self.layers.append(part_class("block", ls.block).build(ls.parts))
         self.final_norm = build_part("norm", spec.final_norm)
         self.head = build_part("head", spec.head)
         self.rt: Optional[Runtime] = None
@@ -75,12 +70,14 @@ class Model:
 
     # ------------------------------------------------------------------ cache needs, run by run
     def run_needs(self):
-        """For every entry of the order: (KVNeed or None, StateNeed or None, cache_of)."""
-        out = []
-        for run in self.spec.order:
-            mixer = self.layers[run.layer].mixer
-            out.append((mixer.cache_need(), mixer.state_need(), run.cache_of))
-        return out
+        """For every entry of the order: (CacheNeed or None, StateNeed(s) or None, cache_of)."""
+        return [(self.layers[run.layer].cache_need(), self.layers[run.layer].state_need(), run.cache_of)
+                for run in self.spec.order]
+
+    def graph_safe(self) -> bool:
+        """Whether a decode step of this model may be captured into a graph (see ``Part.graph_safe``)."""
+        return (all(b.graph_safe() for b in self.layers)
+                and all(p.graph_safe for p in (self.embedding, self.final_norm, self.head)))
 
     # ------------------------------------------------------------------ one step
     def forward(self, ctx: StepContext, caches: List[RunCache]) -> torch.Tensor:

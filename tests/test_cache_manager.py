@@ -60,7 +60,7 @@ def test_layout_groups_runs_by_their_needs():
     assert lay.run_group == [0, 1, 0, 0, None, 2] and lay.run_entry == [0, 0, 1, 0, None, 0]
     assert lay.run_stores == [True, True, True, False, False, True]
     assert lay.state_runs == [4]
-    with pytest.raises(ValueError, match="shapes differ"):
+    with pytest.raises(ValueError, match="hold different tensors"):
         CacheLayout([full(), (KVNeed(4, 16), None, 0)])
     with pytest.raises(ValueError, match="further back"):
         CacheLayout([full(window=8), (KVNeed(2, 16), None, 0)])

@@ -116,7 +116,8 @@ def test_attention_part_in_portions(fw, nh, nkv, d, window, page_size):
     layout = fw.cache.CacheLayout([(part.cache_need(), None, None)])
     m = fw.cache.CacheManager(layout, page_size, 20, 2, 64)
     pools = fw.cache.CachePools(layout, page_size, 20, 2, rt)
-    pools.kv[0].fill_(1e4)                                   # what a reused page may hold must not matter
+    for t in pools.pages[0].values():
+        t.fill_(1e4)                                         # what a reused page may hold must not matter
     builder = fw.engine.BatchBuilder(m, 1000, rt.device)
     m.add("x")
     got, p = [], 0
@@ -137,7 +138,11 @@ def register_toys(fw):
     TensorSpec = fw.weights.TensorSpec
 
     class ToyDecay(parts.Mixer):
-        """state <- decay * state + W_in h_t ;  out_t = W_out state   (state of fixed size per request)"""
+        """state <- decay * state + W_in h_t ; seen <- seen + 1 ; out_t = W_out state / (1 + seen / 100)
+        Two states of fixed size per request, of different types.  Single tokens are handled with device tensors
+        only, so a decode step of this mixer can be captured into a graph."""
+
+        graph_safe = True
 
         def __init__(self, prefix, position, hidden_size, state_size, decay):
             self.prefix, self.H, self.S, self.decay = prefix, hidden_size, state_size, decay
@@ -147,27 +152,80 @@ def register_toys(fw):
 
         def load(self, get, rt):
             self.rt = rt
-            self.w_in, self.w_out = (get(s).float() for s in self.tensor_specs())
+            self.w_in, self.w_out = (get(s).float().contiguous() for s in self.tensor_specs())
 
         def state_need(self):
-            return parts.StateNeed((self.S,), torch.float32)
+            return (parts.StateNeed((self.S,), torch.float32), parts.StateNeed((), torch.int32))
 
         def forward(self, h, ctx, kv, state):
             assert kv is None
-            hin = h.float() @ self.w_in.T
+            s_all, seen_all = state.slots
+            hin = ops.gemm_generic(h.float().contiguous(), self.w_in, torch.empty(h.shape[0], self.S, device=h.device))
+            if ctx.decode_only:                       # one token per request: no look at the host copies
+                idx = ctx.state_slots.long()
+                s = self.decay * s_all.index_select(0, idx) + hin
+                seen = seen_all.index_select(0, idx) + 1
+                s_all.index_copy_(0, idx, s)
+                seen_all.index_copy_(0, idx, seen)
+                out = ops.gemm_generic(s, self.w_out, torch.empty(h.shape[0], self.H, device=h.device))
+                return (out / (1 + seen.float() / 100)[:, None]).to(h.dtype)
             out = torch.empty_like(h)
             o = 0
             for n, slot in zip(ctx.q_lens_host, ctx.state_slots_host):
-                s = state.slots[slot].clone()
+                s, seen = s_all[slot].clone(), int(seen_all[slot])
                 for t in range(n):
                     s = self.decay * s + hin[o + t]
-                    out[o + t] = (self.w_out @ s).to(h.dtype)
-                state.slots[slot] = s
+                    seen += 1
+                    out[o + t] = ((self.w_out @ s) / (1 + seen / 100)).to(h.dtype)
+                s_all[slot] = s
+                seen_all[slot] = seen
                 o += n
             return out
 
+    class ToyLatent(parts.Mixer):
+        """One head of attention over a cache that holds one tensor per token: the latent c_t = W_c h_t, from which
+        keys W_k c and values W_v c are made when they are read."""
+
+        graph_safe = False      # walks the requests on the host
+
+        def __init__(self, prefix, position, hidden_size, latent_size, key_size):
+            self.prefix, self.H, self.r, self.dk = prefix, hidden_size, latent_size, key_size
+
+        def tensor_specs(self):
+            p = self.prefix
+            return [TensorSpec(p + "c.weight", (self.r, self.H)), TensorSpec(p + "q.weight", (self.dk, self.H)),
+                    TensorSpec(p + "k.weight", (self.dk, self.r)), TensorSpec(p + "v.weight", (self.H, self.r))]
+
+        def load(self, get, rt):
+            self.rt = rt
+            self.wc, self.wq, self.wk, self.wv = (get(s).float() for s in self.tensor_specs())
+
+        def cache_need(self):
+            return parts.CacheNeed((parts.PageTensor("latent", 1, self.r),), None)
+
+        def forward(self, h, ctx, kv, state):
+            x = h.float()
+            pages = kv.pages["latent"]                                # [pages, 1, page_size, r]
+            flat = pages.view(-1, self.r)
+            flat[kv.slot_mapping.long()] = (x @ self.wc.T).to(flat.dtype)
+            q = x @ self.wq.T
+            out = torch.empty_like(x)
+            o = 0
+            for r, (n, start) in enumerate(zip(ctx.q_lens_host, ctx.start_pos_host)):
+                held = -(-(start + n) // pages.shape[2])
+                c = pages[kv.block_table[r, :held].long()].reshape(-1, self.r)[:start + n].float()
+                scores = (q[o:o + n] @ (c @ self.wk.T).T) / math.sqrt(self.dk)
+                j = torch.arange(start + n, device=x.device)[None, :]
+                i = torch.arange(start, start + n, device=x.device)[:, None]
+                scores = scores.masked_fill(j > i, float("-inf"))
+                out[o:o + n] = scores.softmax(-1) @ (c @ self.wv.T)
+                o += n
+            return out.to(h.dtype)
+
     class ToyRouted(parts.FeedForward):
         """router logits in float -> softmax -> the best expert alone, weighted by its probability"""
+
+        graph_safe = False      # waits for the device to learn which experts have rows
 
         def __init__(self, prefix, hidden_size, intermediate_size, num_experts):
             self.prefix, self.H, self.I, self.E = prefix, hidden_size, intermediate_size, num_experts
@@ -212,6 +270,20 @@ def register_toys(fw):
             if kv is not None and kv.store:
                 ops.rope_store(qkv, nh, nkv, d, 0, None, None, kv.slot_mapping, kv.k_pages, kv.v_pages, kv.v_transposed)
 
+    class ToySandwich(parts.Block):
+        """Four norms to a layer: x += post_a(mixer(pre_a(x))); x += post_f(feed_forward(pre_f(x)))."""
+
+        takes = {"pre_mixer_norm": "norm", "mixer": "mixer", "post_mixer_norm": "norm", "pre_ff_norm": "norm",
+                 "feed_forward": "feed_forward", "post_ff_norm": "norm"}
+
+        def forward(self, x, pending, ctx, kv, state):
+            if pending is not None:
+                ops.residual_add(x, pending)
+            a = self.mixer.forward(self.pre_mixer_norm.forward(x), ctx, kv, state)
+            ops.residual_add(x, self.post_mixer_norm.forward(a.float().contiguous()))
+            f = self.feed_forward.forward(self.pre_ff_norm.forward(x), ctx)
+            return self.post_ff_norm.forward(f.float().contiguous())       # the next norm adds it
+
     @dataclass(frozen=True)
     class ToyConfig:
         vocab_size: int
@@ -225,6 +297,8 @@ def register_toys(fw):
         decay: float
         window: int
         eps: float
+        latent: int = 12
+        capturable: bool = False     # only parts that a graph can hold: attention, the decaying state, dense feed-forwards
 
         @classmethod
         def from_dict(cls, d):
@@ -237,7 +311,7 @@ def register_toys(fw):
 
         def to_spec(self):
             H, d = self.width, self.head_size
-            PartSpec, LayerSpec, Run = cfgm.PartSpec, cfgm.LayerSpec, cfgm.Run
+            PartSpec, layer, Run = cfgm.PartSpec, cfgm.layer, cfgm.Run
             norm = lambda p: PartSpec("rms_norm", p, {"size": H, "eps": self.eps})
 
             def attn(p, window, position):
@@ -247,25 +321,37 @@ def register_toys(fw):
             rotary = PartSpec("rotary_half", "", {"head_dim": d, "rotary_dim": d // 2, "theta": 100.0})
             dense = lambda p: PartSpec("swiglu", p + "ff.", {"hidden_size": H, "intermediate_size": self.inner})
             routed = lambda p: PartSpec("toy_routed", p + "ff.", {"hidden_size": H, "intermediate_size": self.inner, "num_experts": self.experts})
+            decay = dict(mixer=PartSpec("toy_decay", "l1.mix.", {"hidden_size": H, "state_size": self.state_size, "decay": self.decay}))
+            head = PartSpec("lm_head", "head.", {"hidden_size": H, "vocab_size": self.vocab_size, "tied_to": None})
+            emb = PartSpec("token_embedding", "emb.", {"vocab_size": self.vocab_size, "hidden_size": H})
+            if self.capturable:
+                layers = [layer("pre_norm_residual", feed_forward=dense(f"l{i}."), mixer_norm=norm(f"l{i}.n1."),
+                                feed_forward_norm=norm(f"l{i}.n2."), **mix)
+                          for i, mix in enumerate([attn("l0.", None, rotary), decay])]
+                return cfgm.ModelSpec("ToyForCausalLM", H, self.vocab_size, emb, tuple(layers), (Run(0), Run(1), Run(1)),
+                                      norm("final."), head)
             layers = []
             for i, (mix, ff) in enumerate([
                     (attn("l0.", self.window, rotary), dense("l0.")),
-                    (dict(mixer=PartSpec("toy_decay", "l1.mix.", {"hidden_size": H, "state_size": self.state_size, "decay": self.decay})), routed("l1.")),
+                    (decay, routed("l1.")),
                     (attn("l2.", None, PartSpec("toy_offset", "l2.pos.", {"head_dim": d, "period": 7})), routed("l2.")),
                     (attn("l3.", self.window - 1, rotary), dense("l3."))]):
                 p = f"l{i}."
-                layers.append(LayerSpec(block="pre_norm_residual", feed_forward=ff, mixer_norm=norm(p + "n1."),
-                                        feed_forward_norm=norm(p + "n2."), **mix))
-            # layer 1 runs twice (two states), the last run reads the keys and values that run 0 stored
-            order = (Run(0), Run(1), Run(2), Run(1), Run(3, cache_of=0))
-            return cfgm.ModelSpec("ToyForCausalLM", H, self.vocab_size,
-                                  PartSpec("token_embedding", "emb.", {"vocab_size": self.vocab_size, "hidden_size": H}),
-                                  tuple(layers), order, norm("final."),
-                                  PartSpec("lm_head", "head.", {"hidden_size": H, "vocab_size": self.vocab_size, "tied_to": None}))
+                layers.append(layer("pre_norm_residual", feed_forward=ff, mixer_norm=norm(p + "n1."),
+                                    feed_forward_norm=norm(p + "n2."), **mix))
+            layers.append(layer("toy_sandwich", pre_mixer_norm=norm("l4.n1."), post_mixer_norm=norm("l4.n2."),
+                                pre_ff_norm=norm("l4.n3."), post_ff_norm=norm("l4.n4."), feed_forward=dense("l4."),
+                                mixer=PartSpec("toy_latent", "l4.mix.", {"hidden_size": H, "latent_size": self.latent, "key_size": 8})))
+            # layer 1 runs twice (two states), run 4 reads the keys and values that run 0 stored, the last layer
+            # has four norms and a cache of one tensor per token
+            order = (Run(0), Run(1), Run(2), Run(1), Run(3, cache_of=0), Run(4))
+            return cfgm.ModelSpec("ToyForCausalLM", H, self.vocab_size, emb, tuple(layers), order, norm("final."), head)
 
     parts.register_part("mixer", "toy_decay", ToyDecay)
+    parts.register_part("mixer", "toy_latent", ToyLatent)
     parts.register_part("feed_forward", "toy_routed", ToyRouted)
     parts.register_part("position", "toy_offset", ToyOffset)
+    parts.register_part("block", "toy_sandwich", ToySandwich)
     cfgm.register_architecture("ToyForCausalLM", ToyConfig)
     return ToyConfig
 
@@ -299,8 +385,13 @@ def toy_plain(w, c, ids):
         out = []
         for t in range(T):
             s = c.decay * s + w["l1.mix.in.weight"] @ h[t]
-            out.append(w["l1.mix.out.weight"] @ s)
+            out.append((w["l1.mix.out.weight"] @ s) / (1 + (t + 1) / 100))
         return torch.stack(out)
+
+    def latent(h):
+        cl = h @ w["l4.mix.c.weight"].T
+        q, k, v = h @ w["l4.mix.q.weight"].T, cl @ w["l4.mix.k.weight"].T, cl @ w["l4.mix.v.weight"].T
+        return P.causal_attention(q[None], k[None], v[None])[0]          # one head, scale 1 / sqrt(key size)
 
     def dense(h, p):
         return P.swiglu_mlp(h, {"gate_proj.weight": w[p + "ff.gate_proj.weight"], "up_proj.weight": w[p + "ff.up_proj.weight"],
@@ -317,6 +408,12 @@ def toy_plain(w, c, ids):
         return out
 
     n = lambda t, p: P.rms_norm(t, w[p + "weight"], c.eps)
+    if c.capturable:
+        a, _ = attn(n(x, "l0.n1."), "l0.", None, "rotary"); x = x + a
+        x = x + dense(n(x, "l0.n2."), "l0.")
+        for _ in range(2):
+            x = x + decay(n(x, "l1.n1.")); x = x + dense(n(x, "l1.n2."), "l1.")
+        return n(x, "final.") @ w["head.weight"].T
     a, kv0 = attn(n(x, "l0.n1."), "l0.", c.window, "rotary"); x = x + a
     x = x + dense(n(x, "l0.n2."), "l0.")
     x = x + decay(n(x, "l1.n1.")); x = x + routed(n(x, "l1.n2."), "l1.")
@@ -325,6 +422,8 @@ def toy_plain(w, c, ids):
     x = x + decay(n(x, "l1.n1.")); x = x + routed(n(x, "l1.n2."), "l1.")
     a, _ = attn(n(x, "l3.n1."), "l3.", c.window - 1, "rotary", kv=kv0); x = x + a
     x = x + dense(n(x, "l3.n2."), "l3.")
+    x = x + n(latent(n(x, "l4.n1.")), "l4.n2.")
+    x = x + n(dense(n(x, "l4.n3."), "l4."), "l4.n4.")
     return n(x, "final.") @ w["head.weight"].T
 
 
@@ -334,10 +433,15 @@ def test_toy_architecture_is_registered_built_and_stepped(fw, tmp_path):
                     decay=0.8, window=6, eps=1e-5)
     d = fw.root.write_random_model(tmp_path / "toy", cfg, seed=4, dtype="float32", std=0.25)
     assert type(fw.root.load_config(d)).__name__ == "ToyConfig"
-    runner = fw.engine.load_runner(d, dtype="float32", page_size=4, num_pages=40, max_requests=3, max_len=64)
+    runner = fw.engine.load_runner(d, dtype="float32", page_size=4, num_pages=40, max_requests=3, max_len=64, hip_graphs=True)
+    assert runner.graphs is None            # the routed feed-forward and the latent mixer cannot be captured, and say so
     lay = runner.layout
-    assert len(lay.group_keys) == 2 and lay.state_runs == [1, 3] and lay.run_stores == [True, False, True, False, False]
+    assert len(lay.group_keys) == 3 and lay.state_runs == [1, 3]
+    assert lay.run_stores == [True, False, True, False, False, True]
     assert lay.run_group[4] == lay.run_group[0] and lay.run_entry[4] == lay.run_entry[0]
+    assert [t.name for t in lay.group_keys[lay.run_group[5]].tensors] == ["latent"]
+    assert sorted(runner.pools.pages[lay.run_group[5]]) == ["latent"] and len(runner.pools.state[1]) == 2
+    assert runner.manager.bytes_per_token(4) == 4 * (2 * 2 * 2 * 16 + 12)     # two attention caches of k and v, one latent
     w = P.read_weights(d, torch.float64)
     rng = np.random.default_rng(0)
     seqs = {r: [int(t) for t in rng.integers(0, 101, n)] for r, n in (("a", 37), ("b", 22), ("c", 9))}
@@ -365,12 +469,42 @@ def test_toy_architecture_is_registered_built_and_stepped(fw, tmp_path):
         runner.manager.check_invariants()
     for r in ("b", "c"):
         assert np.abs(np.concatenate(out[r]) - want[r]).max() < 1e-3, r
-    # the windowed group has given pages back along the way; the full group has not
-    full = [i for i, k in enumerate(lay.group_keys) if k.window is None][0]
+    # the windowed group has given pages back along the way; the groups that keep everything have not
     held = runner.manager.pages_held("b")
-    assert len(held[full]) == 6 and len(held[1 - full]) < 6
+    for g, key in enumerate(lay.group_keys):
+        assert (len(held[g]) == 6) == (key.window is None)
     runner.free_request("b"); runner.free_request("c")
     assert all(g.allocator.num_in_use() == 0 for g in runner.manager.groups)
+
+
+def test_a_mixer_with_state_that_says_so_decodes_from_graphs(fw, tmp_path):
+    """The decaying-state mixer handles single tokens with device tensors only and declares ``graph_safe``: a model of
+    it, attention and dense feed-forwards decodes from captured graphs, several steps to a launch too, rows that
+    pad a batch touch nobody's state, a one-token prompt starts from zero state, and a finished request's slot is
+    used again."""
+    ToyConfig = register_toys(fw)
+    cfg = ToyConfig(vocab_size=101, width=40, heads=4, kv_heads=2, head_size=16, inner=56, experts=3, state_size=24,
+                    decay=0.8, window=6, eps=1e-5, capturable=True)
+    d = fw.root.write_random_model(tmp_path / "toy", cfg, seed=6, dtype="float32", std=0.25)
+    w = P.read_weights(d, torch.float64)
+
+    def plain_greedy(prompt, n):
+        ids = list(prompt)
+        for _ in range(n):
+            ids.append(int(toy_plain(w, cfg, torch.tensor(ids))[-1].argmax()))
+        return ids[len(prompt):]
+
+    rng = np.random.default_rng(3)
+    prompts = [[int(t) for t in rng.integers(0, 101, n)] for n in (7, 1, 12, 4, 9)]
+    want = [plain_greedy(p, 14) for p in prompts]
+    model = fw.root.load_model(d, "float32")
+    for per_launch in (1, 4):
+        e = fw.root.Engine(model, block_size=4, max_seqs=3, max_len=32, hip_graphs=True, decode_steps_per_launch=per_launch)
+        assert e.runner.graphs is not None and e.runner.graphs.buckets
+        reqs = [e.add_request(fw.root.Request(p, max_new_tokens=14)) for p in prompts]   # five requests, three rows
+        e.run_until_idle()
+        assert [r.output_ids for r in reqs] == want, per_launch
+        assert any(rec.decode_batch and rec.decode_steps for rec in e.steps)
 
 
 def test_rotary_part_and_block_alone(fw):
