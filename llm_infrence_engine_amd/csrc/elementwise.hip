@@ -34,15 +34,16 @@ extern "C" int ms_embed(const int* ids, const void* table, float* out, int n_tok
 template <typename T, typename TD>
 __global__ void rms_norm_kernel(float* __restrict__ x, const TD* __restrict__ delta, int n_partials,
                                 size_t partial_stride, const float* __restrict__ w,
-                                const int* __restrict__ rows, T* __restrict__ out, int H, float eps, int write_back) {
+                                const int* __restrict__ rows, T* __restrict__ out, int H, float eps, int write_back,
+                                int staged) {
   __shared__ float red[16];
-  extern __shared__ float buf[];  // H floats: the row after the residual sum
+  extern __shared__ float buf[];  // H floats: the row after the residual sum (a row too wide for it is read twice)
   const int r = blockIdx.x;
   const int src = rows ? rows[r] : r;
   float* xr = x + (size_t)src * H;
   T* o = out + (size_t)r * H;
   float ss = 0.f;
-  if (H % 4 == 0 && n_partials == 1) {  // four values at a time (rows start 16-byte aligned when H % 4 == 0)
+  if (H % 4 == 0 && n_partials == 1 && staged) {  // four values at a time (rows start 16-byte aligned when H % 4 == 0)
     const TD* dr = delta ? delta + (size_t)src * H : nullptr;
     for (int i = threadIdx.x * 4; i < H; i += blockDim.x * 4) {
       float4 v = *reinterpret_cast<const float4*>(xr + i);
@@ -71,12 +72,21 @@ __global__ void rms_norm_kernel(float* __restrict__ x, const TD* __restrict__ de
       for (int p = 0; p < n_partials; ++p) v += to_float(delta[p * partial_stride + (size_t)src * H + i]);
       if (write_back) xr[i] = v;
     }
-    buf[i] = v;
+    if (staged) buf[i] = v;
     ss += v * v;
   }
   ss = block_sum(ss, red);
   const float inv = 1.0f / sqrtf(ss / (float)H + eps);
-  for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = from_float<T>(w[i] * (buf[i] * inv));
+  if (staged) {
+    for (int i = threadIdx.x; i < H; i += blockDim.x) o[i] = from_float<T>(w[i] * (buf[i] * inv));
+    return;
+  }
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {   // the same sum again, in the same order: the same value
+    float v = xr[i];                                     // (each thread reads back what it wrote itself)
+    if (delta && !write_back)
+      for (int p = 0; p < n_partials; ++p) v += to_float(delta[p * partial_stride + (size_t)src * H + i]);
+    o[i] = from_float<T>(w[i] * (v * inv));
+  }
 }
 
 extern "C" int ms_rms_norm(float* x, const void* delta, int delta_dtype, int n_partials, long long partial_stride,
@@ -84,10 +94,13 @@ extern "C" int ms_rms_norm(float* x, const void* delta, int delta_dtype, int n_p
                            int write_back, int dtype, hipStream_t stream) {
   if (n_rows <= 0) return MS_OK;
   if (delta && (n_partials < 1 || partial_stride < 0)) return MS_BAD_ARG;
-  if (hidden <= 0 || hidden > 16384) return MS_UNSUPPORTED;  // the row is staged in LDS
+  if (hidden <= 0) return MS_BAD_ARG;
   dim3 grid(n_rows), block(hidden >= 1024 ? 256 : 128);
-  size_t lds = (size_t)hidden * sizeof(float);
-#define LAUNCH(T, TD) rms_norm_kernel<T, TD><<<grid, block, lds, stream>>>(x, (const TD*)delta, n_partials, (size_t)partial_stride, weight, rows, (T*)out, hidden, eps, write_back)
+  // the row is staged in LDS while it fits what a launch may ask for without more ado (64 KB with the 64 bytes
+  // of the reduction); a wider row is read from memory a second time instead
+  const int staged = (size_t)hidden * sizeof(float) + 64 <= 65536 ? 1 : 0;
+  size_t lds = staged ? (size_t)hidden * sizeof(float) : 0;
+#define LAUNCH(T, TD) rms_norm_kernel<T, TD><<<grid, block, lds, stream>>>(x, (const TD*)delta, n_partials, (size_t)partial_stride, weight, rows, (T*)out, hidden, eps, write_back, staged)
   if (dtype == MS_F32) {
     if (delta && delta_dtype == MS_BF16) return MS_BAD_ARG;
     LAUNCH(float, float);

@@ -38,7 +38,7 @@ def test_embed(ops, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H", [72, 896, 1500])
+@pytest.mark.parametrize("H", [72, 896, 1500, 16384, 20000])
 def test_rms_norm(ops, dtype, H):
     g = torch.Generator().manual_seed(1)
     x = (torch.randn(9, H, generator=g) * 3).to(DEV)
@@ -59,6 +59,14 @@ def test_rms_norm(ops, dtype, H):
     out3 = torch.empty(3, H, dtype=dtype, device=DEV)
     ops.rms_norm(x2, w, 1e-5, out3, rows=rows)
     torch.testing.assert_close(out3.double(), want[rows.long()], **tol(dtype))
+    # the sum formed but not kept, from two partial sums
+    x3 = x.clone()
+    halves = torch.stack((delta.float() * 0.25, delta.float() * 0.75)).to(dtype)
+    ops.rms_norm(x3, w, 1e-5, out, delta=halves, write_back=False)
+    assert torch.equal(x3, x)
+    s = x.double() + halves[0].double() + halves[1].double()
+    want = w.double() * (s * torch.rsqrt((s ** 2).mean(-1, keepdim=True) + 1e-5))
+    torch.testing.assert_close(out.double(), want, **tol(dtype))
 
 
 def test_rms_norm_eps_inside_root(ops):

@@ -137,25 +137,36 @@ def test_trace_run_program(tmp_path_factory, tmp_path):
     compare(traces.collect(steps, out, 384), want, "float32", reqs)
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_replay_at_the_widths_of_the_half_billion_model(tmp_path_factory, tmp_path, dtype):
-    """The layer sizes of Qwen2.5-0.5B (hidden 896, 14 heads over 2 key/value heads of 64, intermediate 4864,
-    vocabulary 151936, tied head) with two layers: the kernels at the sizes they serve."""
+HALF_B_WIDTHS = {"architectures": ["Qwen2ForCausalLM"], "num_hidden_layers": 2, "hidden_size": 896, "num_attention_heads": 14,
+                 "num_key_value_heads": 2, "intermediate_size": 4864, "vocab_size": 151936, "rope_theta": 1000000.0,
+                 "rms_norm_eps": 1e-6, "tie_word_embeddings": True}
+
+
+@pytest.fixture(scope="module")
+def half_b(tmp_path_factory):
     from llm_infrence_engine_amd.config import config_from_dict
     from llm_infrence_engine_amd.weights import write_random_model
 
-    cfg = {"architectures": ["Qwen2ForCausalLM"], "num_hidden_layers": 2, "hidden_size": 896, "num_attention_heads": 14,
-           "num_key_value_heads": 2, "intermediate_size": 4864, "vocab_size": 151936, "rope_theta": 1000000.0,
-           "rms_norm_eps": 1e-6, "tie_word_embeddings": True}
     d = tmp_path_factory.mktemp("halfb")
-    write_random_model(d, config_from_dict(cfg), seed=7, dtype="bfloat16", std=0.05)
+    write_random_model(d, config_from_dict(HALF_B_WIDTHS), seed=7, dtype="bfloat16", std=0.05)
     reqs = make_requests(151936, [90, 40, 150], seed=3)
-    want = oracle(d, reqs)
-    steps = traces.mixed(reqs, 64 * 5, seed=2)
-    # logits of every place would be 150 MB a request: ask for the last place of every portion only
+    return d, reqs, oracle(d, reqs)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("mode", ["whole", "bulk_then_single", "changing_portions", "mixed"])
+def test_replay_at_the_widths_of_the_half_billion_model(half_b, tmp_path, dtype, mode):
+    """The layer sizes of Qwen2.5-0.5B (hidden 896, 14 heads over 2 key/value heads of 64, intermediate 4864,
+    vocabulary 151936, tied head) with two layers: the kernels at the sizes they serve, in all four ways of
+    cutting the work."""
+    d, reqs, want = half_b
+    steps = traces.mixed(reqs, 64 * 5, seed=2) if mode == "mixed" else getattr(traces, mode)(reqs)
+    # logits of every place would be 150 MB a request: ask for the last place of every portion only, and of
+    # whole requests every sixteenth place as well
     for st in steps:
         for e in st["entries"]:
-            e["want"] = [len(e["tokens"]) - 1]
+            n = len(e["tokens"])
+            e["want"] = sorted(set(range(15, n, 16)) | {n - 1}) if mode == "whole" else [n - 1]
     run_replay(d, dtype, steps, tmp_path, 64 * 5, page_size=16)
     worst = compare(traces.collect(steps, tmp_path, 151936), want, dtype, reqs)
-    print(f"0.5B widths {dtype}: worst error is {worst:.3f} of its bound")
+    print(f"0.5B widths {dtype} {mode}: worst error is {worst:.3f} of its bound")
