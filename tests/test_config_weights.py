@@ -168,3 +168,35 @@ def test_kept_types():
     assert place(bf[0], TensorSpec("b", (4,), "bias"), torch.bfloat16, "cpu").dtype == torch.float32
     assert place(bf[0], TensorSpec("n", (4,), "norm"), torch.bfloat16, "cpu").dtype == torch.float32
     assert place(torch.arange(4), TensorSpec("t", (4,), "table"), torch.bfloat16, "cpu").dtype == torch.int32
+
+
+def test_a_layer_names_its_parts_and_the_arrangement_says_which_it_takes():
+    """``LayerSpec(block, parts)``: the arrangement builds the parts it names; a part it does not take, or a missing
+    one, is an error that names it; a position encoding is optional and goes to the mixer."""
+    from llm_infrence_engine_amd.config import layer, preset
+    from llm_infrence_engine_amd.parts import CacheNeed, KVNeed, PageTensor
+
+    spec = config_from_dict(preset("tinyA")).to_spec()
+    ls = spec.layers[0]
+    assert ls.block == "pre_norm_residual" and sorted(ls.parts) == ["feed_forward", "feed_forward_norm", "mixer",
+                                                                    "mixer_norm", "position"]
+    assert ls.mixer.kind == "gqa_attention" and ls.no_such_part is None
+    block = Model(spec).layers[0]
+    assert block.mixer.position is block.position and [type(p).__name__ for p in block.parts()] == \
+        ["RMSNorm", "GQAttention", "RMSNorm", "SwiGLU"]
+    assert block.cache_need() == KVNeed(2, 16, None) and block.state_need() is None and block.graph_safe()
+    assert block.cache_need() == CacheNeed((PageTensor("k", 2, 16), PageTensor("v", 2, 16)), None)
+
+    def model_with(parts):
+        return Model(ModelSpec(spec.architecture, spec.hidden_size, spec.vocab_size, spec.embedding,
+                               (layer("pre_norm_residual", **parts),), (Run(0),), spec.final_norm, spec.head))
+
+    parts = dict(ls.parts)
+    with pytest.raises(KeyError, match="post_norm"):
+        model_with({**parts, "post_norm": parts["mixer_norm"]})
+    with pytest.raises(KeyError, match="feed_forward_norm"):
+        model_with({k: v for k, v in parts.items() if k != "feed_forward_norm"})
+    no_position = model_with({k: v for k, v in parts.items() if k != "position"})
+    assert no_position.layers[0].position is None and no_position.layers[0].mixer.position is None
+    with pytest.raises(ValueError, match="each name once"):
+        CacheNeed((PageTensor("k", 1, 8), PageTensor("k", 1, 8)))
