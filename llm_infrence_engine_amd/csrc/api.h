@@ -57,6 +57,8 @@ int ms_gemm_skinny_norm(const float* x, long long ldx, const int* rows, const fl
                         long long ldw, const float* bias, void* out, long long ldo, int M, int N, int K, int epilogue,
                         int out_dtype, hipStream_t stream);
 
+void ms_qkv_rope_store_force(int pair8);
+
 int ms_qkv_rope_store(const float* x, long long ldx, const float* norm_w, float eps, const void* W, const float* bias,
                       const int* positions, const float* inv_freq, const int* slot_mapping, void* q_out,
                       void* k_pages, void* v_pages, int M, int K, int num_heads, int num_kv_heads, int head_dim,

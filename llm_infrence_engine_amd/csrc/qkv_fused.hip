@@ -3,7 +3,8 @@
 //   (half-split pairing, float angles) -> q to its buffer, k and v straight into their cache pages.
 // A block owns two 16-row tiles of the packed [q heads | k heads | v heads] weight that lie half a head
 // apart, so a lane ends up holding both members (j, j + d/2) of four rotary pairs of one token and can
-// rotate them in registers.  Requires the rotary dimension to be the whole head and d/2 a multiple of 16.
+// rotate them in registers; or, for few tokens, one tile of 8 + 8 such rows (see PAIR8).  Requires the rotary
+// dimension to be the whole head and d/2 a multiple of 16.
 #include "common.h"
 #include "api.h"
 
@@ -33,37 +34,46 @@ __device__ __forceinline__ void sincos_rot(float x, float* sn, float* cs) {
   *cs = ((q + 1) & 2) ? -c1 : c1;
 }
 
-template <int MT, int WAVES>
+// PAIR8: a block owns one 16-row tile made of 8 rows from the lower half of a head and the 8 rows half a head
+// above them, so a rotary pair (j, j + d/2) lies in two lanes of one token, 32 lanes apart, and is rotated after
+// one exchange between them.  Twice as many blocks as with two whole tiles, each streaming half the weights: for
+// few tokens, where a block's time is what its CU can draw and there are fewer blocks than CUs.
+template <int MT, int WAVES, bool PAIR8>
 __global__ void __launch_bounds__(WAVES * MS_WAVE)
 qkv_rope_store_kernel(const float* __restrict__ X, size_t ldx, const float* __restrict__ norm_w, float eps,
                       const bf16* __restrict__ W, const float* __restrict__ bias, const int* __restrict__ positions,
                       const float* __restrict__ inv_freq, const int* __restrict__ slot_mapping,
                       bf16* __restrict__ q_out, bf16* __restrict__ k_pages, bf16* __restrict__ v_pages, int M, int K,
                       int nh, int nkv, int d, int page_size, int v_transposed) {
-  __shared__ f32x4 red[WAVES - 1][2][MT][MS_WAVE];
+  constexpr int NACC = PAIR8 ? 1 : 2;
+  __shared__ f32x4 red[WAVES - 1][NACC][MT][MS_WAVE];
   __shared__ float red_ss[WAVES][MT][16];
   const int lane = threadIdx.x & (MS_WAVE - 1), wave = threadIdx.x / MS_WAVE;
   const int col = lane & 15, kq = lane >> 4;
-  const int pairs_per_head = d / 32;
   const int m0 = blockIdx.z * 16 * MT;                    // token groups beyond MT per block: further blocks along z
   const int head = blockIdx.y;                           // 0..nh-1: q, then nkv k heads, then nkv v heads
-  const int j0 = blockIdx.x * 16;                         // first feature of the low tile within the head
   const int half = d / 2;
+  const int j0 = blockIdx.x * (PAIR8 ? 8 : 16);           // first feature of the block's lower rows within the head
   const int total_steps = (K + 31) / 32;
 
-  const bf16* w_lo = W + ((size_t)head * d + j0 + col) * K + kq * 8;
-  const bf16* w_hi = w_lo + (size_t)half * K;
+  // PAIR8: row `col` of the tile is lower feature j0 + col (col < 8) or upper feature j0 + col - 8 + d/2
+  const int row_lo = PAIR8 ? (col < 8 ? j0 + col : j0 + col - 8 + half) : j0 + col;
+  const bf16* w_lo = W + ((size_t)head * d + row_lo) * K + kq * 8;
+  const bf16* w_hi = w_lo + (size_t)half * K;            // not PAIR8: the tile half a head above
   size_t xrow[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) xrow[t] = (size_t)min(m0 + t * 16 + col, M - 1) * ldx + kq * 8;
 
-  // what the epilogue will need from memory is asked for now, so that it arrives under the main loop
-  const int jl = j0 + kq * 4;
+  // what the epilogue will need from memory is asked for now, so that it arrives under the main loop.
+  // A lane ends up with four features of one token: not PAIR8, j0 + kq*4 + r of the lower tile and the same of the
+  // upper; PAIR8, lanes kq = 0, 1 the lower features j0 + kq*4 + r, lanes kq = 2, 3 their partners half a head up.
+  const int jl = PAIR8 ? j0 + (kq & 1) * 4 : j0 + kq * 4;   // the lower feature of this lane's first pair
+  const bool upper = PAIR8 && kq >= 2;
   float b_lo[4], b_hi[4], freq[4];
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
-    b_lo[r] = bias ? bias[head * d + jl + r] : 0.f;
-    b_hi[r] = bias ? bias[head * d + jl + half + r] : 0.f;
+    b_lo[r] = bias ? bias[head * d + jl + r + (upper ? half : 0)] : 0.f;
+    b_hi[r] = (bias && !PAIR8) ? bias[head * d + jl + half + r] : 0.f;
     freq[r] = head < nh + nkv ? inv_freq[jl + r] : 0.f;
   }
   int pos_m[MT], slot_m[MT];
@@ -86,7 +96,7 @@ qkv_rope_store_kernel(const float* __restrict__ X, size_t ldx, const float* __re
     f32x4 nw0 = {0.f, 0.f, 0.f, 0.f}, nw1 = {0.f, 0.f, 0.f, 0.f};
     if (in) {
       wl = *reinterpret_cast<const bf16x8*>(w_lo + k);
-      wh = *reinterpret_cast<const bf16x8*>(w_hi + k);
+      if (!PAIR8) wh = *reinterpret_cast<const bf16x8*>(w_hi + k);
       nw0 = *reinterpret_cast<const f32x4*>(norm_w + k + kq * 8);
       nw1 = *reinterpret_cast<const f32x4*>(norm_w + k + kq * 8 + 4);
     }
@@ -105,7 +115,7 @@ qkv_rope_store_kernel(const float* __restrict__ X, size_t ldx, const float* __re
         }
       }
       lo[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wl, av, lo[t], 0, 0, 0);
-      hi[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wh, av, hi[t], 0, 0, 0);
+      if (!PAIR8) hi[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wh, av, hi[t], 0, 0, 0);
     }
   }
 
@@ -117,19 +127,16 @@ qkv_rope_store_kernel(const float* __restrict__ X, size_t ldx, const float* __re
     const int owner = t % WAVES;  // token group t is finished by wave t; the others leave their share in LDS
     if (wave != owner) {
       red[wave < owner ? wave : wave - 1][0][t][lane] = lo[t];
-      red[wave < owner ? wave : wave - 1][1][t][lane] = hi[t];
+      if (!PAIR8) red[wave < owner ? wave : wave - 1][NACC - 1][t][lane] = hi[t];
     }
   }
   __syncthreads();
 
-  // lane holds features j0 + kq*4 + r (lo) and the same + d/2 (hi) of token t*16 + col
-  const int j = j0 + kq * 4;
-  const int row_lo = head * d + j;
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     const int m = m0 + t * 16 + col;
     const int owner = t % WAVES;
-    if (wave != owner || m >= M) continue;
+    if (wave != owner) continue;       // the same for the whole wave (the exchange below needs all its lanes)
     float total = 0.f;
 #pragma unroll
     for (int w = 0; w < WAVES; ++w) total += red_ss[w][t][col];
@@ -140,10 +147,20 @@ qkv_rope_store_kernel(const float* __restrict__ X, size_t ldx, const float* __re
       float va = 0.f, vb = 0.f;
       for (int w = 0; w < WAVES; ++w) {  // in wave order
         va += w == owner ? lo[t][r] : red[w < owner ? w : w - 1][0][t][lane][r];
-        vb += w == owner ? hi[t][r] : red[w < owner ? w : w - 1][1][t][lane][r];
+        if (!PAIR8) vb += w == owner ? hi[t][r] : red[w < owner ? w : w - 1][NACC - 1][t][lane][r];
       }
       a[r] = va * inv + b_lo[r];
       b[r] = vb * inv + b_hi[r];
+    }
+    if (PAIR8) {
+      // the partner of this lane's feature sits 32 lanes away: a lower lane takes (x1, x2) = (own, partner), an
+      // upper lane (partner, own)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float other = __shfl_xor(a[r], 32, MS_WAVE);
+        b[r] = upper ? a[r] : other;
+        a[r] = upper ? other : a[r];
+      }
     }
     if (head < nh + nkv) {  // q and k heads turn by position * inv_freq[j]
       const float pos = (float)pos_m[t];
@@ -156,13 +173,18 @@ qkv_rope_store_kernel(const float* __restrict__ X, size_t ldx, const float* __re
         b[r] = x2 * cs + x1 * sn;
       }
     }
+    if (m >= M) continue;
+    // what this lane stores: not PAIR8 both members (a at j, b at j + d/2); PAIR8 its own member only
+    const int j = jl;
+    const int row_a = head * d + j;
     bf16x4 pa, pb;
 #pragma unroll
     for (int r = 0; r < 4; ++r) { pa[r] = (__bf16)a[r]; pb[r] = (__bf16)b[r]; }
+    const bool store_a = !PAIR8 || !upper, store_b = !PAIR8 || upper;
     if (head < nh) {
-      bf16* qp = q_out + (size_t)m * nh * d + row_lo;
-      *reinterpret_cast<bf16x4*>(qp) = pa;
-      *reinterpret_cast<bf16x4*>(qp + half) = pb;
+      bf16* qp = q_out + (size_t)m * nh * d + row_a;
+      if (store_a) *reinterpret_cast<bf16x4*>(qp) = pa;
+      if (store_b) *reinterpret_cast<bf16x4*>(qp + half) = pb;
       continue;
     }
     const long long slot = slot_m[t];
@@ -173,40 +195,51 @@ qkv_rope_store_kernel(const float* __restrict__ X, size_t ldx, const float* __re
     const int off = pow2 ? (int)(slot & (page_size - 1)) : (int)(slot % page_size);
     if (head < nh + nkv) {
       bf16* kp = k_pages + (((size_t)page * nkv + (head - nh)) * page_size + off) * d + j;
-      *reinterpret_cast<bf16x4*>(kp) = pa;
-      *reinterpret_cast<bf16x4*>(kp + half) = pb;
+      if (store_a) *reinterpret_cast<bf16x4*>(kp) = pa;
+      if (store_b) *reinterpret_cast<bf16x4*>(kp + half) = pb;
     } else if (v_transposed) {
       bf16* vp = v_pages + (((size_t)page * nkv + (head - nh - nkv)) * d + j) * page_size + off;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        vp[(size_t)r * page_size] = __float2bfloat16(a[r]);
-        vp[(size_t)(half + r) * page_size] = __float2bfloat16(b[r]);
+        if (store_a) vp[(size_t)r * page_size] = __float2bfloat16(a[r]);
+        if (store_b) vp[(size_t)(half + r) * page_size] = __float2bfloat16(b[r]);
       }
     } else {
       bf16* vp = v_pages + (((size_t)page * nkv + (head - nh - nkv)) * page_size + off) * d + j;
-      *reinterpret_cast<bf16x4*>(vp) = pa;
-      *reinterpret_cast<bf16x4*>(vp + half) = pb;
+      if (store_a) *reinterpret_cast<bf16x4*>(vp) = pa;
+      if (store_b) *reinterpret_cast<bf16x4*>(vp + half) = pb;
     }
   }
 }
+
+int g_qkv_pair8 = -1;   // measurements: 0 / 1 force whole tiles / tiles of 8 + 8 rows, -1 leaves the choice
 
 template <int MT>
 int launch(const float* X, size_t ldx, const float* norm_w, float eps, const bf16* W, const float* bias,
            const int* positions, const float* inv_freq, const int* slot_mapping, bf16* q_out, bf16* k_pages,
            bf16* v_pages, int M, int K, int nh, int nkv, int d, int page_size, int v_transposed, hipStream_t stream) {
-  const int blocks = (nh + 2 * nkv) * (d / 32);
   const int steps = (K + 31) / 32;
+  const int token_groups = (M + 16 * MT - 1) / (16 * MT);
+  // Tiles of 8 + 8 rows (twice the blocks, half the weights each) while there are no more of them than CUs: a block's
+  // time is what its CU can draw.  With more blocks than CUs every block reading all the activations costs
+  // more than the shorter stream of weights saves.
+  const int pair_blocks = (nh + 2 * nkv) * (d / 16) * token_groups;
+  const bool pair8 = g_qkv_pair8 >= 0 ? g_qkv_pair8 != 0 : pair_blocks <= ms_compute_units();
+  const int blocks = pair8 ? pair_blocks : pair_blocks / 2;
   // LDS holds (waves - 1) * 2 * MT KB.  (Measured at the 0.5B and 7B shapes: 8 waves are 0.4 to 1 us faster than
   // 16; tiles of 8 or 4 rows on more CUs are slower, by up to 2x, because every block reads all activations.)
   int waves = 4;
   while (waves < 8 && blocks * waves < 1024 && steps >= waves * 2) waves *= 2;
-#define GO(WV) qkv_rope_store_kernel<MT, WV><<<dim3(d / 32, nh + 2 * nkv, (M + 16 * MT - 1) / (16 * MT)), dim3(WV * MS_WAVE), 0, stream>>>(X, ldx, norm_w, eps, W, bias, positions, inv_freq, slot_mapping, q_out, k_pages, v_pages, M, K, nh, nkv, d, page_size, v_transposed)
-  if (waves == 4) GO(4); else GO(8);
+#define GO(WV, P8) qkv_rope_store_kernel<MT, WV, P8><<<dim3(d / (P8 ? 16 : 32), nh + 2 * nkv, token_groups), dim3(WV * MS_WAVE), 0, stream>>>(X, ldx, norm_w, eps, W, bias, positions, inv_freq, slot_mapping, q_out, k_pages, v_pages, M, K, nh, nkv, d, page_size, v_transposed)
+  if (pair8) { if (waves == 4) GO(4, true); else GO(8, true); }
+  else { if (waves == 4) GO(4, false); else GO(8, false); }
 #undef GO
   return ms_launch_status();
 }
 
 }  // namespace
+
+extern "C" void ms_qkv_rope_store_force(int pair8) { g_qkv_pair8 = pair8; }
 
 // x float [M, K] (M <= 64), W bfloat16 [(nh + 2 nkv) d, K] packed q | k | v, bias float or null,
 // q_out bfloat16 [M, nh d], pages bfloat16 as in ms_rope_store, inv_freq float [d / 2].

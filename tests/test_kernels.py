@@ -789,7 +789,21 @@ def test_gemm_skinny_with_the_norm_folded_in(ops, M, N, K):
 
 @pytest.mark.parametrize("M", [1, 8, 40])
 @pytest.mark.parametrize("nh,nkv,d,K,v_transposed", [(14, 2, 64, 896, True), (6, 3, 32, 72, False), (4, 1, 128, 200, True)])
-def test_qkv_rope_store_fused_equals_the_separate_kernels(ops, M, nh, nkv, d, K, v_transposed):
+@pytest.mark.parametrize("tiles", ["whole", "8+8"])
+def test_qkv_rope_store_fused_equals_the_separate_kernels(ops, M, nh, nkv, d, K, v_transposed, tiles):
+    """Both shapes of block: two whole tiles half a head apart, and one tile of 8 + 8 rows whose rotary pairs lie in
+    two lanes (the choice between them goes by the number of blocks; here each is forced in turn)."""
+    from llm_infrence_engine_amd.kernels import build
+
+    lib = build.load()
+    lib.ms_qkv_rope_store_force(0 if tiles == "whole" else 1)
+    try:
+        _qkv_fused_case(ops, M, nh, nkv, d, K, v_transposed)
+    finally:
+        lib.ms_qkv_rope_store_force(-1)
+
+
+def _qkv_fused_case(ops, M, nh, nkv, d, K, v_transposed):
     g = torch.Generator().manual_seed(M + d)
     page_size, pages = 16, 12
     x = (torch.randn(M, K, generator=g) * 2).to(DEV)
