@@ -34,13 +34,13 @@ def main(argv=None) -> int:
     ap.add_argument("--sample-seed", type=int, default=None)
     ap.add_argument("--eos-ids", default="", help="stop ids, e.g. 151645,151643")
     ap.add_argument("--max-len", type=int, default=1024)
-    ap.add_argument("--max-seqs", type=int, default=32)
+    ap.add_argument("--max-seqs", "--max-num-seqs", dest="max_seqs", type=int, default=32)
     ap.add_argument("--num-blocks", type=int, default=None)
     ap.add_argument("--block-size", type=int, default=16)
     ap.add_argument("--max-num-batched-tokens", type=int, default=2048)
     ap.add_argument("--gpu-memory-fraction", type=float, default=None,
                     help="without --num-blocks: size the page pool to this share of the device's memory, weights included")
-    ap.add_argument("--cuda-graphs", "--hip-graphs", dest="hip_graphs", action="store_true", default=None,
+    ap.add_argument("--cuda-graphs", "--hip-graphs", "--hip-graph", dest="hip_graphs", action="store_true", default=None,
                     help="replay decode-only steps from captured HIP graphs (the default in bfloat16)")
     ap.add_argument("--no-hip-graphs", dest="hip_graphs", action="store_false", help="launch every kernel of a decode step")
     ap.add_argument("--decode-steps-per-launch", type=int, default=1,
