@@ -528,14 +528,17 @@ extern "C" int ms_paged_attention_mfma(const void* q, long long q_stride, const 
   const int cols = max_q_len * (num_heads / num_kv_heads);
   int nt = cols > 16 ? (head_dim == 128 ? 2 : 4) : 1;
   int waves = nt > 1 ? 4 : (head_dim == 128 ? 8 : 16);
-  // narrow tiles, far fewer of them than compute units: blocks share a tile's dims while that leaves half the
-  // units free (with every unit busy the keys' repeated reading costs more than the shorter chains save:
-  // 64 requests at 1,000 keys took 12.1 us shared two ways against 11.1)
+  // narrow tiles, fewer of them than compute units: blocks share a tile's dims as far as there is a unit for
+  // every block (measured at 200, 640 and 1,000 keys, head sizes 64 and 128: up to 64 tiles four ways, up to 128
+  // two ways, e.g. 128 tiles at 640 keys 8.0 -> 7.0 us; with more blocks than units the keys' repeated reading
+  // costs more than the shorter streams save).  Very many tiles of the large head size: four waves to a tile
+  // (512 tiles at 640 keys: 32.2 -> 29.3 us).
   int vs = 1;
   if (nt == 1) {
     const long long tiles = (long long)n_requests * num_kv_heads * ((cols + 15) / 16);
     const int cus = ms_compute_units();
-    while (vs < 4 && (head_dim / 16) % (vs * 2) == 0 && tiles * vs * 4 <= cus) vs *= 2;
+    while (vs < 4 && (head_dim / 16) % (vs * 2) == 0 && tiles * vs * 2 <= cus) vs *= 2;
+    if (head_dim == 128 && tiles >= 2LL * cus) waves = 4;
   }
   if (g_force_nt) { nt = g_force_nt; waves = g_force_waves; }
   if (g_force_vs) vs = g_force_vs;
