@@ -84,7 +84,7 @@ def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None
            out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """[M, K] x [N, K] -> [M, N] in ``out_dtype`` (default: a's type).  ``a`` may be a ``LazyNorm``."""
     if isinstance(a, LazyNorm):
-        if ops.skinny_norm_ok(a.x, w, a.num_rows):
+        if ops.skinny_norm_ok(a.x, w, a.num_rows) and ops.fold_norm_pays(a.num_rows, a.x.shape[1]):
             try:
                 return ops.gemm_skinny_norm(a.x, a.weight, a.eps, w, bias, ops.EPI_STORE, out_dtype or a.out_dtype, a.rows)
             except ops.UnsupportedShape:
@@ -125,7 +125,7 @@ def linear_swiglu(a: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
     """silu(a @ gate.T) * (a @ up.T) for ``w_gate_up`` = interleave_rows(gate, up): [M, I].  ``a`` may be a
     ``LazyNorm``."""
     if isinstance(a, LazyNorm):
-        if ops.skinny_norm_ok(a.x, w_gate_up, a.num_rows):
+        if ops.skinny_norm_ok(a.x, w_gate_up, a.num_rows) and ops.fold_norm_pays(a.num_rows, a.x.shape[1]):
             try:
                 return ops.gemm_skinny_norm(a.x, a.weight, a.eps, w_gate_up, None, ops.EPI_SWIGLU, rows=a.rows)
             except ops.UnsupportedShape:

@@ -445,11 +445,32 @@ def qkv_rope_store_ok(x: torch.Tensor, w: torch.Tensor, head_dim: int, rot_dim: 
     return skinny_norm_ok(x, w, x.shape[0]) and head_dim % 32 == 0 and rot_dim == head_dim
 
 
-def qkv_rope_store_pays(x: torch.Tensor) -> bool:
-    """Whether the one kernel is the faster way.  Every block of it reads all the rows of the float residual stream;
-    with many long rows (measured: 64 rows of 5,120 take 85 us fused against 58 us as product and rotation apart,
-    64 rows of 3,584 the same either way) the product that holds the activations in LDS and a rotation kernel win."""
-    return x.shape[0] * x.shape[1] <= 64 * 4096
+_cus = {}
+
+
+def compute_units(device) -> int:
+    """Compute units of the device (256 on an MI355X)."""
+    key = torch.device(device).index or 0
+    if key not in _cus:
+        _cus[key] = torch.cuda.get_device_properties(key).multi_processor_count
+    return _cus[key]
+
+
+def qkv_rope_store_pays(x: torch.Tensor, w_qkv: torch.Tensor) -> bool:
+    """Whether the one kernel is the faster way.  Each of its blocks (32 rows of the weight by 16 tokens) reads the
+    float residual stream of its tokens again; as long as every block has a CU of its own that is cheaper than a
+    kernel boundary, beyond that the norm, the product that holds the activations in LDS and the rotation win as
+    kernels of their own (measured, 64 tokens: width 3,584 45 us fused against 29 + 6; width 5,120 86 against
+    37 + 9; width 896 7 against 9 + 4)."""
+    return (w_qkv.shape[0] // 32) * ((x.shape[0] + 15) // 16) <= compute_units(x.device)
+
+
+def fold_norm_pays(n_rows: int, width: int) -> bool:
+    """Whether a product should read the float residual stream and normalise it itself, rather than read bfloat16
+    rows that a norm kernel of its own (3 to 4 us) has left.  Every block reads all rows of its tokens, so with
+    many long rows the halved read is worth the launch (measured for the gated product: 64 rows of 3,584 82 against
+    72 us, 32 rows of 5,120 129 against 120; 64 rows of 896 15.1 either way; 16 rows: folding wins at every width)."""
+    return n_rows <= 16 or n_rows * width < 72 * 1024
 
 
 def qkv_rope_store(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w_qkv: torch.Tensor,

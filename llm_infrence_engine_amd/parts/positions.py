@@ -28,7 +28,7 @@ class RotaryHalf(PositionEncoding):
 
     def project_encode_store(self, h, w_qkv, bias, num_heads, num_kv_heads, head_dim, ctx, kv):
         if not (isinstance(h, linear.LazyNorm) and h.rows is None and kv is not None and kv.store
-                and ops.qkv_rope_store_ok(h.x, w_qkv, head_dim, self.rotary_dim) and ops.qkv_rope_store_pays(h.x)):
+                and ops.qkv_rope_store_ok(h.x, w_qkv, head_dim, self.rotary_dim) and ops.qkv_rope_store_pays(h.x, w_qkv)):
             return None
         return ops.qkv_rope_store(h.x, h.weight, h.eps, w_qkv, bias, num_heads, num_kv_heads, head_dim, ctx.positions,
                                   self.inv_freq, kv.slot_mapping, kv.k_pages, kv.v_pages, kv.v_transposed)

@@ -205,3 +205,45 @@ def test_random_weights_drawn_on_the_device(eng):
     m2 = eng.load_random_model(cfg, seed=9)
     assert torch.equal(m1.layers[0].mixer.w_qkv, m2.layers[0].mixer.w_qkv)
     assert m1.layers[0].mixer.w_qkv.dtype == torch.bfloat16 and m1.layers[0].mixer.b_qkv.dtype == torch.float32
+
+
+WIDE = {"architectures": ["Qwen2ForCausalLM"], "num_hidden_layers": 2, "hidden_size": 1536,
+        "num_attention_heads": 24, "num_key_value_heads": 12, "intermediate_size": 2304, "vocab_size": 1184,
+        "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "tie_word_embeddings": False}
+
+
+def test_many_rows_of_wide_layers_take_the_norm_kernel_and_follow_plain(eng, tmp_path):
+    """48 decode rows of width 1,536: the products no longer fold the norm in (they read bfloat16 rows that a norm
+    kernel leaves) and the q/k/v projection, rotation and cache store run as kernels of their own.  With 8 rows the
+    same layers take the fused kernels.  Both follow the plain implementation."""
+    from llm_infrence_engine_amd.config import config_from_dict
+    from llm_infrence_engine_amd.engine import StepEntry
+    from llm_infrence_engine_amd.kernels import ops
+
+    n_rows = 48
+    x = torch.empty(n_rows, WIDE["hidden_size"], device="cuda:0")
+    w_qkv = torch.empty((24 + 2 * 12) * 64, WIDE["hidden_size"], dtype=torch.bfloat16, device="cuda:0")
+    assert not ops.fold_norm_pays(n_rows, WIDE["hidden_size"]) and ops.fold_norm_pays(8, WIDE["hidden_size"])
+    assert not ops.qkv_rope_store_pays(x, w_qkv) and ops.qkv_rope_store_pays(x[:8], w_qkv)
+    d = tmp_path / "m"
+    eng.write_random_model(d, config_from_dict(WIDE), seed=21, dtype="bfloat16", std=0.04)
+    cfg, w = P.read_config(d), P.read_weights(d, torch.float64)
+    rng = np.random.default_rng(4)
+    prompts = [[int(t) for t in rng.integers(0, cfg["vocab_size"], 20 + i % 7)] for i in range(n_rows)]
+    model = eng.load_model(str(d), "bfloat16")
+    e = eng.Engine(model, block_size=16, max_seqs=n_rows, max_len=64, max_num_batched_tokens=2048, hip_graphs=True,
+                   capture_at_start=False)
+    runner = e.runner
+    runner.step([StepEntry(i, p[:-1], []) for i, p in enumerate(prompts)])
+    checked = 0
+    for rows in (n_rows, 8):                       # all rows in a step, then the first eight alone
+        lg = runner.step([StepEntry(i, [prompts[i][-1]] if rows == n_rows else [7], [0]) for i in range(rows)])
+        lg = lg.float().cpu().numpy()
+        for i in range(0, rows, 5):
+            seq = prompts[i] + ([7] if rows == 8 else [])
+            exact = P.forward(w, cfg, seq)[-1].numpy()
+            noise = float(np.abs(P.forward(w, cfg, seq, act_dtype=torch.bfloat16)[-1].numpy() - exact).max())
+            err = np.abs(lg[i] - exact).max()
+            assert err < BF16_NOISE * noise, f"{rows} rows, request {i}: {err:.3e} >= {BF16_NOISE * noise:.3e}"
+            checked += 1
+    assert checked == 12
