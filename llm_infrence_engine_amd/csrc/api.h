@@ -53,6 +53,14 @@ int ms_gemm_panel_splitk(const void* A, long long lda, const void* W, long long 
                          long long ldo, int M, int N, int K, int epilogue, int out_dtype, void* partial, int parts,
                          hipStream_t stream);
 
+// Many rows (prompt portions): the tiled matrix-core product, bfloat16 in and out, with the gated activation
+// as epilogue 1; K a multiple of 64 (ms_gemm_tiled_force: measurements, 0 leaves the choice of tile;
+// ms_gemm_tiled_pays: whether the gated product is faster here than as library product and activation kernel).
+int ms_gemm_tiled(const void* A, long long lda, const void* W, long long ldw, void* out, long long ldo, int M, int N,
+                  int K, int epilogue, hipStream_t stream);
+void ms_gemm_tiled_force(int tile);
+int ms_gemm_tiled_pays(int M, int N, int K);
+
 int ms_gemm_skinny_norm(const float* x, long long ldx, const int* rows, const float* norm_w, float eps, const void* W,
                         long long ldw, const float* bias, void* out, long long ldo, int M, int N, int K, int epilogue,
                         int out_dtype, hipStream_t stream);

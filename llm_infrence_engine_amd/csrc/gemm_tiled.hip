@@ -1,0 +1,246 @@
+// out[M,N] = A[M,K] . W[N,K]^T for many tokens (prompt portions), bfloat16 in, float accumulation on the
+// matrix cores (v_mfma_f32_16x16x32_bf16), with the gated activation as an epilogue: the product of the
+// interleaved gate/up weight never goes to memory, which saves the write of [M, 2I], its read and a kernel.
+//
+// A block of 8 waves owns a tile of BN features by BM tokens.  What bounds such a kernel on this chip is what a
+// CU can draw through its load path, so the tile is as large as registers allow (256 x 256: a byte loaded does
+// 128 multiply-adds).  Per step of 64 columns the tile's rows of W and A go from memory straight to LDS
+// (global_load_lds, 16 bytes a lane: no registers, no LDS write instructions) into the other of two buffers
+// while the waves multiply the step before; one barrier ends the step.  LDS rows are 128 bytes with their eight 16-byte
+// pieces permuted by the row number (piece c at place c ^ (row & 7)): fragment reads then run at the full LDS
+// rate (measured 237 bytes a clock; rows 144 bytes apart give 116).
+//
+// W is the A operand of the MFMA and the tokens the B operand, so a lane ends up with 4 output features of one
+// token per tile.  Which 16 features make up a tile is free: tile i of a wave takes, for q = 0..3, the four
+// features q * 4 FT + i * 4 .. + 3 of the wave's FT * 16, so that the lane with quarter q holds 4 FT consecutive
+// features of its token over its FT tiles and stores them as one run.
+#include "common.h"
+#include "api.h"
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+enum { EPI_STORE = 0, EPI_SWIGLU = 1 };
+
+constexpr int BK = 64;                  // columns a step
+constexpr int PITCH = BK;               // LDS rows of 128 bytes; piece c of row l lies at place c ^ (l & 7)
+
+// LDS row l of the block's W rows (l < WF * FT * 16) holds this feature of the tile
+template <int FT>
+__device__ __forceinline__ int feature_of_row(int l) {
+  const int wf = l / (FT * 16), rem = l - wf * (FT * 16);
+  const int i = rem >> 4, rr = rem & 15;
+  return wf * (FT * 16) + (rr >> 2) * (4 * FT) + i * 4 + (rr & 3);
+}
+
+// WF x WT waves along features and tokens, each with FT x TT tiles of 16 x 16.  K is a multiple of 64.
+template <int WF, int WT, int FT, int TT, int EPI, typename TO>
+__global__ void __launch_bounds__(WF * WT * MS_WAVE)
+gemm_tiled_kernel(const bf16* __restrict__ A, size_t lda, const bf16* __restrict__ W, size_t ldw,
+                  TO* __restrict__ out, size_t ldo, int M, int N, int K, int m_tiles, int n_tiles) {
+  constexpr int NWAVES = WF * WT, THREADS = NWAVES * MS_WAVE;
+  constexpr int BN = WF * FT * 16, BM = WT * TT * 16, ROWS = BN + BM;
+  constexpr int LOADS = ROWS / 8 / NWAVES;   // loads of 8 rows (1 KB) a wave makes per step
+  static_assert(ROWS % (8 * NWAVES) == 0, "the tile's rows are dealt out evenly");
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  bf16* lds = reinterpret_cast<bf16*>(lds_raw);          // two buffers of ROWS x PITCH
+
+  // Blocks with consecutive ids go to consecutive XCDs, each with an L2 of its own: an XCD takes every eighth
+  // tile of W with all token tiles (those fastest), so a tile of W is read from memory by one XCD only.  The
+  // host launches 8 * ceil(n_tiles / 8) * m_tiles blocks; one without a tile leaves.
+  const int nt = ((int)(blockIdx.x >> 3) / m_tiles) * 8 + (blockIdx.x & 7);
+  const int mt = (int)(blockIdx.x >> 3) % m_tiles;
+  if (nt >= n_tiles) return;
+  const int n0 = nt * BN, m0 = mt * BM;
+  const int lane = threadIdx.x & (MS_WAVE - 1), wave = threadIdx.x / MS_WAVE;
+  const int wf = wave % WF, wt = wave / WF;
+  const int col = lane & 15, kq = lane >> 4;
+
+  // Load p of a wave fills LDS rows (wave + p * NWAVES) * 8 .. + 7: lane l's 16 bytes land at l * 16 of that 1 KB,
+  // which is place l & 7 of row l >> 3, so the lane asks memory for the piece that belongs there.  Rows past the
+  // end of W or A repeat the last row (their results are not stored).
+  const bf16* src[LOADS];
+#pragma unroll
+  for (int p = 0; p < LOADS; ++p) {
+    const int l = (wave + p * NWAVES) * 8 + (lane >> 3);
+    const int piece = (lane & 7) ^ (l & 7);
+    if (l < BN) src[p] = W + (size_t)min(n0 + feature_of_row<FT>(l), N - 1) * ldw + piece * 8;
+    else src[p] = A + (size_t)min(m0 + l - BN, M - 1) * lda + piece * 8;
+  }
+  typedef __attribute__((address_space(3))) void lds_void;
+  typedef const __attribute__((address_space(1))) void global_void;
+  auto load_rows = [&](int k, int buffer) {
+#pragma unroll
+    for (int p = 0; p < LOADS; ++p)
+      __builtin_amdgcn_global_load_lds((global_void*)(src[p] + k),
+                                       (lds_void*)(lds + buffer + (wave + p * NWAVES) * 8 * PITCH), 16, 0, 0);
+  };
+
+  f32x4 acc[FT][TT];
+#pragma unroll
+  for (int i = 0; i < FT; ++i)
+#pragma unroll
+    for (int j = 0; j < TT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const int steps = K / BK;
+  load_rows(0, 0);
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): the loads to LDS have landed
+  __syncthreads();
+
+  // a lane's fragment pieces: columns kq * 8 of the first 32 columns of a step at place kq ^ (row & 7), of the
+  // second 32 at that place ^ 4 (rows of a tile start at a multiple of 16, so row & 7 is col & 7)
+  constexpr int KS = BK / 32;
+  static_assert(KS == 2, "a step is two products deep");
+  const int place[KS] = {(kq ^ (col & 7)) * 8, ((kq + 4) ^ (col & 7)) * 8};
+  const bf16* w_frag = lds + (wf * FT * 16 + col) * PITCH;
+  const bf16* a_frag = lds + (BN + wt * TT * 16 + col) * PITCH;
+  for (int s = 0; s < steps; ++s) {
+    const int buf = (s & 1) * ROWS * PITCH;
+    // the next step's rows go into the buffer that the step before read; they have this step to arrive
+    if (s + 1 < steps) load_rows((s + 1) * BK, ((s + 1) & 1) * ROWS * PITCH);
+    // the tokens' fragments of both halves of the step first, then the tiles of W one ahead of their products
+    bf16x8 av[KS][TT];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int j = 0; j < TT; ++j) av[ks][j] = *reinterpret_cast<const bf16x8*>(a_frag + buf + j * 16 * PITCH + place[ks]);
+    bf16x8 w_next = *reinterpret_cast<const bf16x8*>(w_frag + buf + place[0]);
+#pragma unroll
+    for (int t = 0; t < FT * KS; ++t) {
+      const int ks = t / FT, i = t % FT;
+      const bf16x8 w_cur = w_next;
+      if (t + 1 < FT * KS)
+        w_next = *reinterpret_cast<const bf16x8*>(w_frag + buf + ((t + 1) % FT) * 16 * PITCH + place[(t + 1) / FT]);
+#pragma unroll
+      for (int j = 0; j < TT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_cur, av[ks][j], acc[i][j], 0, 0, 0);
+    }
+    // the order of the instructions: the first fragments, then one read ahead of every TT products (left to
+    // itself the compiler reads a fragment right before its products and waits for it)
+    __builtin_amdgcn_sched_group_barrier(0x100, KS * TT + 1, 0);
+#pragma unroll
+    for (int t = 0; t + 1 < FT * KS; ++t) {
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x008, TT, 0);
+    }
+    __builtin_amdgcn_sched_group_barrier(0x008, TT, 0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+  }
+
+  // the lane's run of 4 FT features of token m (tile j): acc[i][j][r] is feature f0 + i * 4 + r
+  const int f0 = n0 + wf * (FT * 16) + kq * (4 * FT);
+#pragma unroll
+  for (int j = 0; j < TT; ++j) {
+    const int m = m0 + wt * TT * 16 + j * 16 + col;
+    if (m >= M) continue;
+    if (EPI == EPI_SWIGLU) {   // features 2g, 2g + 1 are gate g and up g: 2 FT outputs from o0 on
+      const int o0 = f0 / 2, n_out = N / 2;
+      TO* o = out + (size_t)m * ldo + o0;
+      float v[2 * FT];
+#pragma unroll
+      for (int i = 0; i < FT; ++i) {
+        v[2 * i] = fast_silu(acc[i][j][0]) * acc[i][j][1];
+        v[2 * i + 1] = fast_silu(acc[i][j][2]) * acc[i][j][3];
+      }
+      if (o0 + 2 * FT <= n_out && ((uintptr_t)o & 15) == 0 && sizeof(TO) == 2) {
+#pragma unroll
+        for (int g = 0; g < 2 * FT; g += 8) {
+          bf16x8 pk;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) pk[e] = (__bf16)v[g + e];
+          *reinterpret_cast<bf16x8*>(reinterpret_cast<bf16*>(o) + g) = pk;
+        }
+      } else {
+#pragma unroll
+        for (int g = 0; g < 2 * FT; ++g)
+          if (o0 + g < n_out) o[g] = from_float<TO>(v[g]);
+      }
+    } else {
+      TO* o = out + (size_t)m * ldo + f0;
+      if (f0 + 4 * FT <= N && ((uintptr_t)o & 15) == 0 && sizeof(TO) == 2) {
+#pragma unroll
+        for (int g = 0; g < 4 * FT; g += 8) {
+          bf16x8 pk;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) pk[e] = (__bf16)acc[(g + e) >> 2][j][(g + e) & 3];
+          *reinterpret_cast<bf16x8*>(reinterpret_cast<bf16*>(o) + g) = pk;
+        }
+      } else {
+#pragma unroll
+        for (int g = 0; g < 4 * FT; ++g)
+          if (f0 + g < N) o[g] = from_float<TO>(acc[g >> 2][j][g & 3]);
+      }
+    }
+  }
+}
+
+template <int WF, int WT, int FT, int TT, int EPI, typename TO>
+int launch(const bf16* A, size_t lda, const bf16* W, size_t ldw, TO* out, size_t ldo, int M, int N, int K,
+           hipStream_t stream) {
+  constexpr int BN = WF * FT * 16, BM = WT * TT * 16;
+  constexpr size_t lds = 2 * (size_t)(BN + BM) * PITCH * sizeof(bf16);
+  static bool raised = false;   // once per instantiation: allow more dynamic LDS than the default 64 KB
+  if (!raised) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_tiled_kernel<WF, WT, FT, TT, EPI, TO>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return MS_LAUNCH_FAILED;
+    raised = true;
+  }
+  const int n_tiles = (N + BN - 1) / BN, m_tiles = (M + BM - 1) / BM;
+  const long long blocks = (long long)((n_tiles + 7) / 8) * 8 * m_tiles;
+  if (blocks > 0x7fffffffLL) return MS_UNSUPPORTED;
+  gemm_tiled_kernel<WF, WT, FT, TT, EPI, TO><<<dim3((unsigned)blocks), dim3(WF * WT * MS_WAVE), lds, stream>>>(
+      A, lda, W, ldw, out, ldo, M, N, K, m_tiles, n_tiles);
+  return ms_launch_status();
+}
+
+int g_tile = 0;   // measurements: 0 leaves the choice of tile, 1 and 2 force one
+
+// Tiles of 256 x 256 (a byte loaded does 128 multiply-adds; one block to a CU, 1.7 us a step of 64 columns) or of
+// 128 x 128 (two blocks to a CU, 1.26 us a step each): the one whose rounds of blocks over the CUs take less.
+int choose_tile(int M, int N) {
+  const long long cus = ms_compute_units();
+  const long long big = (long long)((N + 255) / 256) * ((M + 255) / 256);
+  const long long small = (long long)((N + 127) / 128) * ((M + 127) / 128);
+  const double t_big = (double)((big + cus - 1) / cus) * 1.70, t_small = (double)((small + 2 * cus - 1) / (2 * cus)) * 1.26;
+  return t_big <= t_small ? 1 : 2;
+}
+
+}  // namespace
+
+extern "C" void ms_gemm_tiled_force(int tile) { g_tile = tile; }
+
+// Whether the gated product of M tokens is faster here than as the library's product and an activation kernel
+// (measured with a different W every call, 65 to 8,192 tokens): up to 1,536 columns always (0.5 to 0.98 of the
+// library's time); beyond that the two are within 15 % of each other either way, and this kernel is taken where it
+// won throughout: up to 2,048 tokens whose 256 x 256 tiles fill at least 9/10 of their last round over the CUs.
+extern "C" int ms_gemm_tiled_pays(int M, int N, int K) {
+  if (M <= 0 || N <= 0 || K <= 0 || K % BK) return 0;
+  if (K <= 1536) return 1;
+  if (M > 2048) return 0;
+  const long long cus = ms_compute_units();
+  const long long big = (long long)((N + 255) / 256) * ((M + 255) / 256);
+  return big * 10 >= ((big + cus - 1) / cus) * cus * 9;
+}
+
+// A bfloat16 [M, lda], W bfloat16 [N, ldw] (rows of K, K a multiple of 64), out bfloat16.
+// epilogue 0: out[M, N] = product;  epilogue 1: out[M, N / 2] = silu(gate) * up over interleaved rows of W.
+extern "C" int ms_gemm_tiled(const void* A, long long lda, const void* W, long long ldw, void* out, long long ldo, int M,
+                             int N, int K, int epilogue, hipStream_t stream) {
+  if (M <= 0 || N <= 0) return MS_OK;
+  if (K <= 0 || K % BK || lda % 8 || ldw % 8 || lda < K || ldw < K) return MS_UNSUPPORTED;
+  if (((uintptr_t)A | (uintptr_t)W) % 16) return MS_UNSUPPORTED;
+  if (epilogue == EPI_SWIGLU ? (N % 2 || ldo < N / 2) : (epilogue != EPI_STORE || ldo < N)) return MS_BAD_ARG;
+  const bf16* a = (const bf16*)A;
+  const bf16* w = (const bf16*)W;
+  bf16* o = (bf16*)out;
+  int tile = g_tile;
+  if (tile == 0) tile = choose_tile(M, N);
+#define GO(WF, WT, FT, TT) return epilogue == EPI_SWIGLU ? launch<WF, WT, FT, TT, EPI_SWIGLU, bf16>(a, lda, w, ldw, o, ldo, M, N, K, stream) \
+                                                        : launch<WF, WT, FT, TT, EPI_STORE, bf16>(a, lda, w, ldw, o, ldo, M, N, K, stream)
+  if (tile == 1) GO(2, 4, 8, 4);   // 256 x 256
+  GO(2, 4, 4, 2);                  // 128 x 128
+#undef GO
+}

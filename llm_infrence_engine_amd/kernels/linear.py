@@ -5,7 +5,9 @@ bfloat16, few rows (a decode step)   the weight-streaming matrix-core kernel, wi
                  activation or split-K partial sums as its epilogue.
 bfloat16, many rows (prompt portions)  the library's matrix product (hipBLASLt through torch.mm), as the
                  reference uses a library for every product (F.linear, src/miniserve/model.py:123-165);
-                 shapes it cannot take fall back to the vector-ALU kernel.
+                 shapes it cannot take fall back to the vector-ALU kernel.  The gated gate/up product is
+                 the tiled matrix-core kernel of our own where that is the faster one: its epilogue is
+                 the activation, so the product itself is never written or read again.
 All accumulate in float.
 """
 from __future__ import annotations
@@ -136,6 +138,11 @@ def linear_swiglu(a: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
             return ops.gemm_skinny(a, w_gate_up, None, ops.EPI_SWIGLU)
         except ops.UnsupportedShape:
             _fell_back(a.shape[0], w_gate_up.shape[0], w_gate_up.shape[1], "gated product")
+    if a.shape[0] > ops.SKINNY_MAX_ROWS and ops.gemm_tiled_pays(a, w_gate_up):
+        try:
+            return ops.gemm_tiled(a, w_gate_up, ops.EPI_SWIGLU)   # many rows: the activation is the product's epilogue
+        except ops.UnsupportedShape:
+            _fell_back(a.shape[0], w_gate_up.shape[0], w_gate_up.shape[1], "tiled gated product")
     gu = linear(a, w_gate_up)
     act = torch.empty((a.shape[0], w_gate_up.shape[0] // 2), dtype=a.dtype, device=a.device)
     return ops.silu_mul(gu, act)

@@ -38,6 +38,9 @@ _SIGNATURES = {
     "ms_gemm_panel_splitk_parts": [_c_int, _c_int, _c_int],
     "ms_gemm_panel_splitk": [_c_ptr, _c_ll, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int,
                              _c_ptr, _c_int, _c_ptr],
+    "ms_gemm_tiled": [_c_ptr, _c_ll, _c_ptr, _c_ll, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "ms_gemm_tiled_force": [_c_int],
+    "ms_gemm_tiled_pays": [_c_int, _c_int, _c_int],
     "ms_read_probe_blocks": [],
     "ms_read_probe": [_c_ptr, _c_ll, _c_ptr, _c_ptr],
     "ms_residual_add": [_c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr],
@@ -338,6 +341,28 @@ def gemm_skinny(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] =
             return out
     _call("ms_gemm_skinny", a.data_ptr(), lda, w.data_ptr(), K, _ptr(bias), out.data_ptr(), ldo,
           M, N, K, epilogue, _code(out_dtype), _stream())
+    return out
+
+
+def gemm_tiled_pays(a: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether ``gemm_tiled(a, w, EPI_SWIGLU)`` takes these sizes and is the faster way to the gated product."""
+    return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.dim() == 2 and a.is_contiguous()
+            and w.is_contiguous() and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
+            and bool(_get("ms_gemm_tiled_pays")(a.shape[0], w.shape[0], a.shape[1])))
+
+
+def gemm_tiled(a: torch.Tensor, w: torch.Tensor, epilogue: int = EPI_STORE) -> torch.Tensor:
+    """a [M, K] @ w [N, K].T for many rows on the matrix cores, bfloat16 in and out: EPI_STORE -> [M, N];
+    EPI_SWIGLU over interleaved rows of w (2j: gate j, 2j + 1: up j) -> [M, N / 2], the product itself never
+    written.  K a multiple of 64 (else ``UnsupportedShape``)."""
+    _check(a, "a", torch.bfloat16)
+    _check(w, "w", torch.bfloat16, (None, a.shape[1]))
+    if epilogue not in (EPI_STORE, EPI_SWIGLU):
+        raise ValueError("the tiled product stores its result or the gated activation of it")
+    M, K = a.shape
+    N = w.shape[0]
+    out = torch.empty((M, N // 2 if epilogue == EPI_SWIGLU else N), dtype=torch.bfloat16, device=a.device)
+    _call("ms_gemm_tiled", a.data_ptr(), K, w.data_ptr(), K, out.data_ptr(), out.shape[1], M, N, K, epilogue, _stream())
     return out
 
 

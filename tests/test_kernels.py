@@ -571,6 +571,54 @@ def test_gemm_skinny_refuses_what_it_cannot_take(ops):
         ops.gemm_skinny(a[:4, :60], w[:, :60].contiguous())
 
 
+@pytest.mark.parametrize("tile", [1, 2])
+@pytest.mark.parametrize("M,N,K", [(65, 662, 64), (300, 2 * 331, 192), (257, 130, 896), (1000, 2 * 4864, 896), (2051, 1026, 128),
+                                   (130, 16, 64), (513, 4100, 1536)])
+def test_gemm_tiled(ops, M, N, K, tile):
+    """The many-rows product and its gated epilogue with either tile shape: rows and features that fill no
+    whole tile, one step of 64 columns and many."""
+    force = ops._get("ms_gemm_tiled_force")
+    force.restype = None
+    g = torch.Generator().manual_seed(M + N)
+    a = torch.randn(M, K, generator=g).bfloat16().to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16().to(DEV)
+    a[M - 1] *= 3.0                                        # the last row is told apart from a repeated one before it
+    want = a.double() @ w.double().T
+    force(tile)
+    try:
+        out = ops.gemm_tiled(a, w)
+        act = ops.gemm_tiled(a, w, ops.EPI_SWIGLU)
+    finally:
+        force(0)
+    assert out.shape == (M, N) and act.shape == (M, N // 2) and out.dtype == act.dtype == torch.bfloat16
+    torch.testing.assert_close(out.double(), want, **tol(torch.bfloat16))
+    torch.testing.assert_close(act.double(), torch.nn.functional.silu(want[:, 0::2]) * want[:, 1::2], **tol(torch.bfloat16))
+    # a row's result does not depend on what else is in the batch
+    assert torch.equal(ops.gemm_tiled(a[M - 70:], w), out[M - 70:])
+
+
+def test_gemm_tiled_refuses_what_it_cannot_take_and_linear_goes_on(ops):
+    from llm_infrence_engine_amd.kernels import linear
+
+    g = torch.Generator().manual_seed(5)
+    a = torch.randn(100, 72, generator=g).bfloat16().to(DEV)
+    w = (torch.randn(60, 72, generator=g) / 8).bfloat16().to(DEV)
+    with pytest.raises(ops.UnsupportedShape):
+        ops.gemm_tiled(a, w)                               # 72 columns: no multiple of 64
+    assert not ops.gemm_tiled_pays(a, w)
+    with pytest.raises(TypeError):
+        ops.gemm_tiled(a.float(), w)
+    # the dispatcher: wide enough rows of a narrow model go to the tiled kernel, others to the library
+    a2 = torch.randn(200, 128, generator=g).bfloat16().to(DEV)
+    w2 = (torch.randn(96, 128, generator=g) / 11).bfloat16().to(DEV)
+    assert ops.gemm_tiled_pays(a2, w2)
+    got = linear.linear_swiglu(a2, w2)
+    ref = a2.double() @ w2.double().T
+    torch.testing.assert_close(got.double(), torch.nn.functional.silu(ref[:, 0::2]) * ref[:, 1::2], **tol(torch.bfloat16))
+    assert torch.equal(got, ops.gemm_tiled(a2, w2, ops.EPI_SWIGLU))
+    assert linear.fallback_count() == 0 or all(k[3] != "tiled gated product" for k in linear.fallbacks)
+
+
 def test_linear_picks_a_kernel_for_every_shape(ops):
     from llm_infrence_engine_amd.kernels import linear
 
