@@ -35,6 +35,22 @@ __device__ __forceinline__ int feature_of_row(int l) {
   return wf * (FT * 16) + (rr >> 2) * (4 * FT) + i * 4 + (rr & 3);
 }
 
+// The instruction order of a step's first half, told to the scheduler: before the TT products of tile I the reads
+// that the source has there (the next tile of W but for the last, tile I of the second half, token fragment I
+// of the second half while there are any).  0x100: reads from LDS, 0x008: matrix instructions.
+template <int I, int FT, int TT>
+struct FirstHalfOrder {
+  static __device__ __forceinline__ void apply() {
+    __builtin_amdgcn_sched_group_barrier(0x100, (I + 1 < FT ? 1 : 0) + 1 + (I < TT ? 1 : 0), 0);
+    __builtin_amdgcn_sched_group_barrier(0x008, TT, 0);
+    FirstHalfOrder<I + 1, FT, TT>::apply();
+  }
+};
+template <int FT, int TT>
+struct FirstHalfOrder<FT, FT, TT> {
+  static __device__ __forceinline__ void apply() {}
+};
+
 // WF x WT waves along features and tokens, each with FT x TT tiles of 16 x 16.  K is a multiple of 64.
 template <int WF, int WT, int FT, int TT, int EPI, typename TO>
 __global__ void __launch_bounds__(WF * WT * MS_WAVE)
@@ -84,49 +100,54 @@ gemm_tiled_kernel(const bf16* __restrict__ A, size_t lda, const bf16* __restrict
 #pragma unroll
     for (int j = 0; j < TT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  const int steps = K / BK;
-  load_rows(0, 0);
-  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): the loads to LDS have landed
-  __syncthreads();
-
   // a lane's fragment pieces: columns kq * 8 of the first 32 columns of a step at place kq ^ (row & 7), of the
   // second 32 at that place ^ 4 (rows of a tile start at a multiple of 16, so row & 7 is col & 7)
-  constexpr int KS = BK / 32;
-  static_assert(KS == 2, "a step is two products deep");
-  const int place[KS] = {(kq ^ (col & 7)) * 8, ((kq + 4) ^ (col & 7)) * 8};
+  static_assert(BK == 64, "a step is two products of 32 columns deep");
+  const int place0 = (kq ^ (col & 7)) * 8, place1 = ((kq + 4) ^ (col & 7)) * 8;
   const bf16* w_frag = lds + (wf * FT * 16 + col) * PITCH;
   const bf16* a_frag = lds + (BN + wt * TT * 16 + col) * PITCH;
+
+  // A step has one barrier, in its middle.  First half: the products of the first 32 columns, whose token
+  // fragments are in registers already and whose tiles of W are read one ahead; meanwhile every fragment of the
+  // second 32 columns is read too.  Then nothing of this step is left in its buffer: the wave waits for the rows
+  // of the next step (asked for a step ago), the barrier makes them visible to all and says that all are done
+  // with this buffer, and the rows of the step after next are asked for into it.  Second half: the products of
+  // the second 32 columns from registers, meanwhile the first fragments of the next step are read.  So no read
+  // from LDS and no load from memory is waited for with the matrix pipe idle, except at the barrier itself.
+  const int steps = K / BK;
+  load_rows(0, 0);
+  if (steps > 1) load_rows(BK, ROWS * PITCH);
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): the loads to LDS have landed
+  __syncthreads();
+  bf16x8 a0[TT], a1[TT], w1[FT];
+#pragma unroll
+  for (int j = 0; j < TT; ++j) a0[j] = *reinterpret_cast<const bf16x8*>(a_frag + j * 16 * PITCH + place0);
+  bf16x8 w_next = *reinterpret_cast<const bf16x8*>(w_frag + place0);
   for (int s = 0; s < steps; ++s) {
-    const int buf = (s & 1) * ROWS * PITCH;
-    // the next step's rows go into the buffer that the step before read; they have this step to arrive
-    if (s + 1 < steps) load_rows((s + 1) * BK, ((s + 1) & 1) * ROWS * PITCH);
-    // the tokens' fragments of both halves of the step first, then the tiles of W one ahead of their products
-    bf16x8 av[KS][TT];
+    const int buf = (s & 1) * ROWS * PITCH, other = ((s + 1) & 1) * ROWS * PITCH;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-      for (int j = 0; j < TT; ++j) av[ks][j] = *reinterpret_cast<const bf16x8*>(a_frag + buf + j * 16 * PITCH + place[ks]);
-    bf16x8 w_next = *reinterpret_cast<const bf16x8*>(w_frag + buf + place[0]);
-#pragma unroll
-    for (int t = 0; t < FT * KS; ++t) {
-      const int ks = t / FT, i = t % FT;
+    for (int i = 0; i < FT; ++i) {
       const bf16x8 w_cur = w_next;
-      if (t + 1 < FT * KS)
-        w_next = *reinterpret_cast<const bf16x8*>(w_frag + buf + ((t + 1) % FT) * 16 * PITCH + place[(t + 1) / FT]);
+      if (i + 1 < FT) w_next = *reinterpret_cast<const bf16x8*>(w_frag + buf + (i + 1) * 16 * PITCH + place0);
+      w1[i] = *reinterpret_cast<const bf16x8*>(w_frag + buf + i * 16 * PITCH + place1);
+      if (i < TT) a1[i] = *reinterpret_cast<const bf16x8*>(a_frag + buf + i * 16 * PITCH + place1);
 #pragma unroll
-      for (int j = 0; j < TT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_cur, av[ks][j], acc[i][j], 0, 0, 0);
+      for (int j = 0; j < TT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_cur, a0[j], acc[i][j], 0, 0, 0);
     }
-    // the order of the instructions: the first fragments, then one read ahead of every TT products (left to
-    // itself the compiler reads a fragment right before its products and waits for it)
-    __builtin_amdgcn_sched_group_barrier(0x100, KS * TT + 1, 0);
-#pragma unroll
-    for (int t = 0; t + 1 < FT * KS; ++t) {
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x008, TT, 0);
-    }
-    __builtin_amdgcn_sched_group_barrier(0x008, TT, 0);
-    __builtin_amdgcn_s_waitcnt(0x0F70);
+    // the order of the instructions (left to itself the compiler reads a fragment right before its products and
+    // waits for it): the reads written before each group of TT products stay there
+    FirstHalfOrder<0, FT, TT>::apply();
+    __builtin_amdgcn_s_waitcnt(0x0070);   // vmcnt(0) and lgkmcnt(0): the next step's rows have landed, this step's are read
     __syncthreads();
+    if (s + 2 < steps) load_rows((s + 2) * BK, buf);
+    // (after the last step these reads bring what nobody uses)
+#pragma unroll
+    for (int i = 0; i < FT; ++i) {
+      if (i < TT) a0[i] = *reinterpret_cast<const bf16x8*>(a_frag + other + i * 16 * PITCH + place0);
+      if (i == TT) w_next = *reinterpret_cast<const bf16x8*>(w_frag + other + place0);
+#pragma unroll
+      for (int j = 0; j < TT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w1[i], a1[j], acc[i][j], 0, 0, 0);
+    }
   }
 
   // the lane's run of 4 FT features of token m (tile j): acc[i][j][r] is feature f0 + i * 4 + r
