@@ -2,13 +2,13 @@
 // matrix cores (v_mfma_f32_16x16x32_bf16), with the gated activation as an epilogue: the product of the
 // interleaved gate/up weight never goes to memory, which saves the write of [M, 2I], its read and a kernel.
 //
-// A block of 8 waves owns a tile of BN features by BM tokens.  What bounds such a kernel on this chip is what a
-// CU can draw through its load path, so the tile is as large as registers allow (256 x 256: a byte loaded does
-// 128 multiply-adds).  Per step of 64 columns the tile's rows of W and A go from memory straight to LDS
-// (global_load_lds, 16 bytes a lane: no registers, no LDS write instructions) into the other of two buffers
-// while the waves multiply the step before; one barrier ends the step.  LDS rows are 128 bytes with their eight 16-byte
-// pieces permuted by the row number (piece c at place c ^ (row & 7)): fragment reads then run at the full LDS
-// rate (measured 237 bytes a clock; rows 144 bytes apart give 116).
+// A block of 8 waves owns a tile of BN features by BM tokens, as large as registers allow (256 x 256: a byte
+// loaded does 128 multiply-adds; a CU draws some 80 GB/s from L2).  Per step of 64 columns the tile's rows of W
+// and A go from memory straight to LDS (global_load_lds, 16 bytes a lane: no registers, no LDS write
+// instructions) into one of two buffers, a step before they are multiplied.  LDS rows are 128 bytes with their
+// eight 16-byte pieces permuted by the row number (piece c at place c ^ (row & 7)): fragment reads then run at
+// the full LDS rate (measured 237 bytes a clock; rows 144 bytes apart give 116).  A step has one barrier, in
+// its middle, and the matrix pipe has work on both sides of it (see the main loop).
 //
 // W is the A operand of the MFMA and the tokens the B operand, so a lane ends up with 4 output features of one
 // token per tile.  Which 16 features make up a tile is free: tile i of a wave takes, for q = 0..3, the four
