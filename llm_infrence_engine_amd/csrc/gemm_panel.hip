@@ -4,8 +4,9 @@
 // With this many tokens the activations, not the weights, are most of what a block has to load when it reads
 // them as MFMA operands k-step by k-step: every 16-row tile of W needs all of A again, and what a CU can pull
 // through its load path (from L2 as from memory) is about 1/256 of what the chip can.  So here every block
-// loads A once, whole, into LDS (the panel: bfloat16, K padded to a multiple of 32 with zeros, rows one
-// 16-byte piece apart in the banks), and then streams its share of W against it: the 16-row tiles of W are dealt
+// loads A once, whole, into LDS (the panel: bfloat16, K padded to a multiple of 32 with zeros, rows an odd
+// number of 32 bytes apart, where 16-byte fragment reads run at the full LDS rate; an odd number of 16 bytes
+// gives half of it), and then streams its share of W against it: the 16-row tiles of W are dealt
 // out evenly over as many blocks as the chip has CUs, and inside a block
 //   * rounds of 16 tiles go to the 16 waves whole (no sum across waves);
 //   * the tiles left over (all of them, for a block with fewer than 16) are shared, each among floor(16 / left)
@@ -170,7 +171,7 @@ gemm_panel_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restric
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MS_WAVE);   // the same for the whole wave
   const int col = lane & 15, kq = lane >> 4;
   const int K8 = K / 8, S = (K + 31) / 32;
-  const int pitch = S * 4 + 1;              // odd, so that 16 rows read at one column hit 16 different banks
+  const int pitch = S * 4 + 2;   // rows an odd number of 32 bytes apart: 16-byte fragment reads at the full LDS rate
   const int parts = (K8 + 63) / 64;         // loads of 64 lanes x 8 columns per row of A
   u32x4* xst = smem;
   const u32x4 zero = {0u, 0u, 0u, 0u};
@@ -291,7 +292,7 @@ gemm_panel_chunked_kernel(const void* __restrict__ Av, size_t lda, const bf16* _
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MS_WAVE);   // the same for the whole wave
   const int col = lane & 15, kq = lane >> 4;
   const int C8 = KC / 8;                    // pieces per row of a full chunk (KC is a multiple of 32)
-  const int pitch = C8 + 1;                 // odd, so that 16 rows read at one column hit 16 different banks
+  const int pitch = C8 + 2;      // rows an odd number of 32 bytes apart: 16-byte fragment reads at the full LDS rate
   const int parts = (C8 + 63) / 64;         // loads of 64 lanes x 8 columns per row and chunk
   u32x4* xst = smem;
   const u32x4 zero = {0u, 0u, 0u, 0u};
@@ -476,7 +477,7 @@ int plan(const void* A, size_t lda, const bf16* W, size_t ldw, const float* bias
   const int blocks = tiles < cus ? tiles : cus;
   const int q = tiles / blocks, rem = tiles % blocks;
   const size_t red = (size_t)WAVES * tt * MS_WAVE * 16;
-  size_t lds = (size_t)M * (S * 4 + 1) * 16;
+  size_t lds = (size_t)M * (S * 4 + 2) * 16;
   if (lds <= (size_t)LDS_BUDGET && (K / 8 + 63) / 64 <= MAX_PARTS) {   // the rows fit whole
     if (lds < red) lds = red;
 #define GO(TTV) if (tt == TTV) return launch<TTV, EPI, TO, NORM>(A, lda, W, ldw, bias, out, ldo, M, N, K, norm_w, eps, rows, blocks, q, rem, lds, stream)
@@ -487,10 +488,10 @@ int plan(const void* A, size_t lda, const bf16* W, size_t ldw, const float* bias
   // in chunks of KC columns: the widest of 2048, 1536, 1024, 512 that fits
   int KC = 0;
   for (int kc = 2048; kc >= 512; kc -= 512) {
-    if ((size_t)M * (kc / 8 + 1) * 16 <= (size_t)LDS_BUDGET) { KC = kc; break; }
+    if ((size_t)M * (kc / 8 + 2) * 16 <= (size_t)LDS_BUDGET) { KC = kc; break; }
   }
   if (!KC) return MS_UNSUPPORTED;
-  lds = (size_t)M * (KC / 8 + 1) * 16;
+  lds = (size_t)M * (KC / 8 + 2) * 16;
   if (lds < red) lds = red;
   const int nacc = (q + (rem ? 1 : 0)) / WAVES;   // whole tiles a wave keeps accumulators for
   if (nacc > 3 || (tt == 4 && nacc > 2)) return MS_UNSUPPORTED;   // what a lane's registers hold
@@ -534,10 +535,10 @@ int run_splitk(const bf16* A, size_t lda, const bf16* W, size_t ldw, const float
   const int tt = (M + 15) / 16;
   int KC = 0;
   for (int kc = 2048; kc >= 512; kc -= 512) {
-    if ((size_t)M * (kc / 8 + 1) * 16 <= (size_t)LDS_BUDGET) { KC = kc; break; }
+    if ((size_t)M * (kc / 8 + 2) * 16 <= (size_t)LDS_BUDGET) { KC = kc; break; }
   }
   if (!KC) return MS_UNSUPPORTED;
-  size_t lds = (size_t)M * (KC / 8 + 1) * 16;
+  size_t lds = (size_t)M * (KC / 8 + 2) * 16;
   const size_t red = (size_t)WAVES * tt * MS_WAVE * 16;
   if (lds < red) lds = red;
   int rc = MS_UNSUPPORTED;

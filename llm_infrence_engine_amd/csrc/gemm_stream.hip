@@ -62,7 +62,7 @@ gemm_stream_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
   const int r0 = 4 * (b * q + min(b, rem));
   const int R = 4 * (q + (b < rem ? 1 : 0));   // at most 16 * NT and at most rcap; may run past N in the last block
   const int C8cap = min(KC, (K + 31) / 32 * 32) / 8;   // pieces per row of a full stage
-  const int pitch = C8cap + 1;                          // odd, so that 16 rows read at one column hit 16 banks
+  const int pitch = C8cap + 2;   // rows an odd number of 32 bytes apart: 16-byte fragment reads at the full LDS rate
   const int parts = (C8cap + 63) / 64;                  // loads per row and stage
   const int parts_inv = small_inverse(parts);
   u32x4* wst = smem;
@@ -294,7 +294,7 @@ int plan(const void* A, size_t lda, const bf16* W, size_t ldw, const float* bias
   size_t lds = 0;
   for (int kc = KC_MAX; kc >= 256; kc /= 2) {
     const int c8 = (kc < k32 ? kc : k32) / 8, parts = (c8 + 63) / 64;
-    lds = (size_t)(rcap + M) * (c8 + 1) * 16;
+    lds = (size_t)(rcap + M) * (c8 + 2) * 16;
     if (rcap * parts <= WI_MAX * WAVES && M * parts <= (NORM ? XI_F32 : XI_BF16) * WAVES && lds <= (size_t)LDS_BUDGET) {
       KC = kc;
       break;
