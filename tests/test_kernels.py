@@ -953,6 +953,32 @@ def test_random_product_shapes_are_right_whatever_kernel_takes_them(ops):
         assert (total - x.double() - want).abs().max().item() < (1e-4 if d is None else 0.05), (case, M, N, K)
 
 
+def test_random_gated_products_of_many_rows(ops):
+    """Random shapes of more than 64 rows through ``linear_swiglu``: the tiled kernel where it takes the sizes
+    (columns in steps of 64) and pays, the library's product and the activation kernel otherwise."""
+    from llm_infrence_engine_amd.kernels import linear
+
+    rng = np.random.default_rng(23)
+    g = torch.Generator(device=DEV).manual_seed(23)
+    tiled = 0
+    for case in range(60):
+        M = int(rng.choice([rng.integers(65, 300), rng.integers(300, 3000)]))
+        inter = int(rng.choice([rng.integers(1, 200), rng.integers(200, 6000)]))
+        K = int(rng.choice([64 * rng.integers(1, 40), 8 * rng.integers(1, 300)]))
+        a = torch.randn(M, K, generator=g, device=DEV).bfloat16()
+        gate = (torch.randn(inter, K, generator=g, device=DEV) / math.sqrt(K)).bfloat16()
+        up = (torch.randn(inter, K, generator=g, device=DEV) / math.sqrt(K)).bfloat16()
+        w = linear.interleave_rows(gate, up)
+        tiled += ops.gemm_tiled_pays(a, w)
+        got = linear.linear_swiglu(a, w)
+        want = torch.nn.functional.silu(a.double() @ gate.double().T) * (a.double() @ up.double().T)
+        assert got.shape == (M, inter)
+        err = (got.double() - want).abs().max().item()
+        # the result is rounded to bfloat16 once; where the library writes the product first, that is rounded too
+        assert err < 2.5e-2 * max(1.0, want.abs().max().item()), (case, M, inter, K, err)
+    assert 15 < tiled < 60
+
+
 def test_read_probe_reads_everything_once(ops):
     t = torch.randint(-2 ** 31, 2 ** 31 - 1, (1 << 20,), dtype=torch.int32, device=DEV)
     for n in (1 << 20, 4 * 1000, 4):
