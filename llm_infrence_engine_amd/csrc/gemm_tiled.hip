@@ -60,6 +60,7 @@ gemm_tiled_kernel(const bf16* __restrict__ A, size_t lda, const bf16* __restrict
   constexpr int BN = WF * FT * 16, BM = WT * TT * 16, ROWS = BN + BM;
   constexpr int LOADS = ROWS / 8 / NWAVES;   // loads of 8 rows (1 KB) a wave makes per step
   static_assert(ROWS % (8 * NWAVES) == 0, "the tile's rows are dealt out evenly");
+  static_assert(TT < FT, "the main loop reads the token fragments beside the first TT + 1 tiles of W");
   extern __shared__ __align__(16) unsigned char lds_raw[];
   bf16* lds = reinterpret_cast<bf16*>(lds_raw);          // two buffers of ROWS x PITCH
 
