@@ -415,9 +415,9 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
 }
 
 // out[r, h, :] = sum_s 2^(m_s - M) O_s / sum_s 2^(m_s - M) l_s over the splits that request r used.
-// One block per (request, head): the splits' maxima and sums are fetched side by side (a thread each), the
+// One block per (request, head): the splits' maxima and sums are fetched side by side, the
 // weights are worked out once into LDS, then a thread per dim adds the weighted partial results in split order.
-constexpr int COMBINE_MAX_SPLITS = 64;
+constexpr int COMBINE_MAX_SPLITS = 128;
 
 template <int D>
 __global__ void __launch_bounds__(D < 64 ? 64 : D)
@@ -434,18 +434,17 @@ attention_combine_kernel(const float* __restrict__ part_o, const float* __restri
   const int used = (blocks + per - 1) / per;
   const size_t slot0 = ((size_t)r * nh + h) * n_splits;
   const int t = threadIdx.x;
-  float l_mine = 0.f;
-  if (t < used) {
-    sm_m[t] = part_ml[(slot0 + t) * 2];
-    l_mine = part_ml[(slot0 + t) * 2 + 1];
-  }
+  for (int s = t; s < used; s += blockDim.x) sm_m[s] = part_ml[(slot0 + s) * 2];
   __syncthreads();
   float big = -INFINITY;
   for (int s = 0; s < used; ++s) big = fmaxf(big, sm_m[s]);
-  if (t < used) sm_w[t] = fast_exp2(sm_m[t] - big);
   __syncthreads();
-  // the denominator in split order; sm_m now carries the splits' sums
-  if (t < used) sm_m[t] = sm_w[t] * l_mine;
+  // the weights, and in sm_m (no longer needed) the splits' weighted sums for the denominator in split order
+  for (int s = t; s < used; s += blockDim.x) {
+    const float w = fast_exp2(sm_m[s] - big);
+    sm_w[s] = w;
+    sm_m[s] = w * part_ml[(slot0 + s) * 2 + 1];
+  }
   __syncthreads();
   float den = 0.f;
   for (int s = 0; s < used; ++s) den += sm_m[s];

@@ -603,8 +603,8 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, vt_pages: torch
         # (measured with contexts of 128 to 4,352 keys: 64 requests x 2 kv heads 30.6 us unsplit, 23.8 in 4 splits;
         # 32 x 2: 29.8, 20.7 in 4, 15.4 in 8; 16 x 4 of 128 dims: 50.7, 23.3 in 8; 8 x 2 at 7,600 keys: 45.6, 13.3
         # in 16, 13.1 in 32).  Contexts of tens of thousands of keys may take more splits, as far as the blocks
-        # allow (one request of 100,000 keys: 2.6 ms a decode step in 16 splits).
-        most = MAX_SPLITS * (1 if max_context_len <= 16384 else (2 if max_context_len <= 65536 else 4))
+        # allow (one request of 100,000 keys, two kv heads: 61 us in 16 splits, 24.4 in 64, 23.4 in 128, 27 in 256).
+        most = MAX_SPLITS * (1 if max_context_len <= 16384 else (2 if max_context_len <= 65536 else 8))
         n_splits = max(1, min(most, SPLIT_BLOCKS // max(1, R * nkv)))
         part_o = torch.empty((R, num_heads, n_splits, d), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((R, num_heads, n_splits, 2), dtype=torch.float32, device=q.device)

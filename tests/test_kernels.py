@@ -728,7 +728,7 @@ def test_split_decode_attention_of_a_large_uneven_batch(ops, R, nh, nkv, d, wind
 
 @pytest.mark.parametrize("longest,splits_window", [(17000, None), (70000, None), (70000, 30000)])
 def test_split_decode_attention_of_very_long_contexts(ops, longest, splits_window):
-    """Tens of thousands of keys: more splits than at a few thousand (32 and 64), beside a short request that
+    """Tens of thousands of keys: more splits than at a few thousand (32 and 128), beside a short request that
     uses one of them."""
     nh, nkv, d = 4, 2, 64
     g = torch.Generator().manual_seed(longest)
