@@ -52,6 +52,26 @@ __device__ __forceinline__ float fast_silu(float g) {
   return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g));
 }
 
+// sin and cos of a rotation angle for bfloat16 results: three-part Cody-Waite reduction by pi/2 (the first
+// two parts have 11 bits, so n * part is exact for |x| < 2^13 * pi/2) and short polynomials on [-pi/4, pi/4];
+// absolute error ~2e-7.  Larger angles take the library routine.
+__device__ __forceinline__ void ms_sincos_rot(float x, float* sn, float* cs) {
+  if (fabsf(x) > 12000.f) { sincosf(x, sn, cs); return; }
+  const float n = rintf(x * 0.636619772367581343f);
+  float r = fmaf(-n, 1.5703125f, x);
+  r = fmaf(-n, 4.837512969970703e-4f, r);
+  r = fmaf(-n, 7.549790126404332e-08f, r);
+  const float r2 = r * r;
+  const float sp = fmaf(r2, fmaf(r2, fmaf(r2, 2.7557314297e-6f, -1.9841270114e-4f), 8.3333337680e-3f), -1.6666667163e-1f);
+  const float s0 = fmaf(r * r2, sp, r);
+  const float cp = fmaf(r2, fmaf(r2, fmaf(r2, 2.4801587642e-5f, -1.3888889225e-3f), 4.1666667908e-2f), -0.5f);
+  const float c0 = fmaf(r2, cp, 1.0f);
+  const int q = (int)n & 3;
+  const float s1 = (q & 1) ? c0 : s0, c1 = (q & 1) ? s0 : c0;
+  *sn = (q & 2) ? -s1 : s1;
+  *cs = ((q + 1) & 2) ? -c1 : c1;
+}
+
 // Compute units of the current device (256 on an MI355X); asked once.
 static inline int ms_compute_units() {
   static int n = 0;

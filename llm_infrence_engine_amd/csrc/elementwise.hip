@@ -289,7 +289,12 @@ rope_store_vec_kernel(T* __restrict__ qkv, const float* __restrict__ bias, const
   const int half = rot_dim / 2;
   if (live && half > 0) {
     const float pos = (float)positions[n];
-    for (int j = tl; j < half; j += ROPE_GROUP) sincosf(pos * inv_freq[j], &sm_sin[tg][j], &sm_cos[tg][j]);
+    // bfloat16 results: the short routine that the fused decode kernel uses too (error 2e-7), so a key gets the
+    // same rotation whether a portion or a decode step stores it
+    for (int j = tl; j < half; j += ROPE_GROUP) {
+      if (sizeof(T) == 2) ms_sincos_rot(pos * inv_freq[j], &sm_sin[tg][j], &sm_cos[tg][j]);
+      else sincosf(pos * inv_freq[j], &sm_sin[tg][j], &sm_cos[tg][j]);
+    }
   }
   __syncthreads();
   if (!live) return;

@@ -14,26 +14,6 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
-// sin and cos of a rotation angle for bfloat16 results: three-part Cody-Waite reduction by pi/2 (the first
-// two parts have 11 bits, so n * part is exact for |x| < 2^13 * pi/2) and short polynomials on [-pi/4, pi/4];
-// absolute error ~2e-7.  Larger angles take the library routine.
-__device__ __forceinline__ void sincos_rot(float x, float* sn, float* cs) {
-  if (fabsf(x) > 12000.f) { sincosf(x, sn, cs); return; }
-  const float n = rintf(x * 0.636619772367581343f);
-  float r = fmaf(-n, 1.5703125f, x);
-  r = fmaf(-n, 4.837512969970703e-4f, r);
-  r = fmaf(-n, 7.549790126404332e-08f, r);
-  const float r2 = r * r;
-  const float sp = fmaf(r2, fmaf(r2, fmaf(r2, 2.7557314297e-6f, -1.9841270114e-4f), 8.3333337680e-3f), -1.6666667163e-1f);
-  const float s0 = fmaf(r * r2, sp, r);
-  const float cp = fmaf(r2, fmaf(r2, fmaf(r2, 2.4801587642e-5f, -1.3888889225e-3f), 4.1666667908e-2f), -0.5f);
-  const float c0 = fmaf(r2, cp, 1.0f);
-  const int q = (int)n & 3;
-  const float s1 = (q & 1) ? c0 : s0, c1 = (q & 1) ? s0 : c0;
-  *sn = (q & 2) ? -s1 : s1;
-  *cs = ((q + 1) & 2) ? -c1 : c1;
-}
-
 // PAIR8: a block owns one 16-row tile made of 8 rows from the lower half of a head and the 8 rows half a head
 // above them, so a rotary pair (j, j + d/2) lies in two lanes of one token, 32 lanes apart, and is rotated after
 // one exchange between them.  Twice as many blocks as with two whole tiles, each streaming half the weights: for
@@ -167,7 +147,7 @@ qkv_rope_store_kernel(const float* __restrict__ X, size_t ldx, const float* __re
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         float sn, cs;
-        sincos_rot(pos * freq[r], &sn, &cs);
+        ms_sincos_rot(pos * freq[r], &sn, &cs);
         const float x1 = a[r], x2 = b[r];
         a[r] = x1 * cs - x2 * sn;
         b[r] = x2 * cs + x1 * sn;
