@@ -173,9 +173,9 @@ class CacheManager:
                 raise OutOfPages(f"request {req_id!r} needs {n} pages for {new_len} tokens, "
                                  f"{g.allocator.num_free()} are free")
         for i, (g, n) in enumerate(zip(self.groups, needs)):
-            for _ in range(n):
-                g.tables[h.row, h.next_page[i]] = g.allocator.allocate()
-                h.next_page[i] += 1
+            if n:
+                g.tables[h.row, h.next_page[i]:h.next_page[i] + n] = [g.allocator.allocate() for _ in range(n)]
+                h.next_page[i] += n
 
     def advance(self, req_id, computed: int) -> None:
         """``computed`` tokens are stored now; windowed groups give back the pages the window has passed."""

@@ -10,6 +10,7 @@ iff j <= p, and within the window if there is one).
 """
 from __future__ import annotations
 
+import itertools
 from dataclasses import dataclass
 from typing import Hashable, List, Sequence
 
@@ -49,7 +50,7 @@ class BatchBuilder:
             raise ValueError(f"a request would hold {int(ctx_lens.max())} tokens; the cache is made for {m.max_len}")
         q_start = np.zeros(R + 1, dtype=np.int32)
         np.cumsum(lens, out=q_start[1:])
-        token_ids = np.fromiter((t for e in entries for t in e.tokens), dtype=np.int64, count=N)
+        token_ids = np.fromiter(itertools.chain.from_iterable(e.tokens for e in entries), dtype=np.int64, count=N)
         if token_ids.min() < 0 or token_ids.max() >= self.vocab_size:
             bad = int(token_ids[(token_ids < 0) | (token_ids >= self.vocab_size)][0])
             raise ValueError(f"token id {bad} is outside the vocabulary of {self.vocab_size}")
