@@ -102,7 +102,15 @@ def _say_once(key, message: str) -> None:
         print(f"[llm_infrence_engine_amd] {message}", file=sys.stderr, flush=True)
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def _stream():
+    """The current device's current stream as the handle the C entry points take.  Asked for at every launch:
+    the accessors that build no Python object take 0.3 us against 8 us."""
+    if _raw_stream is not None and _raw_device is not None:
+        return _raw_stream(_raw_device())
     return torch.cuda.current_stream().cuda_stream
 
 
@@ -124,8 +132,15 @@ def _check(t: torch.Tensor, name: str, dtype=None, shape=None, contiguous=True):
     if contiguous and not t.is_contiguous():
         raise ValueError(f"{name} must be contiguous")
     if shape is not None:
-        if t.dim() != len(shape) or any(s is not None and s != a for s, a in zip(shape, t.shape)):
-            raise ValueError(f"{name} must have shape {list(shape)}, got {list(t.shape)}")
+        have = t.shape
+        ok = len(have) == len(shape)
+        if ok:
+            for s, a in zip(shape, have):     # a plain loop: this runs several times per kernel launch
+                if s is not None and s != a:
+                    ok = False
+                    break
+        if not ok:
+            raise ValueError(f"{name} must have shape {list(shape)}, got {list(have)}")
 
 
 def _ptr(t: Optional[torch.Tensor]):
