@@ -60,6 +60,7 @@ int ms_gemm_tiled(const void* A, long long lda, const void* W, long long ldw, vo
                   int K, int epilogue, hipStream_t stream);
 void ms_gemm_tiled_force(int tile);
 int ms_gemm_tiled_pays(int M, int N, int K);
+int ms_gemm_tiled_plain_pays(int M, int N, int K);   // the same question for a plain product (epilogue 0)
 
 int ms_gemm_skinny_norm(const float* x, long long ldx, const int* rows, const float* norm_w, float eps, const void* W,
                         long long ldw, const float* bias, void* out, long long ldo, int M, int N, int K, int epilogue,

@@ -269,3 +269,14 @@ extern "C" int ms_gemm_tiled(const void* A, long long lda, const void* W, long l
   GO(2, 4, 4, 2);                  // 128 x 128
 #undef GO
 }
+
+// Whether a plain product of M tokens should run here rather than in the library.  On the GPU the library's
+// kernels are as fast or faster; but a call into the library costs the host 19 us and a call here 5, and a
+// portion of up to about a thousand tokens of a narrow model is over on the GPU before the host has enqueued
+// its 200 launches.  Measured at the 0.5B shape with the q/k/v and o products here: a prompt of up to 512 tokens
+// 3.3 -> 2.7 ms, of 1,024 tokens 3.3 -> 3.15, of 1,536 tokens 3.4 -> 3.5 (so not beyond 1,024); the down projection's
+// long rows take this kernel three times as long as the library and stay there.
+extern "C" int ms_gemm_tiled_plain_pays(int M, int N, int K) {
+  return M > 0 && M <= 1024 && N > 0 && N <= 2048 && K > 0 && K <= 1024 && K % BK == 0;
+}
+

@@ -77,7 +77,8 @@ def _library_mm(a: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype) -> Opt
 
 
 def goes_to_library(a, w: torch.Tensor) -> bool:
-    """Whether ``linear(a, w)`` is the library's product (which comes without a bias epilogue)."""
+    """Whether ``linear(a, w)`` is a many-rows product, the library's or the tiled kernel's: both come without a
+    bias epilogue."""
     return (isinstance(a, torch.Tensor) and a.dtype == torch.bfloat16 and not ops.skinny_ok(a, w)
             and a.shape[0] > ops.SKINNY_MAX_ROWS and a.is_contiguous())
 
@@ -99,6 +100,12 @@ def linear(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None
                 return ops.gemm_skinny(a, w, bias, ops.EPI_STORE, out_dtype=out_dtype)
             except ops.UnsupportedShape:
                 _fell_back(a.shape[0], w.shape[0], w.shape[1], "product")
+        if (a.shape[0] > ops.SKINNY_MAX_ROWS and out_dtype == torch.bfloat16 and bias is None
+                and ops.gemm_tiled_plain_pays(a, w)):
+            try:
+                return ops.gemm_tiled(a, w)     # a short portion of a narrow model: the cheaper launch counts
+            except ops.UnsupportedShape:
+                _fell_back(a.shape[0], w.shape[0], w.shape[1], "tiled product")
         if a.shape[0] > ops.SKINNY_MAX_ROWS and a.is_contiguous():
             out = _library_mm(a, w, out_dtype)
             if out is not None:

@@ -41,6 +41,7 @@ _SIGNATURES = {
     "ms_gemm_tiled": [_c_ptr, _c_ll, _c_ptr, _c_ll, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "ms_gemm_tiled_force": [_c_int],
     "ms_gemm_tiled_pays": [_c_int, _c_int, _c_int],
+    "ms_gemm_tiled_plain_pays": [_c_int, _c_int, _c_int],
     "ms_read_probe_blocks": [],
     "ms_read_probe": [_c_ptr, _c_ll, _c_ptr, _c_ptr],
     "ms_residual_add": [_c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr],
@@ -364,6 +365,14 @@ def gemm_tiled_pays(a: torch.Tensor, w: torch.Tensor) -> bool:
     return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.dim() == 2 and a.is_contiguous()
             and w.is_contiguous() and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
             and bool(_get("ms_gemm_tiled_pays")(a.shape[0], w.shape[0], a.shape[1])))
+
+
+def gemm_tiled_plain_pays(a: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether ``gemm_tiled(a, w)`` is the better way to a plain product than the library's (short portions of a
+    narrow model, where the host's time to enqueue a launch is what counts)."""
+    return (a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.dim() == 2 and a.is_contiguous()
+            and w.is_contiguous() and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
+            and bool(_get("ms_gemm_tiled_plain_pays")(a.shape[0], w.shape[0], a.shape[1])))
 
 
 def gemm_tiled(a: torch.Tensor, w: torch.Tensor, epilogue: int = EPI_STORE) -> torch.Tensor:
