@@ -16,8 +16,7 @@ PRESETS = {
     "7b": {**_QWEN2, "num_hidden_layers": 28, "hidden_size": 3584, "num_attention_heads": 28,
            "num_key_value_heads": 4, "intermediate_size": 18944, "vocab_size": 152064, "tie_word_embeddings": False},
     "32b": {**_QWEN2, "num_hidden_layers": 64, "hidden_size": 5120, "num_attention_heads": 40,
-            "num_key_value_heads": 8, "intermediate_size": 27648, "vocab_size": 152064, "rms_norm_eps": 1e-5,
-            "tie_word_embeddings": False},
+            "num_key_value_heads": 8, "intermediate_size": 27648, "vocab_size": 152064, "tie_word_embeddings": False},
 }
 
 

@@ -30,13 +30,12 @@ from .batch import StepEntry
 
 
 def default_batch_sizes(max_batch: int) -> List[int]:
-    """1, 2, 4, 8, ... up to ``max_batch``, always including it (graph_decode.py:23-30)."""
-    sizes, b = [], 1
-    while b < max_batch:
-        sizes.append(b)
-        b *= 2
-    sizes.append(max_batch)
-    return sizes
+    """The batch-size buckets graphs are captured for: every power of two below ``max_batch`` and ``max_batch``
+    itself, the rule the reference states for its own buckets (src/miniserve/graph_decode.py:23-30;
+    8 -> 1, 2, 4, 8 and 6 -> 1, 2, 4, 6 in its tests/test_cuda_graph.py:45-48)."""
+    if max_batch < 1:
+        raise ValueError("max_batch must be at least 1")
+    return sorted({1 << e for e in range(max_batch.bit_length()) if (1 << e) < max_batch} | {max_batch})
 
 
 class _Bucket:

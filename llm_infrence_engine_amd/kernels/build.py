@@ -5,7 +5,8 @@ is none, printing a line per file so that a first call in a fresh checkout shows
 library sits beside this file; when that folder cannot be written (a read-only checkout) it goes to a
 folder under the system's temporary directory instead, named for the user and for the sources' contents, so
 that a library built from other sources is never picked up there.  Beside the library lies a stamp with the
-hash of the sources it was built from; ``load()`` says so on stderr when the stamp and the sources differ.
+hash of the sources it was built from; when the stamp and the sources differ, ``load()`` says so on stderr and
+builds again instead of loading it.
 There is no fallback: without the library every op raises.
 """
 from __future__ import annotations
@@ -72,6 +73,12 @@ def _fallback_dir() -> Path:
 
 def _stamp_of(lib: Path) -> Path:
     return lib.with_suffix(".stamp")
+
+
+def built_from(lib: Path) -> str:
+    """The hash of the sources ``lib`` was built from, as its stamp says."""
+    stamp = _stamp_of(lib)
+    return stamp.read_text().strip() if stamp.is_file() else "unknown sources"
 
 
 def library_path() -> Path | None:
@@ -177,14 +184,13 @@ def load() -> ctypes.CDLL:
     import torch  # noqa: F401  (its HIP runtime must be the one in the process before ours binds to it)
 
     path = library_path()
+    if path is not None and built_from(path) != source_hash():
+        # a library older than its sources is never loaded: numbers and test results would be those of other code
+        print(f"[kernels] {path} was built from {built_from(path)}, the sources under {CSRC} are {source_hash()}: "
+              f"building it again", file=sys.stderr, flush=True)
+        path = None
     if path is None:
         path = build(verbose=True)
-    else:
-        stamp = _stamp_of(path)
-        built_from = stamp.read_text().strip() if stamp.is_file() else "unknown sources"
-        if built_from != source_hash():
-            print(f"[kernels] {path} was built from {built_from}, the sources under {CSRC} are {source_hash()}: "
-                  f"build it again (llm_infrence_engine_amd.kernels.build.build())", file=sys.stderr, flush=True)
     try:
         _lib = ctypes.CDLL(str(path))
     except OSError as e:

@@ -1,12 +1,14 @@
 """Weights from safetensors files, by tensor name.
 
 Like the reference's loader (src/miniserve/loader.py:41-43) every ``*.safetensors`` file of the folder
-is read and merged by name, with no renaming.  Unlike it (``strict=False`` at loader.py:45 drops
+is read and merged by name, with no renaming; ``model.safetensors.index.json`` is consulted only to name
+the files of a sharded checkpoint that are not in the folder.  Unlike it (``strict=False`` at loader.py:45 drops
 mismatches silently) the names and shapes are checked against what the model's parts ask for, and one
 error lists everything that is missing, unexpected or of the wrong shape or type.
 """
 from __future__ import annotations
 
+import json
 from pathlib import Path
 from typing import Dict, Iterable, List
 
@@ -15,6 +17,7 @@ from safetensors import safe_open
 
 from .spec import TensorSpec
 
+INDEX_NAME = "model.safetensors.index.json"
 _FLOAT_TYPES = {"F32", "BF16", "F16", "F64"}
 _INT_TYPES = {"I8", "I16", "I32", "I64", "U8"}
 
@@ -45,6 +48,11 @@ class CheckpointReader:
         files = sorted(self.folder.glob("*.safetensors"))
         if not files:
             raise WeightsError(self.folder, missing=["(no *.safetensors file in the folder)"])
+        # a sharded checkpoint's index is read only to say which of its files are not there: the tensors
+        # themselves are found by reading every file's own header
+        absent = sorted(self._shards_named_by_index() - {f.name for f in files})
+        if absent:
+            raise WeightsError(self.folder, missing=[f"(file {n}, named by {INDEX_NAME})" for n in absent])
         self._where: Dict[str, Path] = {}
         self._shape: Dict[str, tuple] = {}
         self._dtype: Dict[str, str] = {}
@@ -56,6 +64,16 @@ class CheckpointReader:
                     self._shape[name] = tuple(sl.get_shape())
                     self._dtype[name] = str(sl.get_dtype())
         self._open: Dict[Path, object] = {}
+
+    def _shards_named_by_index(self) -> set:
+        index = self.folder / INDEX_NAME
+        if not index.is_file():
+            return set()
+        try:
+            weight_map = json.loads(index.read_text()).get("weight_map", {})
+        except (ValueError, AttributeError) as e:
+            raise WeightsError(self.folder, missing=[f"({INDEX_NAME} cannot be read: {e})"]) from e
+        return {str(v) for v in weight_map.values()} if isinstance(weight_map, dict) else set()
 
     def names(self) -> List[str]:
         return sorted(self._where)

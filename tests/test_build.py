@@ -36,3 +36,31 @@ def test_no_kernel_spills_registers_to_memory():
     spills = {k: v["scratch"] for k, v in usage.items() if v.get("scratch", 0) > 0}
     assert not spills, f"kernels that spill registers: {spills}"
     assert all(v.get("lds", 0) <= 64 * 1024 for v in usage.values())
+
+
+def test_a_library_older_than_its_sources_is_built_again_not_loaded(tmp_path, monkeypatch):
+    """``load()`` with a stamp that names other sources calls ``build()`` and loads what that returns."""
+    import ctypes
+
+    old = tmp_path / build.LIB_NAME
+    old.write_bytes(b"not a library")
+    build._stamp_of(old).write_text("0123456789ab\n")
+    fresh = tmp_path / "fresh" / build.LIB_NAME
+    calls, loaded = [], []
+
+    def fake_build(verbose=True):
+        calls.append(1)
+        return fresh
+
+    monkeypatch.setattr(build, "_lib", None)
+    monkeypatch.setattr(build, "library_path", lambda: old)
+    monkeypatch.setattr(build, "build", fake_build)
+    monkeypatch.setattr(ctypes, "CDLL", lambda p: loaded.append(p) or object())
+    build.load()
+    assert calls == [1] and loaded == [str(fresh)]
+    # a stamp that names these sources: loaded as it is
+    build._stamp_of(old).write_text(build.source_hash() + "\n")
+    monkeypatch.setattr(build, "_lib", None)
+    build.load()
+    assert calls == [1] and loaded[-1] == str(old)
+    monkeypatch.setattr(build, "_lib", None)

@@ -139,6 +139,32 @@ def test_one_error_lists_missing_unexpected_and_misshapen(tmp_path):
         assert needle in str(err)
 
 
+def test_shards_in_two_files_and_a_shard_the_index_names_but_the_folder_lacks(tmp_path):
+    """Every ``*.safetensors`` file is read and merged by name; the index is only asked which files should be there."""
+    import json
+
+    from safetensors.torch import save_file
+
+    cfg = TINY["A"]
+    w = plain_random_weights(cfg, 0)
+    names = sorted(w)
+    half = len(names) // 2
+    tmp_path.mkdir(exist_ok=True)
+    (tmp_path / "config.json").write_text(json.dumps(cfg))
+    shards = {"model-00001-of-00002.safetensors": names[:half], "model-00002-of-00002.safetensors": names[half:]}
+    for f, ns in shards.items():
+        save_file({n: w[n].contiguous() for n in ns}, str(tmp_path / f))
+    (tmp_path / "model.safetensors.index.json").write_text(
+        json.dumps({"metadata": {}, "weight_map": {n: f for f, ns in shards.items() for n in ns}}))
+    m = Model(config_from_dict(cfg).to_spec())
+    r = CheckpointReader(tmp_path)
+    r.check(m.tensor_specs(), m.ignorable_tensors())
+    assert torch.equal(r.get(names[0]), w[names[0]]) and torch.equal(r.get(names[-1]), w[names[-1]])
+    (tmp_path / "model-00002-of-00002.safetensors").unlink()
+    with pytest.raises(WeightsError, match="model-00002-of-00002.safetensors, named by model.safetensors.index.json"):
+        CheckpointReader(tmp_path)
+
+
 def test_tied_head_ignores_its_own_copy_and_untied_needs_it(tmp_path):
     cfg = TINY["A"]
     w = plain_random_weights(cfg, 0)

@@ -277,3 +277,17 @@ def test_pool_size_from_a_memory_budget():
         EngineConfig(gpu_memory_fraction=1.5)
     assert EngineConfig(dtype="bfloat16").hip_graphs is True and EngineConfig(dtype="float32").hip_graphs is False
     assert EngineConfig(dtype="float32", hip_graphs=True).hip_graphs is True
+
+
+def test_batch_size_buckets_of_the_decode_graphs():
+    """The reference's own vectors (tests/test_cuda_graph.py:45-48) and the edges around them."""
+    from llm_infrence_engine_amd.engine.graph import default_batch_sizes
+
+    assert default_batch_sizes(8) == [1, 2, 4, 8]
+    assert default_batch_sizes(6) == [1, 2, 4, 6]
+    assert default_batch_sizes(1) == [1]
+    assert default_batch_sizes(2) == [1, 2]
+    assert default_batch_sizes(9) == [1, 2, 4, 8, 9]
+    assert default_batch_sizes(64) == [1, 2, 4, 8, 16, 32, 64]
+    with pytest.raises(ValueError):
+        default_batch_sizes(0)
