@@ -24,6 +24,7 @@ class PageAllocator:
             raise ValueError("a pool needs at least one page beside the null page")
         self.num_pages = num_pages
         self.ref = [0] * (num_pages + 1)
+        self.grants = [0] * (num_pages + 1)     # how often each page has been handed out so far
         self._free = deque(range(1, num_pages + 1))
 
     @property
@@ -41,7 +42,12 @@ class PageAllocator:
             raise OutOfPages()
         p = self._free.popleft()
         self.ref[p] = 1
+        self.grants[p] += 1
         return p
+
+    def pages_granted_again(self) -> int:
+        """Pages that have been handed out more than once: a small pool in use shows reuse here."""
+        return sum(1 for n in self.grants if n > 1)
 
     def incref(self, p: int) -> None:
         if p == NULL_PAGE or self.ref[p] <= 0:

@@ -23,7 +23,8 @@ MAX_LIVE = 8          # request rows (the format allows up to four live requests
 
 
 def replay(model_dir, dtype: str, out_dir, max_tokens: int, lines, log=sys.stdout, page_size: int = PAGE_SIZE,
-           device: str = "cuda:0") -> None:
+           device: str = "cuda:0"):
+    """Runs the steps of ``lines`` and returns the runner they ran on (its cache manager tells how pages were used)."""
     import numpy as np
 
     from .batch import StepEntry
@@ -56,6 +57,7 @@ def replay(model_dir, dtype: str, out_dir, max_tokens: int, lines, log=sys.stdou
             if runner.manager.has(rid):
                 runner.free_request(rid)
         print(f"done {step}", file=log, flush=True)
+    return runner
 
 
 def main(argv=None) -> int:

@@ -891,7 +891,7 @@ def _qkv_fused_case(ops, M, nh, nkv, d, K, v_transposed):
 MODEL_PRODUCTS = {
     "0.5b": [(1152, 896), (896, 896), (9728, 896), (896, 4864), (151936, 896)],
     "7b": [(4608, 3584), (3584, 3584), (37888, 3584), (3584, 18944), (152064, 3584)],
-    "32b": [(7168, 5120), (5120, 5120), (55296, 5120), (5120, 27648)],
+    "32b": [(7168, 5120), (5120, 5120), (55296, 5120), (5120, 27648), (152064, 5120)],
 }
 
 

@@ -57,8 +57,18 @@ def run_replay(model_dir, dtype, steps, out, max_tokens, page_size=16):
     from llm_infrence_engine_amd.engine.trace import replay
 
     log = io.StringIO()
-    replay(model_dir, dtype, out, max_tokens, traces.to_lines(steps), log=log, page_size=page_size)
+    runner = replay(model_dir, dtype, out, max_tokens, traces.to_lines(steps), log=log, page_size=page_size)
     assert log.getvalue().split() == [x for st in steps for x in ("done", str(st["step"]))]
+    runner.manager.check_invariants()
+    assert all(g.allocator.num_in_use() == 0 for g in runner.manager.groups), "a finished request kept pages"
+    return runner
+
+
+def assert_pages_were_used_again(runner):
+    """The pool was so small that pages given back by one request were handed out to another."""
+    for g in runner.manager.groups:
+        again = g.allocator.pages_granted_again()
+        assert again > 0, f"no page of a pool of {g.allocator.num_pages} was handed out twice: the trace reuses nothing"
 
 
 def compare(got, want, dtype, requests):
@@ -104,10 +114,13 @@ def test_replay_modes(setup, tmp_path, dtype, mode):
     else:
         max_tokens = up(max(len(t) for t in reqs.values()))
         steps = getattr(traces, mode)(reqs)
-    run_replay(model_dir, dtype, steps, tmp_path, max_tokens, page_size=page)
+    runner = run_replay(model_dir, dtype, steps, tmp_path, max_tokens, page_size=page)
     got = traces.collect(steps, tmp_path, TINY[name]["vocab_size"])
     if mode != "mixed":
         assert len(got) == sum(len(t) for t in reqs.values())
+    else:
+        assert_pages_were_used_again(runner)
+        assert max(len(st["entries"]) for st in steps) >= 3, "the mixed trace never had three requests in a step"
     worst = compare(got, want, dtype, reqs)
     print(f"tiny {name} page {page} {dtype} {mode}: worst error is {worst:.3f} of its bound over {len(got)} places")
 
@@ -122,51 +135,55 @@ def test_baseline_distribution_weights_too(tmp_path_factory, tmp_path):
     compare(traces.collect(steps, tmp_path, 256), want, "float32", reqs)
 
 
-def test_trace_run_program(tmp_path_factory, tmp_path):
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(tmp_path_factory, tmp_path, dtype):
     """bin/trace_run as a user starts it: steps on standard input, files in --out, `done <step>` lines."""
     model_dir = make_model(tmp_path_factory, "B", std=0.15, seed=5)
-    reqs = make_requests(384, [50, 20], seed=9)
+    reqs = make_requests(384, [50, 20, 70], seed=9)
     want = oracle(model_dir, reqs)
     steps = traces.mixed(reqs, 128, seed=1)
     out = tmp_path / "out"
-    r = subprocess.run([sys.executable, str(ROOT / "bin" / "trace_run"), "--model", str(model_dir), "--dtype", "float32",
+    r = subprocess.run([sys.executable, str(ROOT / "bin" / "trace_run"), "--model", str(model_dir), "--dtype", dtype,
                         "--out", str(out), "--max-tokens", "128"], input="\n".join(traces.to_lines(steps)) + "\n",
                        capture_output=True, text=True, timeout=300)
     assert r.returncode == 0, r.stderr
     assert r.stdout.split() == [x for st in steps for x in ("done", str(st["step"]))]
-    compare(traces.collect(steps, out, 384), want, "float32", reqs)
-
-
-HALF_B_WIDTHS = {"architectures": ["Qwen2ForCausalLM"], "num_hidden_layers": 2, "hidden_size": 896, "num_attention_heads": 14,
-                 "num_key_value_heads": 2, "intermediate_size": 4864, "vocab_size": 151936, "rope_theta": 1000000.0,
-                 "rms_norm_eps": 1e-6, "tie_word_embeddings": True}
+    compare(traces.collect(steps, out, 384), want, dtype, reqs)
 
 
 @pytest.fixture(scope="module")
 def half_b(tmp_path_factory):
-    from llm_infrence_engine_amd.config import config_from_dict
+    """All 24 layers of the Qwen2.5-0.5B configuration with random weights, as a model folder."""
+    from llm_infrence_engine_amd.config import config_from_dict, preset
     from llm_infrence_engine_amd.weights import write_random_model
 
     d = tmp_path_factory.mktemp("halfb")
-    write_random_model(d, config_from_dict(HALF_B_WIDTHS), seed=7, dtype="bfloat16", std=0.05)
+    cfg = preset("0.5b")
+    assert cfg["num_hidden_layers"] == 24 and cfg["vocab_size"] == 151936
+    write_random_model(d, config_from_dict(cfg), seed=7, dtype="bfloat16", std=0.05)
     reqs = make_requests(151936, [90, 40, 150], seed=3)
     return d, reqs, oracle(d, reqs)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("mode", ["whole", "bulk_then_single", "changing_portions", "mixed"])
-def test_replay_at_the_widths_of_the_half_billion_model(half_b, tmp_path, dtype, mode):
-    """The layer sizes of Qwen2.5-0.5B (hidden 896, 14 heads over 2 key/value heads of 64, intermediate 4864,
-    vocabulary 151936, tied head) with two layers: the kernels at the sizes they serve, in all four ways of
-    cutting the work."""
+def test_replay_of_the_half_billion_model_at_its_real_depth(half_b, tmp_path, dtype, mode):
+    """Qwen2.5-0.5B as config.json describes it (24 layers, hidden 896, 14 heads over 2 key/value heads of 64,
+    intermediate 4864, vocabulary 151936, tied head) with random weights, in all four ways of cutting the work,
+    as the reference checks its cache paths on the real model (tests/test_kv_cache.py:30-55,
+    tests/test_paged.py:143-166): what 24 layers do to a rounding error is part of the comparison."""
     d, reqs, want = half_b
-    steps = traces.mixed(reqs, 64 * 5, seed=2) if mode == "mixed" else getattr(traces, mode)(reqs)
+    # mixed: room for the two short requests together or the long one alone, so the long one takes over their pages
+    max_tokens = 64 * 3
+    steps = traces.mixed(reqs, max_tokens, seed=2) if mode == "mixed" else getattr(traces, mode)(reqs)
     # logits of every place would be 150 MB a request: ask for the last place of every portion only, and of
     # whole requests every sixteenth place as well
     for st in steps:
         for e in st["entries"]:
             n = len(e["tokens"])
             e["want"] = sorted(set(range(15, n, 16)) | {n - 1}) if mode == "whole" else [n - 1]
-    run_replay(d, dtype, steps, tmp_path, 64 * 5, page_size=16)
+    runner = run_replay(d, dtype, steps, tmp_path, max_tokens, page_size=16)
+    if mode == "mixed":
+        assert_pages_were_used_again(runner)
     worst = compare(traces.collect(steps, tmp_path, 151936), want, dtype, reqs)
-    print(f"0.5B widths {dtype} {mode}: worst error is {worst:.3f} of its bound")
+    print(f"0.5B, 24 layers, {dtype} {mode}: worst error is {worst:.3f} of its bound")

@@ -170,6 +170,100 @@ def test_generation_in_bfloat16_follows_plain(eng, tmp_path, name):
         assert_tokens_follow_plain(w, cfg, p, o.token_ids)
 
 
+@pytest.fixture(scope="module")
+def tiny_d(tmp_path_factory, eng):
+    """Configuration D (head size 64, seven query heads to a key/value head: the matrix-core kernels) in bfloat16."""
+    from llm_infrence_engine_amd.config import config_from_dict
+
+    d = tmp_path_factory.mktemp("tinyD_serving")
+    eng.write_random_model(d, config_from_dict(TINY["D"]), seed=6, dtype="bfloat16", std=0.08)
+    return eng.load_model(str(d), "bfloat16"), P.read_config(d), P.read_weights(d, torch.float64)
+
+
+def test_sampled_tokens_do_not_depend_on_graphs(tiny_d, eng):
+    """bfloat16 with temperature, top-k and top-p: the sampler reads a view of a graph's static logits when graphs
+    are on.  The same seeds give the same tokens with graphs on and off; top_k = 1 is the greedy choice, which
+    with graphs comes from launches of eight steps."""
+    model, cfg, w = tiny_d
+    rng = np.random.default_rng(17)
+    prompts = [[int(t) for t in rng.integers(0, cfg["vocab_size"], n)] for n in (21, 34, 9, 50)]
+    sp = [eng.SamplingParams(max_new_tokens=20, temperature=0.8, top_k=20, top_p=0.9, seed=100 + i) for i in range(4)]
+    kw = dict(block_size=16, max_len=96, max_seqs=4)
+    with_graphs = eng.LLM(model, hip_graphs=True, decode_steps_per_launch=8, **kw)
+    without = eng.LLM(model, hip_graphs=False, **kw)
+    a = with_graphs.generate(prompts, sp)
+    b = without.generate(prompts, sp)
+    assert [o.token_ids for o in a] == [o.token_ids for o in b]
+    assert len({tuple(o.token_ids) for o in a}) == 4
+    assert with_graphs.engine.runner.graphs.launches > 0
+    other = with_graphs.generate(prompts[:1], eng.SamplingParams(max_new_tokens=20, temperature=0.8, top_k=20, top_p=0.9, seed=7))
+    assert other[0].token_ids != a[0].token_ids
+    greedy = with_graphs.generate(prompts, eng.SamplingParams(max_new_tokens=20))
+    assert any(rec.decode_steps == 8 for rec in with_graphs.engine.steps)
+    k1 = with_graphs.generate(prompts, eng.SamplingParams(max_new_tokens=20, temperature=1.3, top_k=1, seed=5))
+    assert [o.token_ids for o in k1] == [o.token_ids for o in greedy]
+    for p, o in zip(prompts, greedy):
+        assert_tokens_follow_plain(w, cfg, p, o.token_ids)
+
+
+def test_preemption_with_graphs_and_eight_steps_to_a_launch(tiny_d, eng):
+    """bfloat16, graphs, eight steps to a launch and ten pages for four requests that need five each: requests are
+    preempted and their prefixes recomputed as prompt portions (other kernels than the decode steps that first
+    produced them); tokens still follow the plain implementation and every page comes back."""
+    model, cfg, w = tiny_d
+    rng = np.random.default_rng(23)
+    prompts = [[int(t) for t in rng.integers(0, cfg["vocab_size"], n)] for n in (30, 27, 31, 25, 29)]
+    e = eng.Engine(model, num_blocks=10, block_size=16, max_seqs=4, max_len=80, max_num_batched_tokens=64,
+                   hip_graphs=True, decode_steps_per_launch=8)
+    reqs = [e.add_request(eng.Request(p, max_new_tokens=40)) for p in prompts]
+    while e.has_work():
+        e.step()
+        e.runner.manager.check_invariants()
+    assert e.preemptions > 0 and any(r.preemptions > 0 for r in reqs)
+    assert any(rec.decode_steps > 1 for rec in e.steps)
+    assert all(g.allocator.num_in_use() == 0 for g in e.runner.manager.groups)
+    assert all(g.allocator.pages_granted_again() > 0 for g in e.runner.manager.groups)
+    for p, r in zip(prompts, reqs):
+        assert len(r.output_ids) == 40 and r.finish_reason == "length"
+        assert_tokens_follow_plain(w, cfg, p, r.output_ids)
+
+
+def test_cancel_that_arrives_inside_a_launch_of_eight_steps(tiny_d, eng):
+    """``cancel`` called while a launch of eight steps is being handed out (from the token callback, as a server's
+    thread would): the request keeps the tokens of that launch, is dropped before the next one, its pages come
+    back, and the others' outputs are what they are without it."""
+    model, cfg, w = tiny_d
+    rng = np.random.default_rng(29)
+    prompts = [[int(t) for t in rng.integers(0, cfg["vocab_size"], n)] for n in (18, 40, 26)]
+    kw = dict(block_size=16, max_seqs=4, max_len=96, hip_graphs=True, decode_steps_per_launch=8)
+    alone = eng.Engine(model, **kw)
+    full = [alone.add_request(eng.Request(p, max_new_tokens=36)) for p in prompts]
+    alone.run_until_idle()
+
+    state = {}
+
+    def on_token(req, tok):
+        if req is state.get("first") and len(req.output_ids) == 12:     # the third token of the second launch
+            state["engine"].cancel(state["victim"])
+
+    e = eng.Engine(model, on_token=on_token, **kw)
+    state["engine"] = e
+    reqs = [e.add_request(eng.Request(p, max_new_tokens=36)) for p in prompts]
+    state["first"], state["victim"] = reqs[0], reqs[1]
+    before = None
+    while e.has_work():
+        rec = e.step()
+        e.runner.manager.check_invariants()
+        if reqs[1].cancelled and before is None:
+            before = (rec.decode_steps, len(reqs[1].output_ids))
+    assert before is not None and before[0] == 8, before
+    assert reqs[1].finish_reason == "abort" and reqs[1] not in e.finished
+    n = len(reqs[1].output_ids)
+    assert n == before[1] and 12 <= n < 36 and reqs[1].output_ids == full[1].output_ids[:n]
+    assert reqs[0].output_ids == full[0].output_ids and reqs[2].output_ids == full[2].output_ids
+    assert all(g.allocator.num_in_use() == 0 for g in e.runner.manager.groups)
+
+
 def test_random_weights_drawn_on_the_device(eng):
     """Seeded draws straight into the kept types: distributions per role, repeatable from the seed, different
     for another seed and from tensor to tensor."""
