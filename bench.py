@@ -73,7 +73,7 @@ def run_decode(eng_mod, model, batch, steps, warmup, vocab, seed, prompt_len=PRO
                        capture_at_start=False)
     # every graph this run can reach, before any timer: all requests stay alive, so the one bucket of ``batch``
     # rows, in both context classes and every launch size (an engine that serves captures all buckets itself)
-    e.runner.graphs.warm_up(e.launch_sizes(), batch_sizes=[batch])
+    e.runner.graphs.warm_up(e.launch_sizes(), batch_sizes=[batch], portion_tokens=())
     for _ in range(batch):
         e.add_request(eng_mod.Request([int(t) for t in rng.integers(0, vocab, prompt_len)],
                                       max_new_tokens=warmup + steps + extra))

@@ -101,20 +101,31 @@ class CacheLayout:
 
 
 class CacheManager:
-    def __init__(self, layout: CacheLayout, page_size: int, num_pages: int, max_requests: int, max_len: int):
-        """``num_pages`` usable pages in every group's pool; a request may hold up to ``max_len`` tokens."""
+    def __init__(self, layout: CacheLayout, page_size: int, num_pages, max_requests: int, max_len: int):
+        """``num_pages`` usable pages in every group's pool, or one number per group (a group that keeps a tenth
+        of the bytes per token may be given a pool of its own size); a request may hold up to ``max_len`` tokens.
+        The block tables have one row per request and a last row that stays all null pages (rows that pad a
+        captured batch read it)."""
         if page_size <= 0 or max_requests <= 0 or max_len <= 0:
             raise ValueError("page_size, max_requests and max_len must be positive")
         self.layout = layout
-        self.page_size, self.num_pages = page_size, num_pages
+        n_groups = len(layout.group_keys)
+        per_group = [int(num_pages)] * n_groups if isinstance(num_pages, int) else [int(n) for n in num_pages]
+        if len(per_group) != n_groups:
+            raise ValueError(f"{len(per_group)} pool sizes for {n_groups} cache groups")
+        self.page_size, self.pages_per_group = page_size, per_group
+        self.num_pages = min(per_group) if per_group else int(num_pages if isinstance(num_pages, int) else 0)
         self.max_requests, self.max_len = max_requests, max_len
         self.max_pages_per_request = -(-max_len // page_size)
+        self.null_row = max_requests
         self.groups: List[CacheGroup] = [
-            CacheGroup(key, runs, PageAllocator(num_pages),
-                       np.zeros((max_requests, self.max_pages_per_request), dtype=np.int32))
-            for key, runs in zip(layout.group_keys, layout.group_runs)]
+            CacheGroup(key, runs, PageAllocator(n),
+                       np.zeros((max_requests + 1, self.max_pages_per_request), dtype=np.int32))
+            for key, runs, n in zip(layout.group_keys, layout.group_runs, per_group)]
         self._free_rows = list(range(max_requests - 1, -1, -1))
         self._held: Dict[Hashable, _Held] = {}
+        # table entries that changed since ``take_updates`` was last called, per group: flat index -> page
+        self._changed: List[Dict[int, int]] = [{} for _ in self.groups]
 
     # ------------------------------------------------------------------ requests
     def has(self, req_id) -> bool:
@@ -143,12 +154,25 @@ class CacheManager:
     def computed(self, req_id) -> int:
         return self._held[req_id].computed
 
+    def capacity_tokens(self) -> int:
+        """Tokens one request could hold if it had the smallest pool to itself."""
+        return min(self.max_len, self.num_pages * self.page_size) if self.groups else self.max_len
+
     # ------------------------------------------------------------------ pages
     def _first_needed(self, g: CacheGroup, computed: int) -> int:
         """First logical page a query at position >= ``computed`` can still see."""
         if g.key.window is None:
             return 0
         return max(0, computed - g.key.window + 1) // self.page_size
+
+    def _set(self, gi: int, row: int, first: int, pages) -> None:
+        """Table entries ``first``.. of a row take new values; the change is noted for the device's copy."""
+        g = self.groups[gi]
+        g.tables[row, first:first + len(pages)] = pages
+        base = row * self.max_pages_per_request + first
+        changed = self._changed[gi]
+        for k, p in enumerate(pages):
+            changed[base + k] = int(p)
 
     def pages_to_grow(self, req_id, new_len: int) -> List[int]:
         """Pages each group must hand out so that the request can hold ``new_len`` tokens."""
@@ -162,6 +186,16 @@ class CacheManager:
             return False
         return all(g.allocator.num_free() >= n + reserve for g, n in zip(self.groups, self.pages_to_grow(req_id, new_len)))
 
+    def tokens_that_fit(self, req_id, reserve: int = 0) -> int:
+        """How many more tokens than it has stored the request could hold with the free pages of every group,
+        ``reserve`` of them left alone."""
+        h = self._held[req_id]
+        fit = self.max_len - h.computed
+        for i, g in enumerate(self.groups):
+            room = (h.next_page[i] + max(0, g.allocator.num_free() - reserve)) * self.page_size - h.computed
+            fit = min(fit, room)
+        return fit
+
     def grow(self, req_id, new_len: int) -> None:
         """Allocate pages in every group for tokens up to ``new_len``; all groups or none."""
         if new_len > self.max_len:
@@ -174,7 +208,7 @@ class CacheManager:
                                  f"{g.allocator.num_free()} are free")
         for i, (g, n) in enumerate(zip(self.groups, needs)):
             if n:
-                g.tables[h.row, h.next_page[i]:h.next_page[i] + n] = [g.allocator.allocate() for _ in range(n)]
+                self._set(i, h.row, h.next_page[i], [g.allocator.allocate() for _ in range(n)])
                 h.next_page[i] += n
 
     def advance(self, req_id, computed: int) -> None:
@@ -187,10 +221,11 @@ class CacheManager:
         h.computed = computed
         for i, g in enumerate(self.groups):
             first = min(self._first_needed(g, computed), h.next_page[i])
-            for p in range(h.first_live[i], first):
-                g.allocator.decref(int(g.tables[h.row, p]))
-                g.tables[h.row, p] = NULL_PAGE
-            h.first_live[i] = max(h.first_live[i], first)
+            if first > h.first_live[i]:
+                for p in range(h.first_live[i], first):
+                    g.allocator.decref(int(g.tables[h.row, p]))
+                self._set(i, h.row, h.first_live[i], [NULL_PAGE] * (first - h.first_live[i]))
+                h.first_live[i] = first
 
     def free(self, req_id) -> None:
         """Give back everything the request holds."""
@@ -198,7 +233,8 @@ class CacheManager:
         for i, g in enumerate(self.groups):
             for p in range(h.first_live[i], h.next_page[i]):
                 g.allocator.decref(int(g.tables[h.row, p]))
-            g.tables[h.row, :h.next_page[i]] = NULL_PAGE
+            if h.next_page[i] > h.first_live[i]:
+                self._set(i, h.row, h.first_live[i], [NULL_PAGE] * (h.next_page[i] - h.first_live[i]))
         self._free_rows.append(h.row)
 
     def pages_held(self, req_id) -> List[List[int]]:
@@ -207,6 +243,21 @@ class CacheManager:
 
     def num_free_pages(self) -> List[int]:
         return [g.allocator.num_free() for g in self.groups]
+
+    # ------------------------------------------------------------------ the device's copy of the tables
+    def pending_updates(self) -> int:
+        """The most entries any group's table has changed by since ``take_updates``."""
+        return max((len(c) for c in self._changed), default=0)
+
+    def take_updates(self) -> List[Tuple[np.ndarray, np.ndarray]]:
+        """Per group (flat indices into the [rows, pages] table, their new values), each index once, and forget
+        them: applied to a copy of the tables in this order of calls, the copy equals ``groups[g].tables``."""
+        out = []
+        for c in self._changed:
+            out.append((np.fromiter(c.keys(), dtype=np.int32, count=len(c)),
+                        np.fromiter(c.values(), dtype=np.int32, count=len(c))))
+            c.clear()
+        return out
 
     # ------------------------------------------------------------------ accounting
     def bytes_per_token(self, bytes_per_value: int) -> int:
@@ -227,7 +278,7 @@ class CacheManager:
                 assert (g.tables[h.row, h.next_page[i]:] == NULL_PAGE).all(), "the table holds a page beyond its end"
                 for p in live:
                     owners[int(p)] = owners.get(int(p), 0) + 1
-            for r in self._free_rows:
+            for r in self._free_rows + [self.null_row]:
                 assert (g.tables[r] == NULL_PAGE).all(), "a free row still holds pages"
             for p in range(1, g.allocator.num_pages + 1):
                 assert g.allocator.ref[p] == owners.get(p, 0), \

@@ -24,6 +24,9 @@ class EngineConfig:
     max_prefill_chunk: Optional[int] = None  # largest portion of one prompt in one step (None: the budget)
     hip_graphs: Optional[bool] = None  # replay decode-only steps from captured graphs; None: when serving in bfloat16
     decode_steps_per_launch: int = 1   # decode steps queued in one graph launch while everybody decodes greedily
+    graph_portion_tokens: Optional[int] = None  # with hip_graphs: steps with prompt portions of up to this many tokens
+                                       # are replayed from graphs too (None: as far as the host would be what the
+                                       # step waits for; 0: decode steps only)
     device: str = "cuda:0"
 
     def __post_init__(self):
@@ -45,17 +48,19 @@ class EngineConfig:
         return -(-self.max_len // self.block_size)
 
     def resolved_num_blocks(self, bytes_per_token: Optional[int] = None, device_total_bytes: Optional[int] = None,
-                            device_used_bytes: int = 0) -> int:
+                            device_used_bytes: int = 0, other_bytes: int = 0) -> int:
         """Pages of every group's pool.  Given by hand, or what ``max_seqs`` requests of ``max_len`` tokens can
         fill (the reference's default is the same product, src/miniserve/server.py:145); with
         ``gpu_memory_fraction`` no more than fits into that share of the device's memory beside what is held
-        already (the weights), counted in bytes as the reference counts its pool (src/miniserve/paged.py:162-168)."""
+        already (``device_used_bytes``: the weights, and whatever the allocator keeps cached) and what the engine
+        will take beside the pages (``other_bytes``: per-request state, the static logits and activations of the
+        captured graphs), counted in bytes as the reference counts its pool (src/miniserve/paged.py:162-168)."""
         if self.num_blocks is not None:
             return self.num_blocks
         most = self.max_seqs * self.pages_per_request
         if self.gpu_memory_fraction is None or not bytes_per_token or not device_total_bytes:
             return most
-        budget = int(self.gpu_memory_fraction * device_total_bytes) - device_used_bytes
+        budget = int(self.gpu_memory_fraction * device_total_bytes) - device_used_bytes - other_bytes
         pages = budget // (bytes_per_token * self.block_size) - 1          # one of them is the null page
         if pages < self.pages_per_request:
             raise ValueError(f"{self.gpu_memory_fraction:.2f} of the device's memory leaves {max(budget, 0)} bytes for the "

@@ -8,33 +8,51 @@ architecture's configuration again; the parts are built from ``PartSpec`` alone.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
+from types import MappingProxyType
 from typing import Any, Mapping, Optional, Tuple
 
 
-@dataclass(frozen=True)
+@dataclass(frozen=True, eq=True)
 class PartSpec:
     """One part: ``kind`` is its name in the part registry, ``prefix`` the beginning of its tensor
-    names in the checkpoint, ``params`` its sizes and constants."""
+    names in the checkpoint, ``params`` its sizes and constants (kept read-only)."""
 
     kind: str
     prefix: str = ""
     params: Mapping[str, Any] = field(default_factory=dict)
 
+    def __post_init__(self):
+        object.__setattr__(self, "params", MappingProxyType(dict(self.params)))
 
-@dataclass(frozen=True)
+    def __hash__(self):
+        return hash((self.kind, self.prefix, tuple(sorted((k, repr(v)) for k, v in self.params.items()))))
+
+
+@dataclass(frozen=True, eq=True)
 class LayerSpec:
     """One layer: an arrangement (``block``, a name in the block registry) and the parts it is given, by the
-    names the arrangement takes.  ``pre_norm_residual`` takes ``mixer``, ``feed_forward``, ``mixer_norm``,
-    ``feed_forward_norm`` and optionally ``position`` (the mixer's position encoding); another arrangement
-    may take other parts (more norms, no feed-forward, two mixers)."""
+    names the arrangement takes (kept read-only).  ``pre_norm_residual`` takes ``mixer``, ``feed_forward``,
+    ``mixer_norm``, ``feed_forward_norm`` and optionally ``position`` (the mixer's position encoding); another
+    arrangement may take other parts (more norms, no feed-forward, two mixers).  ``layer.mixer`` is the part of
+    that name; a name the layer was not given raises (``layer.parts.get(name)`` asks without raising)."""
 
     block: str
     parts: Mapping[str, PartSpec]
 
-    def __getattr__(self, name):      # layer.mixer, layer.position, ...: the named part, None if it has none
+    def __post_init__(self):
+        object.__setattr__(self, "parts", MappingProxyType(dict(self.parts)))
+
+    def __hash__(self):
+        return hash((self.block, tuple(sorted(self.parts.items(), key=lambda kv: kv[0]))))
+
+    def __getattr__(self, name):
         if name.startswith("__") or name in ("block", "parts"):
             raise AttributeError(name)
-        return self.parts.get(name)
+        try:
+            return self.parts[name]
+        except KeyError:
+            raise AttributeError(f"this {self.block} layer has no part named {name!r}; it has "
+                                 f"{', '.join(sorted(self.parts))}") from None
 
 
 def layer(block: str, **parts: Optional[PartSpec]) -> LayerSpec:

@@ -14,10 +14,22 @@ int ms_rms_norm(float* x, const void* delta, int delta_dtype, int n_partials, lo
 
 int ms_bias_add(void* x, const float* bias, int n_rows, int width, int dtype, hipStream_t stream);
 
-// tables / slots: host arrays of n_groups device pointers (block table int32 [rows, table_stride], slot mapping int32 [rows])
+// tables / slots: host arrays of n_groups device pointers (block table int32 [table rows, table_stride], slot
+// mapping int32 [n_rows]); table_rows int32 [n_rows]: the table's row of each row of the batch.  At most
+// ms_max_cache_groups() groups.
+int ms_max_cache_groups();
 int ms_decode_advance(const int* prev_tokens, int* token_ids, int* positions, int* context_lens, const int* n_live,
-                      const int* const* tables, int* const* slots, int n_groups, int table_stride, int page_size,
-                      int n_rows, hipStream_t stream);
+                      const int* table_rows, const int* const* tables, int* const* slots, int n_groups,
+                      int table_stride, int page_size, int n_rows, hipStream_t stream);
+
+// Block tables kept on the device: tables[g][index[g][i]] = value[g][i] for i < counts[g] (counts: device ints),
+// every index at most once per group; max_updates bounds counts, table_elems bounds the indices.
+int ms_table_update(int* const* tables, const int* const* index, const int* const* value, const int* counts,
+                    int n_groups, int max_updates, long long table_elems, hipStream_t stream);
+
+// rows[i] of a [n, row_bytes] tensor become zero (row_bytes a multiple of 4), i < n_rows; `count` (null: n_rows)
+// is a device int that may ask for fewer.
+int ms_zero_rows(void* base, long long row_bytes, const int* rows, const int* count, int n_rows, hipStream_t stream);
 
 // A plain streaming read of `bytes` for bandwidth measurements; sink: unsigned [ms_read_probe_blocks()].
 int ms_read_probe_blocks();
@@ -74,7 +86,8 @@ int ms_qkv_rope_store(const float* x, long long ldx, const float* norm_w, float 
                       int page_size, int v_transposed, hipStream_t stream);
 
 int ms_paged_attention_generic(const void* q, long long q_stride, const void* k_pages, const void* v_pages,
-                               const int* block_table, int table_stride, const int* token_req, const int* positions,
+                               const int* block_table, int table_stride, const int* table_rows,
+                               const int* n_live_tokens, const int* token_req, const int* positions,
                                void* out, long long out_stride, int n_tokens, int num_heads, int num_kv_heads,
                                int head_dim, int page_size, long long num_pages, float scale, int window,
                                int v_transposed, int dtype, hipStream_t stream);
@@ -82,13 +95,15 @@ int ms_paged_attention_generic(const void* q, long long q_stride, const void* k_
 int ms_attention_mfma_supported(int head_dim, int page_size);
 
 int ms_paged_attention_mfma(const void* q, long long q_stride, const void* k_pages, const void* vt_pages,
-                            const int* block_table, int table_stride, const int* q_start, const int* context_lens,
-                            void* out, long long out_stride, int n_requests, int max_q_len, int num_heads,
-                            int num_kv_heads, int head_dim, int page_size, float scale, int window, hipStream_t stream);
+                            const int* block_table, int table_stride, const int* table_rows, const int* q_start,
+                            const int* context_lens, void* out, long long out_stride, int n_requests, int n_tokens,
+                            int max_q_len, int num_heads, int num_kv_heads, int head_dim, int page_size, float scale,
+                            int window, hipStream_t stream);
 
 int ms_paged_attention_mfma_decode(const void* q, long long q_stride, const void* k_pages, const void* vt_pages,
-                                   const int* block_table, int table_stride, const int* q_start,
-                                   const int* context_lens, void* out, long long out_stride, void* part_o,
+                                   const int* block_table, int table_stride, const int* table_rows,
+                                   const int* q_start, const int* context_lens, void* out, long long out_stride,
+                                   void* part_o,
                                    void* part_ml, int n_requests, int num_heads, int num_kv_heads, int head_dim,
                                    int page_size, float scale, int window, int min_blocks, int n_splits,
                                    hipStream_t stream);

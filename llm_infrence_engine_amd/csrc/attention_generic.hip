@@ -3,6 +3,8 @@
 // maximum, exponentials, their sum and the weighted sum of values are all float.  It reads keys and
 // values in place through the request's block table and never reads a key beyond the token's own
 // position, so what a reused page still holds from an earlier request cannot reach the result.
+// block_table int32 [rows, table_stride]; request r of the step has row table_rows[r] (null: row r).
+// n_live_tokens (null: all): a device int; tokens from that index on belong to no request and are skipped.
 // This is the attention of the 32-bit path and the any-shape fallback of the bfloat16 path.
 #include "common.h"
 #include "api.h"
@@ -16,6 +18,7 @@ template <typename T>
 __global__ void __launch_bounds__(WAVES * MS_WAVE)
 paged_attention_generic_kernel(const T* __restrict__ q, size_t q_stride, const T* __restrict__ k_pages,
                                const T* __restrict__ v_pages, const int* __restrict__ block_table, int table_stride,
+                               const int* __restrict__ table_rows, const int* __restrict__ n_live_tokens,
                                const int* __restrict__ token_req, const int* __restrict__ positions,
                                T* __restrict__ out, size_t out_stride, int n_tokens, int nh, int nkv, int d,
                                int page_size, float scale, int window, int v_transposed) {
@@ -24,9 +27,11 @@ paged_attention_generic_kernel(const T* __restrict__ q, size_t q_stride, const T
   const long long item = (long long)blockIdx.x * WAVES + wave;
   if (item >= (long long)n_tokens * nh) return;  // whole wave leaves; no block-wide barrier below
   const int n = (int)(item / nh), h = (int)(item - (long long)n * nh);
+  if (n_live_tokens && n >= *n_live_tokens) return;   // a token that pads a captured batch belongs to no request
   const int kvh = h / (nh / nkv);
   const int pos = positions[n];
-  const int* table = block_table + (size_t)token_req[n] * table_stride;
+  const int req = token_req[n];
+  const int* table = block_table + (size_t)(table_rows ? table_rows[req] : req) * table_stride;
 
   const T* qp = q + (size_t)n * q_stride + (size_t)h * d;
   for (int i = lane; i < d; i += MS_WAVE) qs[wave][i] = to_float(qp[i]) * scale;
@@ -94,7 +99,8 @@ paged_attention_generic_kernel(const T* __restrict__ q, size_t q_stride, const T
 }  // namespace
 
 extern "C" int ms_paged_attention_generic(const void* q, long long q_stride, const void* k_pages, const void* v_pages,
-                                          const int* block_table, int table_stride, const int* token_req,
+                                          const int* block_table, int table_stride, const int* table_rows,
+                                          const int* n_live_tokens, const int* token_req,
                                           const int* positions, void* out, long long out_stride, int n_tokens,
                                           int num_heads, int num_kv_heads, int head_dim, int page_size,
                                           long long num_pages, float scale, int window, int v_transposed,
@@ -106,7 +112,7 @@ extern "C" int ms_paged_attention_generic(const void* q, long long q_stride, con
   if (num_pages * num_kv_heads * page_size >= (1ll << 31)) return MS_UNSUPPORTED;  // row index is an int
   const long long items = (long long)n_tokens * num_heads;
   dim3 grid((unsigned)((items + WAVES - 1) / WAVES)), block(WAVES * MS_WAVE);
-#define LAUNCH(T) paged_attention_generic_kernel<T><<<grid, block, 0, stream>>>((const T*)q, (size_t)q_stride, (const T*)k_pages, (const T*)v_pages, block_table, table_stride, token_req, positions, (T*)out, (size_t)out_stride, n_tokens, num_heads, num_kv_heads, head_dim, page_size, scale, window, v_transposed)
+#define LAUNCH(T) paged_attention_generic_kernel<T><<<grid, block, 0, stream>>>((const T*)q, (size_t)q_stride, (const T*)k_pages, (const T*)v_pages, block_table, table_stride, table_rows, n_live_tokens, token_req, positions, (T*)out, (size_t)out_stride, n_tokens, num_heads, num_kv_heads, head_dim, page_size, scale, window, v_transposed)
   if (dtype == MS_F32) LAUNCH(float);
   else if (dtype == MS_BF16) LAUNCH(bf16);
   else return MS_BAD_ARG;

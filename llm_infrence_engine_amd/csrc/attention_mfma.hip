@@ -29,6 +29,7 @@
 // write unnormalised partial results, and a second kernel combines them).
 #include "common.h"
 #include "api.h"
+#include <algorithm>
 
 namespace {
 
@@ -117,12 +118,13 @@ template <int D, int NT, int WAVES, bool SPLIT, int VS>
 __global__ void __launch_bounds__(WAVES * MS_WAVE, (NT > 1 ? 2 : 1))
 attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* __restrict__ k_pages,
                       const bf16* __restrict__ vt_pages, const int* __restrict__ block_table, int table_stride,
-                      const int* __restrict__ q_start, const int* __restrict__ context_lens,
-                      bf16* __restrict__ out, size_t out_stride, float* __restrict__ part_o,
-                      float* __restrict__ part_ml, int nh, int nkv, int page_size, int page_shift,
-                      float scale_log2e, int window, int min_blocks, int n_splits) {
-  // SPLIT: min_blocks and n_splits say how a request's key blocks are spread; else min_blocks != 0 asks for
-  // the order of tiles in which a long tile's companion on its CU is a short one (see below)
+                      const int* __restrict__ table_rows, const int* __restrict__ q_start,
+                      const int* __restrict__ context_lens, bf16* __restrict__ out, size_t out_stride,
+                      float* __restrict__ part_o, float* __restrict__ part_ml, int nh, int nkv, int page_size,
+                      int page_shift, float scale_log2e, int window, int min_blocks, int n_splits) {
+  // SPLIT: min_blocks and n_splits say how a request's key blocks are spread.  Else min_blocks != 0 asks for
+  // the order of tiles in which a long tile's companion on its CU is a short one (see below), and n_splits is
+  // the number of requests whose tiles the grid's second dimension runs over (0: one tile to a request)
   __shared__ float sm_m[WAVES][NT][16], sm_l[WAVES][NT][16];
   static_assert(VS == 1 || (NT == 1 && !SPLIT), "only narrow tiles of the general shape share their dims out");
   static_assert((D / 16) % VS == 0, "whole tiles of 16 dims to a block");
@@ -131,13 +133,56 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
   const int lane = threadIdx.x & (MS_WAVE - 1);
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / MS_WAVE);   // the same for the whole wave
   const int col16 = lane & 15, kq = lane >> 4;
-  // general shape: grid (kv heads, requests, tiles): blocks are handed out with the kv head running fastest and
-  // the tile slowest; split shape: grid (splits, kv heads, requests)
-  const int r = SPLIT ? blockIdx.z : blockIdx.y, g = SPLIT ? blockIdx.y : blockIdx.x;
-  const int bx = SPLIT ? blockIdx.x : blockIdx.z, nbx = SPLIT ? gridDim.x : gridDim.z;
+  // general shape: grid (kv heads, column tiles of the whole step, blocks that share a tile's dims): blocks are
+  // handed out with the kv head running fastest; split shape: grid (splits, kv heads, requests)
+  const int g = SPLIT ? blockIdx.y : blockIdx.x;
+  const int bx = SPLIT ? blockIdx.x : blockIdx.z;
   const int rep = nh / nkv;
   const PageGeom pg = {page_size, page_shift};
-  const int* table = block_table + (size_t)r * table_stride;
+  // Which request, and which of its tiles.  A request owns ceil(columns / tile width) tiles, requests in order,
+  // so the launch needs to know only how many tokens and requests a step has, not how the tokens are dealt out
+  // (a captured graph serves every mix).  The waves of a block find their place alike: a lane per request
+  // works out its tiles, a prefix sum over the wave and a vote say where this block's tile falls.
+  int r, rank, n_tiles;
+  if (SPLIT) {
+    r = blockIdx.z; rank = 0; n_tiles = 1;
+  } else if (n_splits == 0) {
+    r = blockIdx.y; rank = 0; n_tiles = 1;
+  } else if (n_splits == 1) {
+    r = 0; rank = blockIdx.y;
+    n_tiles = ((q_start[1] - q_start[0]) * rep + 16 * NT - 1) / (16 * NT);
+    if (rank >= n_tiles) return;
+  } else {
+    const int flat = blockIdx.y;
+    int before = 0;
+    r = -1; rank = 0; n_tiles = 0;
+    for (int base = 0; base < n_splits; base += MS_WAVE) {
+      const int i = base + lane;
+      int mine = 0;
+      if (i < n_splits) mine = ((q_start[i + 1] - q_start[i]) * rep + 16 * NT - 1) / (16 * NT);
+      int upto = mine;   // tiles of the requests base..i
+#pragma unroll
+      for (int o = 1; o < MS_WAVE; o <<= 1) {
+        const int v = __shfl_up(upto, o, MS_WAVE);
+        if (lane >= o) upto += v;
+      }
+      const unsigned long long hit = __builtin_amdgcn_ballot_w64(flat < before + upto);
+      if (hit) {
+        const int first = __builtin_ctzll(hit);
+        r = base + first;
+        n_tiles = __shfl(mine, first, MS_WAVE);
+        rank = flat - before - (__shfl(upto, first, MS_WAVE) - n_tiles);
+        break;
+      }
+      before += __shfl(upto, MS_WAVE - 1, MS_WAVE);
+    }
+    if (r < 0) return;   // the grid has room for a partial tile of every request; this block is surplus
+    r = __builtin_amdgcn_readfirstlane(r);
+    rank = __builtin_amdgcn_readfirstlane(rank);
+    n_tiles = __builtin_amdgcn_readfirstlane(n_tiles);
+  }
+  const int row = table_rows ? table_rows[r] : r;
+  const int* table = block_table + (size_t)row * table_stride;
   // Without a window a wave's first key block is known before the request's lengths are: ask for its page
   // ids at once, so that they travel together with the lengths instead of after them.
   int first_pages[2] = {0, 0};
@@ -155,8 +200,7 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
   // all blocks fit on the chip at once (two to a CU), only the later half goes first, latest tile first, and
   // then the earlier half, earliest first: blocks that start one round of the chip apart tend to share a CU, and
   // so a long tile's companion is a short one that soon leaves the SIMDs to it (2,048 tokens: 34.0 -> 29.4 us).
-  const int rank = VS > 1 ? bx / VS : bx, n_tiles = VS > 1 ? nbx / VS : nbx;
-  const int dim0 = VS > 1 ? (bx % VS) * CT * 16 : 0;   // the first of this block's output dims
+  const int dim0 = VS > 1 ? bx * CT * 16 : 0;   // the first of this block's output dims
   const int half = (!SPLIT && min_blocks) ? (n_tiles + 1) / 2 : n_tiles;
   const int tile = rank < half ? n_tiles - 1 - rank : rank - half;
   const int c0 = SPLIT ? 0 : tile * 16 * NT;
@@ -427,6 +471,7 @@ attention_combine_kernel(const float* __restrict__ part_o, const float* __restri
                          int n_splits) {
   __shared__ float sm_m[COMBINE_MAX_SPLITS], sm_w[COMBINE_MAX_SPLITS];
   const int r = blockIdx.x / nh, h = blockIdx.x % nh;
+  if (q_start[r + 1] == q_start[r]) return;   // a row that pads a captured batch: no token, nothing to write
   const int key_hi = context_lens[r] - 1;
   const int key_lo = window > 0 ? max(0, key_hi - window + 1) : 0;
   const int blocks = key_hi / 32 + 1 - key_lo / 32;
@@ -469,24 +514,29 @@ inline int page_shift_of(int page_size) {   // log2 of a power of two, else -1
 
 template <int D, int NT, int WAVES, int VS>
 int launch_general(const bf16* q, size_t q_stride, const bf16* k, const bf16* vt, const int* table, int table_stride,
-                   const int* q_start, const int* ctx, bf16* out, size_t out_stride, int n_requests, int max_q_len,
-                   int nh, int nkv, int page_size, float scale, int window, hipStream_t stream) {
+                   const int* table_rows, const int* q_start, const int* ctx, bf16* out, size_t out_stride,
+                   int n_requests, int n_tokens, int max_q_len, int nh, int nkv, int page_size, float scale,
+                   int window, hipStream_t stream) {
   const int rep = nh / nkv;
-  const int tiles = (max_q_len * rep + 16 * NT - 1) / (16 * NT);
-  if ((long long)tiles * VS > 65535) return MS_UNSUPPORTED;   // grid.z
-  const int pair_order = (long long)tiles * VS * nkv * n_requests <= 2LL * ms_compute_units() ? 1 : 0;
-  dim3 grid(nkv, n_requests, tiles * VS), block(WAVES * MS_WAVE);
-  attention_mfma_kernel<D, NT, WAVES, false, VS><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, q_start, ctx, out, out_stride, nullptr, nullptr, nh, nkv, page_size, page_shift_of(page_size), scale * 1.4426950408889634f, window, pair_order, 0);
+  const long long per_request = ((long long)max_q_len * rep + 16 * NT - 1) / (16 * NT);
+  // every request may end in a partial tile; no step has more tiles than if each request were the longest
+  long long tiles = (long long)n_tokens * rep / (16 * NT) + n_requests;
+  if (tiles > per_request * n_requests) tiles = per_request * n_requests;
+  if (tiles > 65535) return MS_UNSUPPORTED;   // grid.y
+  const int pair_order = tiles * VS * nkv <= 2LL * ms_compute_units() ? 1 : 0;
+  const int scan = per_request == 1 ? 0 : n_requests;   // one tile to a request: the tile's index is the request's
+  dim3 grid(nkv, (unsigned)tiles, VS), block(WAVES * MS_WAVE);
+  attention_mfma_kernel<D, NT, WAVES, false, VS><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, table_rows, q_start, ctx, out, out_stride, nullptr, nullptr, nh, nkv, page_size, page_shift_of(page_size), scale * 1.4426950408889634f, window, pair_order, scan);
   return ms_launch_status();
 }
 
 template <int D>
 int launch_split(const bf16* q, size_t q_stride, const bf16* k, const bf16* vt, const int* table, int table_stride,
-                 const int* q_start, const int* ctx, bf16* out, size_t out_stride, float* part_o, float* part_ml,
+                 const int* table_rows, const int* q_start, const int* ctx, bf16* out, size_t out_stride, float* part_o, float* part_ml,
                  int n_requests, int nh, int nkv, int page_size, float scale, int window, int min_blocks,
                  int n_splits, hipStream_t stream) {
   dim3 grid(n_splits, nkv, n_requests), block(4 * MS_WAVE);
-  attention_mfma_kernel<D, 1, 4, true, 1><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, q_start, ctx, out, out_stride, part_o, part_ml, nh, nkv, page_size, page_shift_of(page_size), scale * 1.4426950408889634f, window, min_blocks, n_splits);
+  attention_mfma_kernel<D, 1, 4, true, 1><<<grid, block, 0, stream>>>(q, q_stride, k, vt, table, table_stride, table_rows, q_start, ctx, out, out_stride, part_o, part_ml, nh, nkv, page_size, page_shift_of(page_size), scale * 1.4426950408889634f, window, min_blocks, n_splits);
   attention_combine_kernel<D><<<dim3(n_requests * nh), dim3(D < 64 ? 64 : D), 0, stream>>>(part_o, part_ml, q_start, ctx, out, out_stride, nh, window, min_blocks, n_splits);
   return ms_launch_status();
 }
@@ -508,20 +558,23 @@ extern "C" int ms_attention_mfma_supported(int head_dim, int page_size) {
 }
 
 // General shape.  q [N, >= nh*d] bfloat16 (row stride q_stride), k_pages [P, nkv, page_size, d],
-// vt_pages [P, nkv, d, page_size], block_table int32 [R, table_stride], q_start int32 [R + 1],
-// context_lens int32 [R] (keys held after this step), out [N, nh*d] (row stride out_stride).
+// vt_pages [P, nkv, d, page_size], block_table int32 [rows, table_stride], table_rows int32 [R] (the table's row
+// of each request; null: request r has row r), q_start int32 [R + 1], context_lens int32 [R] (keys held after
+// this step), out [N, nh*d] (row stride out_stride).  n_tokens = q_start[R] or more, max_q_len the longest
+// portion or more: the launch is sized by these two and n_requests alone, so tokens beyond q_start[R] and
+// requests without tokens cost a block that leaves at once.
 extern "C" int ms_paged_attention_mfma(const void* q, long long q_stride, const void* k_pages, const void* vt_pages,
-                                       const int* block_table, int table_stride, const int* q_start,
-                                       const int* context_lens, void* out, long long out_stride, int n_requests,
-                                       int max_q_len, int num_heads, int num_kv_heads, int head_dim, int page_size,
-                                       float scale, int window, hipStream_t stream) {
-  if (n_requests <= 0 || max_q_len <= 0) return MS_OK;
+                                       const int* block_table, int table_stride, const int* table_rows,
+                                       const int* q_start, const int* context_lens, void* out, long long out_stride,
+                                       int n_requests, int n_tokens, int max_q_len, int num_heads, int num_kv_heads,
+                                       int head_dim, int page_size, float scale, int window, hipStream_t stream) {
+  if (n_requests <= 0 || max_q_len <= 0 || n_tokens <= 0) return MS_OK;
   if (num_heads <= 0 || num_kv_heads <= 0 || num_heads % num_kv_heads || table_stride <= 0) return MS_BAD_ARG;
   if (!(scale > 0.f)) return MS_BAD_ARG;   // maxima are taken of the raw scores
   if (!ms_attention_mfma_supported(head_dim, page_size)) return MS_UNSUPPORTED;
   if (q_stride % 8 || out_stride % 4 || ((uintptr_t)q % 16) || ((uintptr_t)out % 8)) return MS_UNSUPPORTED;
   if (n_requests > 65535 || num_kv_heads > 65535) return MS_UNSUPPORTED;
-#define GO(D, NT, WV, VS) return launch_general<D, NT, WV, VS>((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)vt_pages, block_table, table_stride, q_start, context_lens, (bf16*)out, out_stride, n_requests, max_q_len, num_heads, num_kv_heads, page_size, scale, window, stream)
+#define GO(D, NT, WV, VS) return launch_general<D, NT, WV, VS>((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)vt_pages, block_table, table_stride, table_rows, q_start, context_lens, (bf16*)out, out_stride, n_requests, n_tokens, max_q_len, num_heads, num_kv_heads, page_size, scale, window, stream)
   // Tile width (NT * 16 columns) and waves over a tile's keys.  Few columns (a decode step): one narrow tile
   // per request and many waves over its keys.
   const int cols = max_q_len * (num_heads / num_kv_heads);
@@ -534,7 +587,8 @@ extern "C" int ms_paged_attention_mfma(const void* q, long long q_stride, const 
   // (512 tiles at 640 keys: 32.2 -> 29.3 us).
   int vs = 1;
   if (nt == 1) {
-    const long long tiles = (long long)n_requests * num_kv_heads * ((cols + 15) / 16);
+    const long long per_request = (cols + 15) / 16;
+    const long long tiles = num_kv_heads * std::min(per_request * n_requests, (long long)n_tokens * (num_heads / num_kv_heads) / 16 + n_requests);
     const int cus = ms_compute_units();
     while (vs < 4 && (head_dim / 16) % (vs * 2) == 0 && tiles * vs * 2 <= cus) vs *= 2;
     if (head_dim == 128 && tiles >= 2LL * cus) waves = 4;
@@ -563,7 +617,7 @@ extern "C" int ms_paged_attention_mfma(const void* q, long long q_stride, const 
 // how long the contexts are.
 extern "C" int ms_paged_attention_mfma_decode(const void* q, long long q_stride, const void* k_pages,
                                               const void* vt_pages, const int* block_table, int table_stride,
-                                              const int* q_start, const int* context_lens, void* out,
+                                              const int* table_rows, const int* q_start, const int* context_lens, void* out,
                                               long long out_stride, void* part_o, void* part_ml, int n_requests,
                                               int num_heads, int num_kv_heads, int head_dim, int page_size,
                                               float scale, int window, int min_blocks, int n_splits,
@@ -576,7 +630,7 @@ extern "C" int ms_paged_attention_mfma_decode(const void* q, long long q_stride,
   if (min_blocks <= 0 || n_splits <= 0 || n_splits > COMBINE_MAX_SPLITS) return MS_BAD_ARG;
   if (q_stride % 8 || out_stride % 4 || ((uintptr_t)q % 16) || ((uintptr_t)out % 8) || ((uintptr_t)part_o % 16)) return MS_UNSUPPORTED;
   if (n_requests > 65535 || num_kv_heads > 65535) return MS_UNSUPPORTED;
-#define GO(D) return launch_split<D>((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)vt_pages, block_table, table_stride, q_start, context_lens, (bf16*)out, out_stride, (float*)part_o, (float*)part_ml, n_requests, num_heads, num_kv_heads, page_size, scale, window, min_blocks, n_splits, stream)
+#define GO(D) return launch_split<D>((const bf16*)q, q_stride, (const bf16*)k_pages, (const bf16*)vt_pages, block_table, table_stride, table_rows, q_start, context_lens, (bf16*)out, out_stride, (float*)part_o, (float*)part_ml, n_requests, num_heads, num_kv_heads, page_size, scale, window, min_blocks, n_splits, stream)
   if (head_dim == 32) GO(32);
   if (head_dim == 64) GO(64);
   GO(128);

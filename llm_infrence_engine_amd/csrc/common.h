@@ -5,7 +5,7 @@
 #include <stdint.h>
 
 #define MS_WAVE 64
-#define MS_MAX_GROUPS 4   // cache groups one ms_decode_advance call serves
+#define MS_MAX_GROUPS 8   // cache groups one ms_decode_advance / ms_table_update call serves
 
 // Element type codes of the C entry points.
 enum { MS_F32 = 0, MS_BF16 = 1 };

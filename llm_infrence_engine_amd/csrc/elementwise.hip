@@ -4,6 +4,7 @@
 // and the activation are computed in float.
 #include "common.h"
 #include "api.h"
+#include <algorithm>
 
 // ------------------------------------------------------------------------------------------------
 // out[n, :] = float(table[ids[n], :])
@@ -409,6 +410,7 @@ struct AdvanceArgs {
   int* positions;
   int* context_lens;
   const int* n_live;
+  const int* table_rows;
   const int* tables[MS_MAX_GROUPS];
   int* slots[MS_MAX_GROUPS];
   int n_groups, table_stride, page_size, n_rows;
@@ -421,20 +423,80 @@ __global__ void decode_advance_kernel(AdvanceArgs a) {
   a.positions[r] = pos;
   a.context_lens[r] = pos + 1;
   a.token_ids[r] = a.prev_tokens[r];
+  const size_t row = a.table_rows ? a.table_rows[r] : r;
   for (int g = 0; g < a.n_groups; ++g)
-    a.slots[g][r] = a.tables[g][(size_t)r * a.table_stride + pos / a.page_size] * a.page_size + pos % a.page_size;
+    a.slots[g][r] = a.tables[g][row * a.table_stride + pos / a.page_size] * a.page_size + pos % a.page_size;
 }
 
+extern "C" int ms_max_cache_groups() { return MS_MAX_GROUPS; }
+
 extern "C" int ms_decode_advance(const int* prev_tokens, int* token_ids, int* positions, int* context_lens,
-                                 const int* n_live, const int* const* tables, int* const* slots, int n_groups,
-                                 int table_stride, int page_size, int n_rows, hipStream_t stream) {
+                                 const int* n_live, const int* table_rows, const int* const* tables,
+                                 int* const* slots, int n_groups, int table_stride, int page_size, int n_rows,
+                                 hipStream_t stream) {
   if (n_rows <= 0) return MS_OK;
   if (n_groups < 0 || n_groups > MS_MAX_GROUPS || table_stride <= 0 || page_size <= 0) return MS_BAD_ARG;
   AdvanceArgs a;
   a.prev_tokens = prev_tokens; a.token_ids = token_ids; a.positions = positions; a.context_lens = context_lens;
-  a.n_live = n_live; a.n_groups = n_groups; a.table_stride = table_stride; a.page_size = page_size; a.n_rows = n_rows;
+  a.n_live = n_live; a.table_rows = table_rows; a.n_groups = n_groups; a.table_stride = table_stride;
+  a.page_size = page_size; a.n_rows = n_rows;
   for (int g = 0; g < MS_MAX_GROUPS; ++g) { a.tables[g] = g < n_groups ? tables[g] : nullptr; a.slots[g] = g < n_groups ? slots[g] : nullptr; }
   decode_advance_kernel<<<dim3((n_rows + 63) / 64), dim3(64), 0, stream>>>(a);
+  return ms_launch_status();
+}
+
+// ------------------------------------------------------------------------------------------------
+// The block tables live on the device for as long as the cache does; a step brings only the entries that
+// changed since the last one (pages granted, pages a window has passed, rows given back).
+struct TableUpdateArgs {
+  int* tables[MS_MAX_GROUPS];
+  const int* index[MS_MAX_GROUPS];
+  const int* value[MS_MAX_GROUPS];
+  const int* counts;
+  long long table_elems;
+};
+
+__global__ void table_update_kernel(TableUpdateArgs a) {
+  const int g = blockIdx.y;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= a.counts[g]) return;
+  const long long at = a.index[g][i];
+  if (at >= 0 && at < a.table_elems) a.tables[g][at] = a.value[g][i];
+}
+
+extern "C" int ms_table_update(int* const* tables, const int* const* index, const int* const* value,
+                               const int* counts, int n_groups, int max_updates, long long table_elems,
+                               hipStream_t stream) {
+  if (n_groups <= 0 || max_updates <= 0) return MS_OK;
+  if (n_groups > MS_MAX_GROUPS || table_elems <= 0 || counts == nullptr) return MS_BAD_ARG;
+  TableUpdateArgs a;
+  for (int g = 0; g < MS_MAX_GROUPS; ++g) {
+    a.tables[g] = g < n_groups ? tables[g] : nullptr;
+    a.index[g] = g < n_groups ? index[g] : nullptr;
+    a.value[g] = g < n_groups ? value[g] : nullptr;
+  }
+  a.counts = counts; a.table_elems = table_elems;
+  table_update_kernel<<<dim3((max_updates + 255) / 256, n_groups), dim3(256), 0, stream>>>(a);
+  return ms_launch_status();
+}
+
+// Rows of a tensor set to zero: the state slots of requests whose first portion runs in this step.
+__global__ void zero_rows_kernel(unsigned* __restrict__ base, size_t row_words, const int* __restrict__ rows,
+                                 const int* __restrict__ count) {
+  const int i = blockIdx.y;
+  if (count && i >= *count) return;
+  unsigned* p = base + (size_t)rows[i] * row_words;
+  for (size_t w = (size_t)blockIdx.x * blockDim.x + threadIdx.x; w < row_words; w += (size_t)gridDim.x * blockDim.x)
+    p[w] = 0u;
+}
+
+extern "C" int ms_zero_rows(void* base, long long row_bytes, const int* rows, const int* count, int n_rows,
+                            hipStream_t stream) {
+  if (n_rows <= 0 || row_bytes <= 0) return MS_OK;
+  if (row_bytes % 4 || ((uintptr_t)base % 4) || n_rows > 65535) return MS_BAD_ARG;
+  const size_t words = (size_t)row_bytes / 4;
+  const unsigned bx = (unsigned)std::min<size_t>((words + 255) / 256, 64);
+  zero_rows_kernel<<<dim3(bx, n_rows), dim3(256), 0, stream>>>((unsigned*)base, words, rows, count);
   return ms_launch_status();
 }
 

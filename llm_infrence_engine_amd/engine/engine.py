@@ -24,6 +24,32 @@ from .runner import ModelRunner
 from .scheduler import Scheduler
 
 
+def memory_beside_the_pages(config: EngineConfig, model: Model, layout: CacheLayout) -> int:
+    """An estimate, in bytes, of what an engine holds on the device beside its weights and cache pages: the
+    per-request state of the runs that keep one (one slot more than requests), the block tables, and with graphs
+    the float logits that every batch-size bucket keeps and the activations of the largest captured step (all
+    graphs share one pool): some ten rows of the widest activation per token."""
+    itemsize = model.rt.dtype.itemsize
+    total = 0
+    for need in layout.state_needs.values():
+        for n in (need if isinstance(need, tuple) else (need,)):
+            size = 1
+            for s in n.shape:
+                size *= s
+            total += (config.max_seqs + 1) * size * torch.empty(0, dtype=n.dtype).element_size()
+    total += len(layout.group_keys) * (config.max_seqs + 1) * config.pages_per_request * 4
+    widest = max([model.spec.hidden_size * 4] + [s.shape[0] * itemsize for s in model.tensor_specs()
+                                                  if s.role == "matrix" and len(s.shape) == 2
+                                                  and s.shape[0] != model.spec.vocab_size])
+    tokens = config.max_num_batched_tokens
+    if config.hip_graphs:
+        from .graph import default_batch_sizes
+
+        total += sum(default_batch_sizes(config.max_seqs)) * model.spec.vocab_size * 4
+        tokens += config.max_seqs
+    return total + 10 * tokens * widest
+
+
 class Engine:
     def __init__(self, model: Model, num_blocks: Optional[int] = None, block_size: int = 16, max_seqs: int = 32,
                  max_len: int = 1024, max_num_batched_tokens: int = 2048, max_prefill_chunk: Optional[int] = None,
@@ -31,7 +57,7 @@ class Engine:
                  on_finish: Optional[Callable[[Request], None]] = None,
                  clock: Callable[[], float] = time.perf_counter, hip_graphs: Optional[bool] = None,
                  decode_steps_per_launch: int = 1, capture_at_start: bool = True,
-                 gpu_memory_fraction: Optional[float] = None):
+                 gpu_memory_fraction: Optional[float] = None, graph_portion_tokens: Optional[int] = None):
         """``hip_graphs`` None: on when the model serves in bfloat16 (float32 is the checking path and launches
         every kernel itself).  ``num_blocks`` None: as many pages as ``max_seqs`` requests of ``max_len`` tokens can
         fill, or with ``gpu_memory_fraction`` as many of them as that share of the device's memory has room for
@@ -42,20 +68,26 @@ class Engine:
         ``decode_steps_per_launch`` > 1 (with ``hip_graphs``): while every running request is decoding
         greedily and nobody waits, up to that many decode steps run in one graph launch, each fed the argmax of
         the one before on the device; a stop id is then noticed up to that many steps late (the surplus tokens
-        are dropped), so outputs do not change."""
+        are dropped), so outputs do not change.
+        ``graph_portion_tokens`` (with ``hip_graphs``): steps with prompt portions of up to that many tokens are
+        replayed from graphs too (None: as far as the host would otherwise be what such a step waits for)."""
         dtype = {torch.float32: "float32", torch.bfloat16: "bfloat16"}[model.rt.dtype]
         self.config = EngineConfig(dtype=dtype, block_size=block_size, num_blocks=num_blocks, max_seqs=max_seqs,
                                    max_len=max_len, max_num_batched_tokens=max_num_batched_tokens,
                                    max_prefill_chunk=max_prefill_chunk, hip_graphs=hip_graphs,
                                    decode_steps_per_launch=decode_steps_per_launch,
-                                   gpu_memory_fraction=gpu_memory_fraction, device=str(model.rt.device))
+                                   gpu_memory_fraction=gpu_memory_fraction, graph_portion_tokens=graph_portion_tokens,
+                                   device=str(model.rt.device))
         self.model = model
         pages = self.config.resolved_num_blocks()
         if num_blocks is None and gpu_memory_fraction is not None:
             free, total = torch.cuda.mem_get_info(model.rt.device)
-            per_token = CacheLayout(model.run_needs()).bytes_per_token(model.rt.dtype.itemsize)
-            pages = self.config.resolved_num_blocks(per_token, total, total - free)
-        self.runner = ModelRunner(model, block_size, pages, max_seqs, max_len, hip_graphs=self.config.hip_graphs)
+            layout = CacheLayout(model.run_needs())
+            per_token = layout.bytes_per_token(model.rt.dtype.itemsize)
+            pages = self.config.resolved_num_blocks(per_token, total, total - free,
+                                                    memory_beside_the_pages(self.config, model, layout))
+        self.runner = ModelRunner(model, block_size, pages, max_seqs, max_len, hip_graphs=self.config.hip_graphs,
+                                  graph_portion_tokens=self.config.graph_portion_tokens)
         self.scheduler = Scheduler(self.runner.manager, self.config, clock, on_token, on_finish)
         self.sampler = Sampler(model.rt.device)
         self.clock = clock
@@ -235,7 +267,7 @@ def generate(model: Model, prompt_ids: Sequence[int], max_new_tokens: int = 64, 
         if len(req.output_ids) > n:
             marks.append(time.perf_counter())
     total = time.perf_counter() - t0
-    per_token = model.config.kv_bytes_per_token(model.rt.dtype.itemsize) if hasattr(model, "config") else 0
+    per_token = eng.runner.layout.bytes_per_token(model.rt.dtype.itemsize)    # whatever the model's runs keep per token
     return GenerationResult(
         token_ids=list(req.output_ids), prompt_len=len(prompt_ids), ttft=(marks[0] - t0) if marks else total,
         total_time=total, step_times=[b - a for a, b in zip(marks, marks[1:])],

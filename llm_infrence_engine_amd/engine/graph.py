@@ -1,18 +1,26 @@
-"""Decode-only steps replayed from captured HIP graphs, one graph per batch-size bucket.
+"""Steps replayed from captured HIP graphs.
 
-A decode step of a small model is bound by kernel launches, not by the GPU (the reference measured the
-same on its hardware and answered with CUDA graphs, src/miniserve/graph_decode.py:33-86).  The whole
-forward of a batch of single tokens is captured once per bucket {1, 2, 4, ..., max} (graph_decode.py:23-30)
-over static input buffers; a step then fills a pinned host copy of those buffers, sends it in one copy and
-replays.  Nothing in the captured kernels depends on how long the contexts are (block tables have their
-full width, the attention kernel spreads each request's keys over its waves itself), so a graph stays valid
-for the life of the engine; only the choice between the attention's two launch shapes (contexts up to
-``ops.LONG_CONTEXT`` or beyond) is made per step, and each has graphs of its own.  Rows that pad a batch up to its bucket read the null page and store nothing.
-The greedy choice (argmax) of every row is part of the graph.
+A step of a small model is bound by kernel launches, not by the GPU (the reference measured the same on its
+hardware and answered with CUDA graphs for its decode steps, src/miniserve/graph_decode.py:33-86).  Two kinds
+of step are captured here, both over a static description of the batch (``engine/batch.py``: one int32 array
+of fixed capacity per graph, padded by the same builder that describes a step launched kernel by kernel):
 
-A graph may also hold several decode steps in a row: between two steps a small kernel moves every live
-request one position on, feeds it the token just chosen and looks up its new slots in the block tables, all
-on the device, so the host is needed once per launch instead of once per step.
+* decode steps, one graph per batch-size bucket {1, 2, 4, ..., max} (graph_decode.py:23-30): the whole
+  forward of a batch of single tokens with the greedy choice (argmax) of every row.  A graph may hold several
+  decode steps in a row: between two of them a small kernel moves every live request one position on, feeds
+  it the token just chosen and looks up its new slots in the block tables, all on the device, so the host is
+  needed once per launch instead of once per step;
+* steps with prompt portions (alone or beside decoded tokens), one graph per bucket of the step's number of
+  tokens: embedding and all layers; the final norm and the head run on the wanted rows afterwards, outside the
+  graph, so that any number of rows may be wanted.  A short portion of a narrow model is over on the GPU
+  before the host has enqueued its launches one by one; replayed, it costs the host one launch.
+
+Nothing in the captured kernels depends on how the tokens are dealt out over the requests or on how long the
+contexts are: the attention's launch is sized by the numbers of tokens and requests alone, block tables live on
+the device with their full width, and the changed table entries and the state slots to zero travel in the
+description.  So a graph stays valid for the life of the engine; only the choice between the decode
+attention's two launch shapes (contexts up to ``ops.LONG_CONTEXT`` or beyond) is made per step, and each has
+graphs of its own.
 """
 from __future__ import annotations
 
@@ -24,9 +32,9 @@ import numpy as np
 import torch
 
 from ..kernels import ops
-from ..parts.base import StepContext
-from ..parts.model import RunCache
-from .batch import StepEntry
+from .batch import BatchBuilder, StepBuffers, StepEntry, StepLayout
+
+PORTION_BUCKETS = (16, 32, 64, 128, 256, 384, 512, 768, 1024, 1536, 2048, 3072, 4096)
 
 
 def default_batch_sizes(max_batch: int) -> List[int]:
@@ -38,65 +46,51 @@ def default_batch_sizes(max_batch: int) -> List[int]:
     return sorted({1 << e for e in range(max_batch.bit_length()) if (1 << e) < max_batch} | {max_batch})
 
 
+def portion_graph_limit(model) -> int:
+    """Up to how many tokens a step with prompt portions is worth replaying from a graph: as long as the GPU
+    would be done before the host has enqueued the step's launches one by one (a few hundred launches at 10 to
+    15 us each), at a rate of matrix work that short portions reach.  Beyond that the host hides behind the
+    GPU anyway and a graph's padding up to its bucket would only add work."""
+    weights = sum(s.shape[0] * s.shape[1] for s in model.tensor_specs() if s.role == "matrix" and len(s.shape) == 2)
+    ends = sum(s.shape[0] * s.shape[1] for part in (model.embedding, model.head) for s in part.tensor_specs())
+    per_token = 2.0 * max(1, weights - ends)
+    launches = 9 * len(model.spec.order)
+    tokens = launches * 13e-6 * 0.4e15 / per_token
+    fits = [b for b in PORTION_BUCKETS if b <= tokens]
+    return fits[-1] if fits else 0
+
+
 class _Bucket:
-    def __init__(self, B: int, width: int, n_groups: int, device, steps: int = 1, null_state_slot: int = 0):
-        self.B, self.width, self.steps, self.null_state_slot = B, width, steps, null_state_slot
-        # layout of the static int32 buffer
-        self.off: Dict[str, slice] = {}
-        o = 0
-        for name, n in (("token_ids", B), ("positions", B), ("token_req", B), ("q_start", B + 1),
-                        ("context_lens", B), ("state_slots", B), ("logit_rows", B), ("n_live", 1)):
-            self.off[name] = slice(o, o + n)
-            o += n
-        self.tables, self.slots = [], []
-        for g in range(n_groups):
-            self.tables.append(slice(o, o + B * width)); o += B * width
-            self.slots.append(slice(o, o + B)); o += B
-        self.size = o
-        self.host = torch.zeros(o, dtype=torch.int32).pin_memory()
-        self.np = self.host.numpy()
-        self.dev = torch.zeros(o, dtype=torch.int32, device=device)
-        self.reset_host()
-        self.dev.copy_(self.host)
-        self.last_rows = 0
+    """One captured graph with the static description it reads."""
+
+    def __init__(self, layout: StepLayout, device, steps: int = 1):
+        self.layout, self.steps = layout, steps
+        self.buf = StepBuffers(layout.size, device)
+        self.fields = self.buf.views(layout)
+        self.slots = [self.fields[f"slots{g}"] for g in range(layout.n_groups)]
         self.graph: Optional[torch.cuda.CUDAGraph] = None
-        self.logits: Optional[torch.Tensor] = None
-        self.tokens = torch.zeros((steps, B), dtype=torch.int32, device=device)   # the argmax of every step
-        self.copied: Optional[torch.cuda.Event] = None   # set once the last copy of ``host`` has left it
-
-    def reset_host(self) -> None:
-        """Every row a padding row: token 0 at position 0, one visible key on the null page, nothing stored."""
-        a, B = self.np, self.B
-        a[:] = 0
-        a[self.off["token_req"]] = np.arange(B)
-        a[self.off["q_start"]] = np.arange(B + 1)
-        a[self.off["context_lens"]] = 1
-        a[self.off["logit_rows"]] = np.arange(B)
-        a[self.off["n_live"]] = 0
-        a[self.off["state_slots"]] = self.null_state_slot      # nobody's slot
-        for s in self.slots:
-            a[s] = -1
-
-    def context(self) -> StepContext:
-        d, o = self.dev, self.off
-        return StepContext(
-            num_tokens=self.B, num_requests=self.B, token_ids=d[o["token_ids"]], positions=d[o["positions"]],
-            token_req=d[o["token_req"]], q_start=d[o["q_start"]], context_lens=d[o["context_lens"]],
-            state_slots=d[o["state_slots"]], logit_rows=d[o["logit_rows"]], max_q_len=1,
-            max_context_len=self.width, q_lens_host=[1] * self.B, start_pos_host=[0] * self.B,
-            state_slots_host=[self.null_state_slot] * self.B)
+        self.logits: Optional[torch.Tensor] = None       # decode: [rows, V] of the last step
+        self.hidden = None                                # portions: (residual stream, unsummed addend)
+        self.tokens = torch.zeros((steps, layout.n_requests), dtype=torch.int32, device=device)   # the argmax of every step
 
 
-class DecodeGraphs:
-    def __init__(self, runner, batch_sizes: Optional[Sequence[int]] = None):
+class StepGraphs:
+    def __init__(self, runner, batch_sizes: Optional[Sequence[int]] = None, portion_tokens: Optional[int] = None):
+        """``portion_tokens``: steps with prompt portions of up to that many tokens are replayed from graphs too
+        (None: ``portion_graph_limit`` decides; 0: decode steps only)."""
         m = runner.manager
         if not runner.model.graph_safe():
             raise ValueError("HIP graphs are not used for this model: one of its parts says it cannot be captured "
                              "(Part.graph_safe)")
-        self.runner, self.manager = runner, m
+        self.runner, self.manager, self.builder = runner, m, runner.builder
         self.sizes = sorted(set(batch_sizes or default_batch_sizes(m.max_requests)))
+        limit = portion_graph_limit(runner.model) if portion_tokens is None else portion_tokens
+        if runner.model.graph_safe() is not True:      # a part that can be captured only while it decodes
+            limit = 0
+        self.portion_sizes = [b for b in PORTION_BUCKETS if b <= limit]
         self.width = m.max_pages_per_request
-        self.buckets: Dict[tuple, _Bucket] = {}
+        self.buckets: Dict[tuple, _Bucket] = {}            # decode: (rows, long contexts, steps)
+        self.portion_buckets: Dict[int, _Bucket] = {}      # steps with portions: tokens
         self.pool = None   # one memory pool for all graphs: they never run at the same time
         # what launching costs the host: seconds spent filling the buffers and enqueuing, and launches so far
         # (the reference separates a launch-bound from a GPU-bound step the same way, benchmarks/diag_gpu_launch.py:1-8)
@@ -107,67 +101,97 @@ class DecodeGraphs:
     def max_batch(self) -> int:
         return self.sizes[-1]
 
+    @property
+    def max_portion_tokens(self) -> int:
+        return self.portion_sizes[-1] if self.portion_sizes else 0
+
     def context_classes(self) -> List[bool]:
         """The attention's launch shapes a decode step of this cache can need: short contexts, and long ones
         if a request can grow beyond ``ops.LONG_CONTEXT``."""
         return [False, True] if self.manager.max_len > ops.LONG_CONTEXT else [False]
 
-    def warm_up(self, steps: Sequence[int] = (1,), batch_sizes: Optional[Sequence[int]] = None) -> int:
+    def warm_up(self, steps: Sequence[int] = (1,), batch_sizes: Optional[Sequence[int]] = None,
+                portion_tokens: Optional[Sequence[int]] = None) -> int:
         """Capture, before serving, every graph that serving can reach: each batch-size bucket (or those of
-        ``batch_sizes``), each context class, each number of steps per launch in ``steps``; the reference
-        captures all its buckets in the constructor (src/miniserve/graph_decode.py:46-47).  Afterwards
-        ``run`` captures nothing.  Returns the number of graphs held."""
+        ``batch_sizes``), each context class, each number of steps per launch in ``steps``, and each bucket of
+        portion tokens (or those that ``portion_tokens`` fall into); the reference captures all its buckets in
+        the constructor (src/miniserve/graph_decode.py:46-47).  Afterwards ``run`` captures nothing.  Returns
+        the number of graphs held."""
         sizes = self.sizes if batch_sizes is None else sorted({next(b for b in self.sizes if b >= n) for n in batch_sizes})
-        for B in reversed(sizes):            # the largest first: the others fit into the memory it leaves
+        portions = self.portion_sizes if portion_tokens is None else \
+            sorted({self._portion_size(n) for n in portion_tokens if self._portion_size(n)})
+        for n in reversed(portions):         # the largest first: the others fit into the memory it leaves
+            self._portion_bucket(n)
+        for B in reversed(sizes):
             for long_context in self.context_classes():
                 for k in sorted(set(steps), reverse=True):
                     self._bucket(B, long_context, k)
-        return len(self.buckets)
+        return len(self.buckets) + len(self.portion_buckets)
 
+    # ------------------------------------------------------------------ buckets
     def _bucket(self, n: int, long_context: bool, steps: int = 1) -> _Bucket:
         B = next(b for b in self.sizes if b >= n)
         key = (B, long_context, steps)
         bk = self.buckets.get(key)
         if bk is None:
-            bk = self.buckets[key] = _Bucket(B, self.width, len(self.manager.groups), self.runner.rt.device, steps,
-                                             self.runner.pools.null_state_slot)
-            self._capture(bk, long_context)
+            ps = self.manager.page_size
+            layout = StepLayout(B, B, B, len(self.manager.groups), B * (steps // ps + 2))
+            bk = self.buckets[key] = _Bucket(layout, self.runner.rt.device, steps)
+            cap = self.width * ps
+            self._capture(bk, max_q_len=1, max_context_len=cap if long_context else min(cap, ops.LONG_CONTEXT))
         return bk
 
-    def _caches(self, bk: _Bucket) -> List[RunCache]:
-        r = self.runner
-        caches = []
-        for i in range(len(r.model.spec.order)):
-            g = r.layout.run_group[i]
-            kv = None
-            if g is not None:
-                kv = r.pools.kv_view(i, bk.dev[bk.tables[g]].view(bk.B, bk.width), bk.dev[bk.slots[g]])
-            state = r.pools.state_view(i) if i in r.layout.state_needs else None
-            caches.append(RunCache(kv, state))
-        return caches
+    def _portion_size(self, n_tokens: int) -> int:
+        return next((b for b in self.portion_sizes if b >= n_tokens), 0)
 
-    def _capture(self, bk: _Bucket, long_context: bool) -> None:
-        ctx, caches = bk.context(), self._caches(bk)
-        cap = self.width * self.manager.page_size
-        ctx.max_context_len = cap if long_context else min(cap, ops.LONG_CONTEXT)
-        model = self.runner.model
-        d, o = bk.dev, bk.off
-        tables = [d[s].view(bk.B, bk.width) for s in bk.tables]
-        slots = [d[s] for s in bk.slots]
+    def _portion_bucket(self, size: int) -> _Bucket:
+        bk = self.portion_buckets.get(size)
+        if bk is None:
+            m = self.manager
+            R = m.max_requests
+            layout = StepLayout(size, R, size, len(m.groups), size // m.page_size + 2 * R + 8)
+            bk = self.portion_buckets[size] = _Bucket(layout, self.runner.rt.device)
+            cap = self.width * m.page_size
+            self._capture(bk, max_q_len=min(size, cap), max_context_len=cap)
+        return bk
 
-        def advance(k):   # n_live is 0 in the buffer while capturing and warming up: nothing moves
-            ops.decode_advance(bk.tokens[k - 1], d[o["token_ids"]], d[o["positions"]], d[o["context_lens"]],
-                               d[o["n_live"]], tables, slots, self.manager.page_size)
+    def _capture(self, bk: _Bucket, max_q_len: int, max_context_len: int) -> None:
+        lay, f = bk.layout, bk.fields
+        runner, model = self.runner, self.runner.model
+        decode = max_q_len == 1 and lay.n_tokens == lay.n_requests
+        ctx = self.builder.context(f, lay.n_tokens, lay.n_requests, max_q_len, max_context_len, padded=True)
+        caches = runner.caches(ctx.state_slots, bk.slots)
+        G = lay.n_groups
+        # what the table entries of the last steps changed must be on the device before a description that is all
+        # padding stands in for a step
+        self.builder.flush_updates()
+        bk.buf.wait_until_sent()
+        self.builder.write(None, lay, bk.buf.np)
+        bk.buf.send()
+
+        def body():
+            if G:
+                runner.pools.apply_updates([f[f"update_index{g}"] for g in range(G)],
+                                           [f[f"update_value{g}"] for g in range(G)], f["update_counts"], lay.n_updates)
+            if runner.pools.state:
+                runner.pools.zero_state(f["fresh_rows"], f["n_fresh"])
+            if not decode:
+                bk.hidden = model.forward_hidden(ctx, caches)
+                return
+            for k in range(bk.steps):
+                if k > 0:      # n_live is 0 in the buffer while capturing and warming up: nothing moves
+                    ops.decode_advance(bk.tokens[k - 1], f["token_ids"], f["positions"], f["context_lens"], f["n_live"],
+                                       f["state_slots"], runner.pools.tables, bk.slots, self.manager.page_size)
+                bk.logits = model.head_logits(*model.forward_hidden(ctx, caches), ctx.logit_rows)
+                ops.sample(bk.logits, bk.tokens[k])
 
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
             # load the kernels of this shape before capturing (twice for the first graph, which also
             # settles the allocator)
-            for _ in range(1 if self.buckets.keys() - {(bk.B, long_context, bk.steps)} else 2):
-                ops.sample(model.forward(ctx, caches), bk.tokens[0])
-            if bk.steps > 1:
-                advance(1)
+            for _ in range(1 if self.pool is not None else 2):
+                body()
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         # Nothing that owns device memory or graphs of its own (a runner that went out of use and waits in a
@@ -182,57 +206,57 @@ class DecodeGraphs:
                 self.pool = torch.cuda.graph_pool_handle()
             bk.graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(bk.graph, pool=self.pool):
-                for k in range(bk.steps):
-                    if k > 0:
-                        advance(k)
-                    bk.logits = model.forward(ctx, caches)
-                    ops.sample(bk.logits, bk.tokens[k])
+                body()
         finally:
             if collecting:
                 gc.enable()
         torch.cuda.synchronize()
+
+    # ------------------------------------------------------------------ steps
+    def takes(self, entries: List[StepEntry]) -> Optional[str]:
+        """"decode", "portions", or None if the step is launched kernel by kernel."""
+        if len(entries) <= self.max_batch and all(len(e.tokens) == 1 for e in entries):
+            return "decode"
+        if len(entries) <= self.manager.max_requests and self._portion_size(sum(len(e.tokens) for e in entries)):
+            return "portions"
+        return None
+
+    def _fill_and_replay(self, bk: _Bucket, entries: List[StepEntry], steps: int, every_row: bool = False):
+        if self.manager.pending_updates() > bk.layout.n_updates:
+            self.builder.flush_updates()
+        d = self.builder.describe(entries, steps)
+        if every_row:     # a decode graph works out the logits and the greedy choice of every request, wanted or not
+            d.logit_rows = np.arange(d.n_requests, dtype=np.int32)
+        bk.buf.wait_until_sent()
+        self.builder.write(d, bk.layout, bk.buf.np)
+        bk.buf.send()
+        bk.graph.replay()
+        return d
 
     def run(self, entries: List[StepEntry], steps: int = 1):
         """``steps`` decode steps for ``entries`` (one token each, pages already grown for all the steps).
         Returns (logits [R, V] of the last step, greedy tokens int32 [steps, R]); both are views of static
         buffers that the next replay overwrites."""
         t_begin = time.perf_counter()
-        m = self.manager
         R = len(entries)
-        rows = np.fromiter((m.row(e.req_id) for e in entries), dtype=np.int32, count=R)
-        pos = np.fromiter((m.computed(e.req_id) for e in entries), dtype=np.int32, count=R)
-        bk = self._bucket(R, int(pos.max()) + steps > ops.LONG_CONTEXT, steps)
-        a, o, ps = bk.np, bk.off, m.page_size
-        if bk.copied is not None:
-            bk.copied.synchronize()      # the last launch's copy must have read the pinned buffer before it changes
-        toks = np.fromiter((e.tokens[0] for e in entries), dtype=np.int64, count=R)
-        if toks.min() < 0 or toks.max() >= self.runner.model.spec.vocab_size:
-            raise ValueError("a token id is outside the vocabulary")
-        if int(pos.max()) + steps > m.max_len:
-            raise ValueError(f"a request would hold {int(pos.max()) + steps} tokens; the cache is made for {m.max_len}")
-        if R < bk.last_rows:
-            bk.reset_host()
-        bk.last_rows = R
-        if self.runner.layout.state_runs and (pos == 0).any():
-            self.runner.pools.zero_state([int(r) for r in rows[pos == 0]])      # a first token starts from zero state
-        a[o["token_ids"]][:R] = toks
-        a[o["positions"]][:R] = pos
-        a[o["context_lens"]][:R] = pos + 1
-        a[o["state_slots"]][:R] = rows
-        a[o["n_live"]] = R
-        used = (int(pos.max()) + steps - 1) // ps + 1
-        for g, grp in enumerate(m.groups):
-            t = a[bk.tables[g]].reshape(bk.B, bk.width)
-            t[:R, :used] = grp.tables[rows, :used]
-            page = t[np.arange(R), pos // ps]
-            if (page == 0).any() or (t[np.arange(R), (pos + steps - 1) // ps] == 0).any():
-                raise RuntimeError("a token of this launch has no page; grow the requests before it")
-            a[bk.slots[g]][:R] = page * ps + pos % ps
-        bk.dev.copy_(bk.host, non_blocking=True)
-        if bk.copied is None:
-            bk.copied = torch.cuda.Event()
-        bk.copied.record()
-        bk.graph.replay()
+        longest = max(self.manager.computed(e.req_id) for e in entries) + steps
+        bk = self._bucket(R, longest > ops.LONG_CONTEXT, steps)
+        self._fill_and_replay(bk, entries, steps, every_row=True)
         self.enqueue_seconds += time.perf_counter() - t_begin
         self.launches += 1
         return bk.logits[:R], bk.tokens[:, :R]
+
+    def run_portions(self, entries: List[StepEntry]) -> torch.Tensor:
+        """A step with prompt portions from its bucket's graph; the head runs on the wanted rows afterwards.
+        Returns float logits [wanted, V]."""
+        t_begin = time.perf_counter()
+        bk = self._portion_bucket(self._portion_size(sum(len(e.tokens) for e in entries)))
+        d = self._fill_and_replay(bk, entries, 1)
+        x, pending = bk.hidden
+        logits = self.runner.model.head_logits(x, pending, bk.fields["logit_rows"][:d.logit_rows.size])
+        self.enqueue_seconds += time.perf_counter() - t_begin
+        self.launches += 1
+        return logits
+
+
+DecodeGraphs = StepGraphs   # the name this class had while it replayed decode steps only

@@ -58,7 +58,7 @@ class Scheduler:
         need = len(req.prompt_ids) + req.max_new_tokens
         if need > self.config.max_len:
             raise ValueError(f"request needs {need} cache positions but max_len is {self.config.max_len}")
-        if need > self.manager.num_pages * self.manager.page_size:
+        if need > self.manager.capacity_tokens():
             raise ValueError("request can never fit in the page pool")
         with self._lock:
             req.id = self._next_id
@@ -108,7 +108,7 @@ class Scheduler:
             left = r.num_tokens - r.num_computed
             if r.state != "running" or left <= 1 or budget == 0:
                 continue
-            n = min(left, budget, chunk, self._tokens_that_fit(r, reserve=0))
+            n = min(left, budget, chunk, m.tokens_that_fit(r.id))
             if n <= 0:
                 continue
             m.grow(r.id, r.num_computed + n)
@@ -135,16 +135,6 @@ class Scheduler:
             out.append(Scheduled(r, 0, n, n == r.num_tokens))
             budget -= n
         return out
-
-    def _tokens_that_fit(self, r: Request, reserve: int) -> int:
-        """How many more tokens the free pages let the request hold."""
-        m = self.manager
-        fit = None
-        for i, g in enumerate(m.groups):
-            held = m._held[r.id].next_page[i]
-            t = (held + max(0, g.allocator.num_free() - reserve)) * m.page_size - r.num_computed
-            fit = t if fit is None else min(fit, t)
-        return m.max_len - r.num_computed if fit is None else min(fit, m.max_len - r.num_computed)
 
     # ------------------------------------------------------------------ after the model ran
     def commit(self, scheduled: List[Scheduled], sampled: List[int]) -> int:

@@ -38,8 +38,9 @@ def replay(model_dir, dtype: str, out_dir, max_tokens: int, lines, log=sys.stdou
     if max_tokens <= 0:
         raise ValueError("--max-tokens must be positive")
     tokens = -(-max_tokens // unit) * unit
+    # bfloat16 is the serving path, and serving replays its steps from captured graphs
     runner = load_runner(model_dir, dtype=dtype, device=device, page_size=page_size, num_pages=tokens // page_size,
-                         max_requests=MAX_LIVE, max_len=tokens)
+                         max_requests=MAX_LIVE, max_len=tokens, hip_graphs=dtype == "bfloat16")
     for line in lines:
         line = line.strip()
         if not line:

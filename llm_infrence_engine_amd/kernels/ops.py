@@ -27,7 +27,11 @@ _SIGNATURES = {
                             _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "ms_qkv_rope_store": [_c_ptr, _c_ll, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                           _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
-    "ms_decode_advance": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "ms_decode_advance": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int,
+                          _c_ptr],
+    "ms_max_cache_groups": [],
+    "ms_table_update": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ll, _c_ptr],
+    "ms_zero_rows": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_int, _c_ptr],
     "ms_bias_add": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "ms_gemm_skinny": [_c_ptr, _c_ll, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int,
                        _c_ptr],
@@ -50,15 +54,15 @@ _SIGNATURES = {
                       _c_int, _c_int, _c_int, _c_ptr],
     "ms_gemm_generic": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ll, _c_ll, _c_ll, _c_int,
                         _c_int, _c_int, _c_ptr],
-    "ms_paged_attention_generic": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ll,
-                                   _c_int, _c_int, _c_int, _c_int, _c_int, _c_ll, _c_float, _c_int, _c_int, _c_int,
-                                   _c_ptr],
+    "ms_paged_attention_generic": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                                   _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ll, _c_float, _c_int, _c_int,
+                                   _c_int, _c_ptr],
     "ms_attention_mfma_supported": [_c_int, _c_int],
-    "ms_paged_attention_mfma": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ll, _c_int,
-                                _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
-    "ms_paged_attention_mfma_decode": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ll,
-                                       _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int,
-                                       _c_int, _c_int, _c_ptr],
+    "ms_paged_attention_mfma": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ll,
+                                _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
+    "ms_paged_attention_mfma_decode": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                                       _c_ll, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
+                                       _c_int, _c_int, _c_int, _c_ptr],
     "ms_argmax": [_c_ptr, _c_ll, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr],
     "ms_sample": [_c_ptr, _c_ll, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
 }
@@ -194,29 +198,83 @@ def bias_add(x: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
     return x
 
 
-MAX_GROUPS = 4
+MAX_CACHE_GROUPS = 8   # cache groups one call of ``decode_advance`` or ``table_update`` serves (the library's MS_MAX_GROUPS)
+
+
+def max_cache_groups() -> int:
+    """The same number, as the loaded library states it."""
+    n = int(_get("ms_max_cache_groups")())
+    if n != MAX_CACHE_GROUPS:
+        raise build.KernelLibraryError(f"the library serves {n} cache groups, this module expects {MAX_CACHE_GROUPS}")
+    return n
+
+
+def _pointer_array(tensors):
+    arr = (ctypes.c_void_p * max(1, len(tensors)))(*[t.data_ptr() for t in tensors])
+    return arr, ctypes.cast(arr, ctypes.c_void_p)
 
 
 def decode_advance(prev_tokens: torch.Tensor, token_ids: torch.Tensor, positions: torch.Tensor,
-                   context_lens: torch.Tensor, n_live: torch.Tensor, tables, slots, page_size: int) -> None:
+                   context_lens: torch.Tensor, n_live: torch.Tensor, table_rows: Optional[torch.Tensor], tables, slots,
+                   page_size: int) -> None:
     """Between two decode steps queued back to back: rows below ``n_live[0]`` move one position on, take
-    ``prev_tokens`` as their input and get their new slots from ``tables`` (one [rows, width] per cache group)."""
+    ``prev_tokens`` as their input and get their new slots from ``tables`` (one [table rows, width] per cache
+    group; row r of the batch has the table row ``table_rows[r]``, or r without it)."""
     R = token_ids.numel()
     for t, name in ((prev_tokens, "prev_tokens"), (token_ids, "token_ids"), (positions, "positions"),
                     (context_lens, "context_lens")):
         _check(t, name, torch.int32, (R,))
     _check(n_live, "n_live", torch.int32, (1,))
-    if len(tables) != len(slots) or len(tables) > MAX_GROUPS:
-        raise ValueError(f"at most {MAX_GROUPS} cache groups, one table and one slot mapping each")
+    if len(tables) != len(slots) or len(tables) > max_cache_groups():
+        raise ValueError(f"at most {max_cache_groups()} cache groups, one table and one slot mapping each")
     width = tables[0].shape[1] if tables else 1
+    if table_rows is not None:
+        _check(table_rows, "table_rows", torch.int32, (R,))
     for t, sl in zip(tables, slots):
-        _check(t, "table", torch.int32, (R, width))
+        _check(t, "table", torch.int32, (None if table_rows is not None else R, width))
         _check(sl, "slots", torch.int32, (R,))
-    tp = (ctypes.c_void_p * max(1, len(tables)))(*[t.data_ptr() for t in tables])
-    sp = (ctypes.c_void_p * max(1, len(slots)))(*[t.data_ptr() for t in slots])
+    keep_t, tp = _pointer_array(tables)
+    keep_s, sp = _pointer_array(slots)
     _call("ms_decode_advance", prev_tokens.data_ptr(), token_ids.data_ptr(), positions.data_ptr(),
-          context_lens.data_ptr(), n_live.data_ptr(), ctypes.cast(tp, ctypes.c_void_p), ctypes.cast(sp, ctypes.c_void_p),
-          len(tables), width, page_size, R, _stream())
+          context_lens.data_ptr(), n_live.data_ptr(), _ptr(table_rows), tp, sp, len(tables), width, page_size, R,
+          _stream())
+
+
+def table_update(tables, index, value, counts: torch.Tensor, max_updates: int) -> None:
+    """tables[g].view(-1)[index[g][i]] = value[g][i] for i < counts[g]: the entries of the device's block tables
+    that changed since the last step.  ``index`` / ``value``: per group int32 [max_updates]; ``counts`` int32
+    [groups] on the device.  An index appears at most once per group."""
+    G = len(tables)
+    if not (G == len(index) == len(value)) or G > max_cache_groups():
+        raise ValueError(f"one index and one value array per table, at most {max_cache_groups()} tables")
+    if G == 0 or max_updates <= 0:
+        return
+    _check(counts, "counts", torch.int32, (G,))
+    elems = tables[0].numel()
+    for t, ix, v in zip(tables, index, value):
+        _check(t, "table", torch.int32)
+        if t.numel() != elems:
+            raise ValueError("the block tables of all groups have one shape")
+        _check(ix, "index", torch.int32, (max_updates,))
+        _check(v, "value", torch.int32, (max_updates,))
+    keep_t, tp = _pointer_array(tables)
+    keep_i, ip = _pointer_array(index)
+    keep_v, vp = _pointer_array(value)
+    _call("ms_table_update", tp, ip, vp, counts.data_ptr(), G, max_updates, elems, _stream())
+
+
+def zero_rows(t: torch.Tensor, rows: torch.Tensor, count: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """t[rows[i]] = 0 for every i (for i < count[0] with ``count``, a device int): rows of a tensor whose first
+    dimension is indexed by ``rows``."""
+    _check(t, "t")
+    _check(rows, "rows", torch.int32)
+    if count is not None:
+        _check(count, "count", torch.int32, (1,))
+    row_bytes = (t.numel() // max(1, t.shape[0])) * t.element_size()
+    if row_bytes % 4:
+        raise ValueError("rows must be a multiple of 4 bytes long")
+    _call("ms_zero_rows", t.data_ptr(), row_bytes, rows.data_ptr(), _ptr(count), rows.numel(), _stream())
+    return t
 
 
 def read_probe(t: torch.Tensor) -> torch.Tensor:
@@ -550,13 +608,17 @@ def qkv_rope_store(x: torch.Tensor, norm_weight: torch.Tensor, eps: float, w_qkv
 
 def paged_attention_generic(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, block_table: torch.Tensor,
                             token_req: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, num_heads: int,
-                            scale: float, window: Optional[int] = None, v_transposed: bool = False) -> torch.Tensor:
+                            scale: float, window: Optional[int] = None, v_transposed: bool = False,
+                            table_rows: Optional[torch.Tensor] = None,
+                            n_live_tokens: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[n, h] = softmax(scale * q[n, h] . K[keys visible to n]) V, keys read in place from pages.
 
     q: [N, >= nh * d] (a row slice of the fused projection is fine), out [N, nh * d],
     pages [P, nkv, page_size, d] (values [P, nkv, d, page_size] with ``v_transposed``), block_table int32
-    [R, max_pages], token_req / positions int32 [N].
-    Token n sees keys 0..positions[n] of request token_req[n] (the last ``window`` of them if given)."""
+    [rows, max_pages], token_req / positions int32 [N].
+    Token n sees keys 0..positions[n] of request token_req[n] (the last ``window`` of them if given), whose
+    pages are row ``table_rows[token_req[n]]`` of the table (row token_req[n] without ``table_rows``).  With
+    ``n_live_tokens`` (a device int) tokens from that index on are left alone."""
     _check(k_pages, "k_pages")
     P, nkv, page_size, d = k_pages.shape
     _check(v_pages, "v_pages", k_pages.dtype, _v_shape(k_pages, v_transposed))
@@ -570,10 +632,15 @@ def paged_attention_generic(q: torch.Tensor, k_pages: torch.Tensor, v_pages: tor
         raise ValueError("block_table must be [requests, pages]")
     _check(token_req, "token_req", torch.int32, (N,))
     _check(positions, "positions", torch.int32, (N,))
+    if table_rows is not None:
+        _check(table_rows, "table_rows", torch.int32)
+    if n_live_tokens is not None:
+        _check(n_live_tokens, "n_live_tokens", torch.int32, (1,))
     if num_heads % nkv:
         raise ValueError(f"{num_heads} query heads cannot share {nkv} key/value heads")
     _call("ms_paged_attention_generic", q.data_ptr(), q.stride(0) if N > 1 else q.shape[1], k_pages.data_ptr(),
-          v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], token_req.data_ptr(), positions.data_ptr(),
+          v_pages.data_ptr(), block_table.data_ptr(), block_table.shape[1], _ptr(table_rows), _ptr(n_live_tokens),
+          token_req.data_ptr(), positions.data_ptr(),
           out.data_ptr(), num_heads * d, N, num_heads, nkv, d, page_size, P, float(scale), int(window or 0),
           int(v_transposed), _code(q.dtype), _stream())
     return out
@@ -598,10 +665,13 @@ def attention_splits_keys(n_requests: int, num_kv_heads: int, group: int, max_q_
 
 def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, vt_pages: torch.Tensor, block_table: torch.Tensor,
                          q_start: torch.Tensor, context_lens: torch.Tensor, out: torch.Tensor, num_heads: int,
-                         scale: float, max_q_len: int, max_context_len: int, window: Optional[int] = None) -> torch.Tensor:
+                         scale: float, max_q_len: int, max_context_len: int, window: Optional[int] = None,
+                         table_rows: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Matrix-core attention, bfloat16.  k_pages [P, nkv, page_size, d], vt_pages [P, nkv, d, page_size];
-    request r owns tokens q_start[r]..q_start[r+1]-1 and holds context_lens[r] keys after this step.  A
-    small batch of single tokens with long contexts also splits the keys over blocks (and combines)."""
+    request r owns tokens q_start[r]..q_start[r+1]-1, holds context_lens[r] keys after this step and has row
+    ``table_rows[r]`` of ``block_table`` (row r without ``table_rows``).  ``max_q_len`` and ``max_context_len``
+    are upper bounds; tokens from q_start[R] on belong to no request, a request may have no token.  A small
+    batch of single tokens with long contexts also splits the keys over blocks (and combines)."""
     _check(k_pages, "k_pages", torch.bfloat16)
     P, nkv, page_size, d = k_pages.shape
     _check(vt_pages, "vt_pages", torch.bfloat16, (P, nkv, d, page_size))
@@ -611,9 +681,13 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, vt_pages: torch
         raise ValueError(f"q must be [N, >= {num_heads * d}] with unit stride along rows, got {list(q.shape)}")
     _check(out, "out", torch.bfloat16, (N, num_heads * d))
     _check(block_table, "block_table", torch.int32)
-    R = block_table.shape[0]
+    R = context_lens.numel()
     _check(q_start, "q_start", torch.int32, (R + 1,))
     _check(context_lens, "context_lens", torch.int32, (R,))
+    if table_rows is not None:
+        _check(table_rows, "table_rows", torch.int32, (R,))
+    elif block_table.shape[0] < R:
+        raise ValueError(f"the block table has {block_table.shape[0]} rows for {R} requests")
     if num_heads % nkv:
         raise ValueError(f"{num_heads} query heads cannot share {nkv} key/value heads")
     if max_q_len < 1 or max_context_len < max_q_len or max_context_len > block_table.shape[1] * page_size:
@@ -633,13 +707,14 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, vt_pages: torch
         part_o = torch.empty((R, num_heads, n_splits, d), dtype=torch.float32, device=q.device)
         part_ml = torch.empty((R, num_heads, n_splits, 2), dtype=torch.float32, device=q.device)
         _call("ms_paged_attention_mfma_decode", q.data_ptr(), q_stride, k_pages.data_ptr(), vt_pages.data_ptr(),
-              block_table.data_ptr(), block_table.shape[1], q_start.data_ptr(), context_lens.data_ptr(), out.data_ptr(),
-              num_heads * d, part_o.data_ptr(), part_ml.data_ptr(), R, num_heads, nkv, d, page_size, float(scale),
+              block_table.data_ptr(), block_table.shape[1], _ptr(table_rows), q_start.data_ptr(), context_lens.data_ptr(),
+              out.data_ptr(), num_heads * d, part_o.data_ptr(), part_ml.data_ptr(), R, num_heads, nkv, d, page_size, float(scale),
               int(window or 0), MIN_BLOCKS_PER_SPLIT, n_splits, _stream())
     else:
         _call("ms_paged_attention_mfma", q.data_ptr(), q_stride, k_pages.data_ptr(), vt_pages.data_ptr(),
-              block_table.data_ptr(), block_table.shape[1], q_start.data_ptr(), context_lens.data_ptr(), out.data_ptr(),
-              num_heads * d, R, max_q_len, num_heads, nkv, d, page_size, float(scale), int(window or 0), _stream())
+              block_table.data_ptr(), block_table.shape[1], _ptr(table_rows), q_start.data_ptr(), context_lens.data_ptr(),
+              out.data_ptr(), num_heads * d, R, N, max_q_len, num_heads, nkv, d, page_size, float(scale), int(window or 0),
+              _stream())
     return out
 
 
@@ -680,6 +755,6 @@ def paged_attention(q: torch.Tensor, kv, ctx, out: torch.Tensor, num_heads: int,
     if (q.dtype == torch.bfloat16 and kv.v_transposed and attention_mfma_supported(d, page_size)
             and q.data_ptr() % 16 == 0 and (q.shape[0] == 1 or q.stride(0) % 8 == 0)):
         return paged_attention_mfma(q, kv.k_pages, kv.v_pages, kv.block_table, ctx.q_start, ctx.context_lens, out,
-                                    num_heads, scale, ctx.max_q_len, ctx.max_context_len, window)
+                                    num_heads, scale, ctx.max_q_len, ctx.max_context_len, window, kv.table_rows)
     return paged_attention_generic(q, kv.k_pages, kv.v_pages, kv.block_table, ctx.token_req, ctx.positions, out,
-                                   num_heads, scale, window, kv.v_transposed)
+                                   num_heads, scale, window, kv.v_transposed, kv.table_rows, ctx.n_live_tokens)

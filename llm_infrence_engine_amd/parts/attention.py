@@ -63,9 +63,8 @@ class GQAttention(Mixer):
     def cache_need(self):
         # in bfloat16 the matrix-core attention reads value pages as an operand as they lie, transposed, which it
         # can for pages of a multiple of 16 tokens
-        rt = getattr(self, "rt", None)
-        at = 16 if rt is not None and rt.dtype == torch.bfloat16 else None
-        return KVNeed(self.num_kv_heads, self.head_dim, self.window, transpose_values_at=at)
+        return KVNeed(self.num_kv_heads, self.head_dim, self.window, transpose_values_at=16,
+                      transpose_values_in=torch.bfloat16)
 
     # ---- step
     def forward(self, h, ctx, kv, state):

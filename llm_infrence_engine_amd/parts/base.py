@@ -40,12 +40,15 @@ class Runtime:
 class PageTensor:
     """One tensor of a cache page: ``heads`` x ``width`` values per token, kept as [heads, page_size, width].
     With ``transpose_at`` = n the pool keeps it as [heads, width, page_size] instead whenever the page size is
-    a multiple of n (a mixer asks for that when its kernels read the tensor as a matrix operand as it lies)."""
+    a multiple of n (a mixer asks for that when its kernels read the tensor as a matrix operand as it lies),
+    with ``transpose_in`` only when the cache holds that type.  What a part declares here does not depend on
+    whether it has been loaded or in which type: the pool, which knows both, decides."""
 
     name: str
     heads: int
     width: int
     transpose_at: Optional[int] = None
+    transpose_in: Optional[torch.dtype] = None
 
 
 @dataclass(frozen=True)
@@ -68,10 +71,10 @@ class CacheNeed:
 
 
 def KVNeed(num_kv_heads: int, head_dim: int, window: Optional[int] = None,
-           transpose_values_at: Optional[int] = None) -> CacheNeed:
+           transpose_values_at: Optional[int] = None, transpose_values_in: Optional[torch.dtype] = None) -> CacheNeed:
     """The usual need of attention: keys "k" and values "v", [num_kv_heads, head_dim] each."""
-    return CacheNeed((PageTensor("k", num_kv_heads, head_dim), PageTensor("v", num_kv_heads, head_dim, transpose_values_at)),
-                     window)
+    return CacheNeed((PageTensor("k", num_kv_heads, head_dim),
+                      PageTensor("v", num_kv_heads, head_dim, transpose_values_at, transpose_values_in)), window)
 
 
 @dataclass(frozen=True)
@@ -86,14 +89,21 @@ class StateNeed:
 
 @dataclass
 class KVView:
-    """One run's pages of its cache group, with the group's tables for the step's requests."""
+    """One run's pages of its cache group, with the group's block table and the step's slots.  The table lives
+    on the device for as long as the cache does, one row per request the engine can hold (and a last row of
+    null pages); request r of the step reads row ``table_rows[r]``."""
 
     pages: Dict[str, torch.Tensor]       # name -> [pages, heads, page_size, width], or [pages, heads, width, page_size]
     transposed: Dict[str, bool]          # name -> which of the two
-    block_table: torch.Tensor            # int32 [R, max pages]
-    slot_mapping: torch.Tensor           # int32 [N]: page * page_size + offset of each token
+    block_table: torch.Tensor            # int32 [rows, max pages]
+    slot_mapping: torch.Tensor           # int32 [N]: page * page_size + offset of each token; < 0: not stored
     store: bool = True                   # False: the run reads another run's cache and writes nothing
     window: Optional[int] = None
+    table_rows: Optional[torch.Tensor] = None   # int32 [R]; None: request r reads row r
+
+    def pages_of(self, r: int) -> torch.Tensor:
+        """The block-table row of the step's request ``r`` (for parts written in plain tensor code)."""
+        return self.block_table[r if self.table_rows is None else self.table_rows[r].long()]
 
     # the usual pair of attention
     @property
@@ -133,8 +143,10 @@ class StepContext:
     context_lens: torch.Tensor   # [R] keys each request holds once this step's tokens are stored
     state_slots: torch.Tensor    # [R] slot of each request's fixed-size state
     logit_rows: torch.Tensor     # [M] tokens whose logits are wanted
-    max_q_len: int = 0
-    max_context_len: int = 0
+    max_q_len: int = 0           # an upper bound of the portions' lengths (the longest, outside a captured graph)
+    max_context_len: int = 0     # and of the context lengths
+    # [1], = q_start[R]: in a captured batch the tokens from there on belong to no request (None: there are none)
+    n_live_tokens: Optional[torch.Tensor] = None
     # host copies for parts written in plain tensor code (tests' toy parts) and for kernel choice
     q_lens_host: List[int] = field(default_factory=list)
     start_pos_host: List[int] = field(default_factory=list)
@@ -149,11 +161,24 @@ class StepContext:
 Getter = Callable[[TensorSpec], torch.Tensor]
 
 
+def weakest(answers) -> object:
+    """The least of several ``graph_safe`` answers: False < "decode" < True."""
+    rank = {False: 0, "decode": 1, True: 2}
+    worst = True
+    for a in answers:
+        a = a if a == "decode" else bool(a)
+        if rank[a] < rank[worst]:
+            worst = a
+    return worst
+
+
 class Part:
-    # Whether a decode step that runs this part may be captured into a graph and replayed: the part reads the
-    # step's batch from the device tensors of its StepContext only (never from the host copies), does not wait
-    # for the device and launches the same work whatever those tensors hold.  A model with a part that says
-    # False steps without graphs.
+    # Whether a step that runs this part may be captured into a graph and replayed: the part reads the step's
+    # batch from the device tensors of its StepContext only (never from the host copies, which a captured step
+    # does not have), does not wait for the device and launches the same work whatever those tensors hold:
+    # tokens dealt out over the requests in any way, requests without tokens and tokens of no request padding
+    # the batch (``StepContext.n_live_tokens``).  True: every step; "decode": only steps in which every request
+    # has one token (``ctx.decode_only``); False: none, and a model with such a part steps without graphs.
     graph_safe = True
 
     def tensor_specs(self) -> List[TensorSpec]:
@@ -198,9 +223,9 @@ class Mixer(Part):
     accepts_lazy_norm = False   # True: h may be a LazyNorm that the part hands to kernels.linear
 
     @property
-    def graph_safe(self) -> bool:
+    def graph_safe(self):
         """A mixer with per-request state is taken to walk its requests on the host unless its class says
-        ``graph_safe = True``."""
+        ``graph_safe = True`` or ``"decode"``."""
         return self.state_need() is None
 
     def cache_need(self) -> Optional[CacheNeed]:
@@ -300,8 +325,8 @@ class Block(Part):
             return None
         return needs[0] if len(needs) == 1 else tuple(needs)
 
-    def graph_safe(self) -> bool:
-        return all(p.graph_safe for p in self.built.values() if p is not None)
+    def graph_safe(self):
+        return weakest(p.graph_safe for p in self.built.values() if p is not None)
 
     def tensor_specs(self) -> List[TensorSpec]:
         return [s for p in self.parts() for s in p.tensor_specs()]

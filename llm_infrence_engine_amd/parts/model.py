@@ -14,7 +14,7 @@ from ..config.spec import ModelSpec
 from ..weights.reader import CheckpointReader, place
 from ..weights.spec import TensorSpec
 from . import attention, blocks, ends, feed_forward, norms, positions  # noqa: F401  (register the built-in parts)
-from .base import KVView, Runtime, StateView, StepContext, build_part, part_class
+from .base import KVView, Runtime, StateView, StepContext, build_part, part_class, weakest
 
 
 @dataclass
@@ -74,20 +74,31 @@ class Model:
         return [(self.layers[run.layer].cache_need(), self.layers[run.layer].state_need(), run.cache_of)
                 for run in self.spec.order]
 
-    def graph_safe(self) -> bool:
-        """Whether a decode step of this model may be captured into a graph (see ``Part.graph_safe``)."""
-        return (all(b.graph_safe() for b in self.layers)
-                and all(p.graph_safe for p in (self.embedding, self.final_norm, self.head)))
+    def graph_safe(self):
+        """Which steps of this model may be captured into graphs: True (all), "decode" (steps of single tokens)
+        or False (none); the weakest answer of its parts (see ``Part.graph_safe``)."""
+        return weakest([b.graph_safe() for b in self.layers] +
+                       [p.graph_safe for p in (self.embedding, self.final_norm, self.head)])
 
     # ------------------------------------------------------------------ one step
     def forward(self, ctx: StepContext, caches: List[RunCache]) -> torch.Tensor:
         """Float logits [M, V] at ``ctx.logit_rows``.  Runs only the step's tokens, from the cache."""
+        x, pending = self.forward_hidden(ctx, caches)
+        return self.head_logits(x, pending, ctx.logit_rows)
+
+    def forward_hidden(self, ctx: StepContext, caches: List[RunCache]):
+        """Embedding and all runs of the order: the float residual stream [N, H] and the last run's addend that
+        is still to be summed into it (or None)."""
         x = self.embedding.forward(ctx)
         pending = None
         for i, run in enumerate(self.spec.order):
             c = caches[i]
             pending = self.layers[run.layer].forward(x, pending, ctx, c.kv, c.state)
-        if ctx.logit_rows.numel() == 0:
+        return x, pending
+
+    def head_logits(self, x: torch.Tensor, pending: Optional[torch.Tensor], rows: torch.Tensor) -> torch.Tensor:
+        """Final norm and head on the rows ``rows`` (int32) of what ``forward_hidden`` returned; x is left as it is."""
+        if rows.numel() == 0:
             return torch.empty(0, self.spec.vocab_size, dtype=torch.float32, device=x.device)
         norm = self.final_norm.lazy if self.head.accepts_lazy_norm else self.final_norm.forward
-        return self.head.forward(norm(x, delta=pending, rows=ctx.logit_rows, write_back=False))
+        return self.head.forward(norm(x, delta=pending, rows=rows, write_back=False))

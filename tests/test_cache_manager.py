@@ -152,3 +152,45 @@ def test_random_orders_lose_nothing(seed):
     m.check_invariants()
     assert all(g.allocator.num_in_use() == 0 for g in m.groups) and m.free_rows() == 4
     assert all((g.tables == NULL_PAGE).all() for g in m.groups)
+
+
+def test_a_copy_kept_by_the_changed_entries_equals_the_tables():
+    """What ``take_updates`` lists (each entry once per call) keeps a second copy of the block tables, the one the
+    device holds, equal to the manager's, under random adds, growth, windows passing and frees; the last row
+    stays all null pages."""
+    rng = random.Random(5)
+    m = CacheManager(CacheLayout([full(), full(window=6), full(4, 32)]), page_size=4, num_pages=[40, 12, 25],
+                     max_requests=5, max_len=64)
+    assert m.pages_per_group == [40, 12, 25] and m.num_pages == 12 and m.capacity_tokens() == 48
+    copies = [np.zeros_like(g.tables) for g in m.groups]
+    live, next_id = {}, 0
+    for step in range(600):
+        op = rng.random()
+        if op < 0.25 and m.free_rows():
+            m.add(next_id); live[next_id] = 0; next_id += 1
+        elif op < 0.8 and live:
+            r = rng.choice(list(live))
+            n = min(64, live[r] + rng.randint(1, 9))
+            if m.can_grow(r, n):
+                m.grow(r, n); m.advance(r, n); live[r] = n
+        elif live:
+            r = rng.choice(list(live)); m.free(r); del live[r]
+        if rng.random() < 0.4:                       # several operations between two steps is the usual case
+            assert m.pending_updates() == max(len(c) for c in m._changed)
+            for copy, (index, value) in zip(copies, m.take_updates()):
+                assert len(set(index.tolist())) == index.size
+                copy.reshape(-1)[index] = value
+            assert m.pending_updates() == 0
+            for copy, g in zip(copies, m.groups):
+                assert (copy == g.tables).all() and (copy[m.null_row] == NULL_PAGE).all()
+            m.check_invariants()
+
+
+def test_tokens_that_fit_counts_every_group():
+    m = CacheManager(CacheLayout([full(), full(4, 32)]), page_size=4, num_pages=[10, 3], max_requests=2, max_len=64)
+    m.add("a")
+    assert m.tokens_that_fit("a") == 12 and m.tokens_that_fit("a", reserve=1) == 8
+    m.grow("a", 5); m.advance("a", 5)
+    assert m.tokens_that_fit("a") == 7          # two pages held (8 tokens) and one free in the small pool, 5 stored
+    with pytest.raises(ValueError, match="pool sizes"):
+        CacheManager(CacheLayout([full()]), 4, [3, 3], 2, 64)

@@ -206,12 +206,20 @@ def test_a_layer_names_its_parts_and_the_arrangement_says_which_it_takes():
     ls = spec.layers[0]
     assert ls.block == "pre_norm_residual" and sorted(ls.parts) == ["feed_forward", "feed_forward_norm", "mixer",
                                                                     "mixer_norm", "position"]
-    assert ls.mixer.kind == "gqa_attention" and ls.no_such_part is None
+    assert ls.mixer.kind == "gqa_attention" and ls.parts.get("no_such_part") is None
+    with pytest.raises(AttributeError, match="no part named 'mixr'"):     # a misspelt name is an error, not None
+        ls.mixr
+    with pytest.raises(TypeError):
+        ls.parts["mixer"] = ls.mixer                                       # the spec is read-only
+    assert hash(spec) == hash(config_from_dict(preset("tinyA")).to_spec()) and spec == config_from_dict(preset("tinyA")).to_spec()
     block = Model(spec).layers[0]
     assert block.mixer.position is block.position and [type(p).__name__ for p in block.parts()] == \
         ["RMSNorm", "GQAttention", "RMSNorm", "SwiGLU"]
-    assert block.cache_need() == KVNeed(2, 16, None) and block.state_need() is None and block.graph_safe()
-    assert block.cache_need() == CacheNeed((PageTensor("k", 2, 16), PageTensor("v", 2, 16)), None)
+    # what a mixer declares does not depend on whether it is loaded or in which type: values may be kept
+    # transposed for pages of a multiple of 16 tokens in bfloat16, and the pool decides
+    need = CacheNeed((PageTensor("k", 2, 16), PageTensor("v", 2, 16, 16, torch.bfloat16)), None)
+    assert block.cache_need() == need == KVNeed(2, 16, None, 16, torch.bfloat16)
+    assert block.state_need() is None and block.graph_safe()
 
     def model_with(parts):
         return Model(ModelSpec(spec.architecture, spec.hidden_size, spec.vocab_size, spec.embedding,
@@ -224,5 +232,6 @@ def test_a_layer_names_its_parts_and_the_arrangement_says_which_it_takes():
         model_with({k: v for k, v in parts.items() if k != "feed_forward_norm"})
     no_position = model_with({k: v for k, v in parts.items() if k != "position"})
     assert no_position.layers[0].position is None and no_position.layers[0].mixer.position is None
+    assert no_position.spec.layers[0].parts.get("position") is None
     with pytest.raises(ValueError, match="each name once"):
         CacheNeed((PageTensor("k", 1, 8), PageTensor("k", 1, 8)))

@@ -210,7 +210,9 @@ def test_hip_graph_decode_equals_eager(tiny, eng, dtype):
     seqs = {i: [int(t) for t in rng.integers(0, cfg["vocab_size"], n)] for i, n in enumerate((40, 29, 37))}
     runs = {}
     for graphs in (False, True):
-        r = load_runner(d, dtype=dtype, page_size=16, num_pages=12, max_requests=4, max_len=64, hip_graphs=graphs)
+        # decode steps only: a portion replayed from its bucket's graph runs products of other row counts
+        r = load_runner(d, dtype=dtype, page_size=16, num_pages=12, max_requests=4, max_len=64, hip_graphs=graphs,
+                        graph_portion_tokens=0)
         out = []
         out.append(r.step([StepEntry(0, seqs[0][:20], [19])]).cpu())                       # eager: a prompt
         for p in range(20, 26):

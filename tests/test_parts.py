@@ -100,7 +100,7 @@ def test_attention_part_in_portions(fw, nh, nkv, d, window, page_size):
     t = random_for(part, 3, fw, std=0.4)
     rt = rt_for(fw, torch.float32)
     part.load(getter(t, fw, rt), rt)
-    assert part.cache_need() == fw.parts.KVNeed(nkv, d, window)
+    assert part.cache_need() == fw.parts.KVNeed(nkv, d, window, 16, torch.bfloat16)    # loaded or not, whatever the type
     h = torch.randn(T, H)
     w = {k: v.double() for k, v in t.items()}
     cfg = {"num_heads": nh, "num_kv_heads": nkv, "head_dim": d}
@@ -115,16 +115,18 @@ def test_attention_part_in_portions(fw, nh, nkv, d, window, page_size):
         want = o.transpose(0, 1).reshape(T, nh * d) @ w["a.o_proj.weight"].T
     layout = fw.cache.CacheLayout([(part.cache_need(), None, None)])
     m = fw.cache.CacheManager(layout, page_size, 20, 2, 64)
-    pools = fw.cache.CachePools(layout, page_size, 20, 2, rt)
+    pools = fw.cache.CachePools(layout, page_size, 20, 2, rt, m.max_pages_per_request)
     for t in pools.pages[0].values():
         t.fill_(1e4)                                         # what a reused page may hold must not matter
-    builder = fw.engine.BatchBuilder(m, 1000, rt.device)
+    builder = fw.engine.BatchBuilder(m, pools, 1000, rt.device)
+    m.add("other")                                           # so that the request's table row is not row 0
     m.add("x")
     got, p = [], 0
     for n in (23, 2, 24, 1):
         m.grow("x", p + n)
-        ctx, tables, slots = builder.build([fw.engine.StepEntry("x", [1] * n, [])])
-        got.append(part.forward(h[p:p + n].to(DEV), ctx, pools.kv_view(0, tables[0], slots[0]), None).cpu())
+        b = builder.build([fw.engine.StepEntry("x", [1] * n, [])])
+        ctx = b.ctx
+        got.append(part.forward(h[p:p + n].to(DEV), ctx, pools.kv_view(0, ctx.state_slots, b.slots[0]), None).cpu())
         p += n
         m.advance("x", p)
     torch.testing.assert_close(torch.cat(got).double(), want, atol=2e-4, rtol=2e-4)
@@ -140,9 +142,9 @@ def register_toys(fw):
     class ToyDecay(parts.Mixer):
         """state <- decay * state + W_in h_t ; seen <- seen + 1 ; out_t = W_out state / (1 + seen / 100)
         Two states of fixed size per request, of different types.  Single tokens are handled with device tensors
-        only, so a decode step of this mixer can be captured into a graph."""
+        only, so a decode step of this mixer can be captured into a graph; portions walk the requests on the host."""
 
-        graph_safe = True
+        graph_safe = "decode"
 
         def __init__(self, prefix, position, hidden_size, state_size, decay):
             self.prefix, self.H, self.S, self.decay = prefix, hidden_size, state_size, decay
@@ -213,7 +215,7 @@ def register_toys(fw):
             o = 0
             for r, (n, start) in enumerate(zip(ctx.q_lens_host, ctx.start_pos_host)):
                 held = -(-(start + n) // pages.shape[2])
-                c = pages[kv.block_table[r, :held].long()].reshape(-1, self.r)[:start + n].float()
+                c = pages[kv.pages_of(r)[:held].long()].reshape(-1, self.r)[:start + n].float()
                 scores = (q[o:o + n] @ (c @ self.wk.T).T) / math.sqrt(self.dk)
                 j = torch.arange(start + n, device=x.device)[None, :]
                 i = torch.arange(start, start + n, device=x.device)[:, None]
@@ -541,15 +543,16 @@ def test_rotary_part_and_block_alone(fw):
     want = P.decoder_layer(x.double(), w, 0, cfg, cos, sin)
     layout = fw.cache.CacheLayout(model.run_needs())
     m = fw.cache.CacheManager(layout, 4, 20, 2, 32)
-    pools = fw.cache.CachePools(layout, 4, 20, 2, rt)
-    builder = fw.engine.BatchBuilder(m, 50, rt.device)
+    pools = fw.cache.CachePools(layout, 4, 20, 2, rt, m.max_pages_per_request)
+    builder = fw.engine.BatchBuilder(m, pools, 50, rt.device)
     m.add("x")
     got, p = [], 0
     for n in (13, 8):
         m.grow("x", p + n)
-        ctx, tables, slots = builder.build([fw.engine.StepEntry("x", [1] * n, [])])
+        b = builder.build([fw.engine.StepEntry("x", [1] * n, [])])
+        ctx = b.ctx
         xs = x[p:p + n].to(DEV).clone()
-        pending = block.forward(xs, None, ctx, pools.kv_view(0, tables[0], slots[0]), None)
+        pending = block.forward(xs, None, ctx, pools.kv_view(0, ctx.state_slots, b.slots[0]), None)
         got.append((xs if pending is None else xs + pending.float()).cpu())
         p += n
         m.advance("x", p)

@@ -61,6 +61,16 @@ def run_replay(model_dir, dtype, steps, out, max_tokens, page_size=16):
     assert log.getvalue().split() == [x for st in steps for x in ("done", str(st["step"]))]
     runner.manager.check_invariants()
     assert all(g.allocator.num_in_use() == 0 for g in runner.manager.groups), "a finished request kept pages"
+    if dtype == "bfloat16":
+        # the serving path: steps are replayed from captured graphs, single tokens and portions alike
+        g = runner.graphs
+        assert g is not None and g.launches > 0 and g.max_portion_tokens > 0
+        n_steps = sum(1 for st in steps if st["entries"])
+        small = sum(1 for st in steps if st["entries"] and (sum(len(e["tokens"]) for e in st["entries"]) <= g.max_portion_tokens
+                                                            or all(len(e["tokens"]) == 1 for e in st["entries"])))
+        assert g.launches == small, f"{g.launches} of {n_steps} steps were replayed from graphs, {small} could have been"
+    else:
+        assert runner.graphs is None
     return runner
 
 
