@@ -10,9 +10,14 @@ uses once plus the cache of the live requests); ``points`` holds decode throughp
 ``launch`` says how many decode steps one graph launch holds and what it costs the host to enqueue it against
 the whole launch (a step bound by launching would show the two close together).  Every graph is captured
 when the engine is built, before any timer starts; ``launch.graphs_captured_while_timed`` is asserted to be 0.
-``roofline.measured_peak`` is the bandwidth a plain streaming read of 2 GiB reaches on this device (the
-reference measures its own the same way, benchmarks/diag_gpu_launch.py:29-40); fractions are against the
-published peak.
+``roofline.measured_peak`` is the bandwidth a plain streaming read of 2 GiB reaches on this device and
+``prefill.measured_peak_tflops`` the rate of a large square bfloat16 product on its matrix cores (the reference
+measures its own denominators the same way, benchmarks/diag_gpu_launch.py:29-40, benchmarks/bench_micro.py:49-51);
+fractions are against the published peaks.  After the headline the default run measures the two larger shapes
+the same way, all their layers with weights drawn on the GPU: ``shapes["7b"]`` (decode at batch 8 and 64, the
+2,048-token prompt, a queue of 64 requests with prompts of 128 to 4,096 tokens and 256 decoded each) and
+``shapes["32b"]`` (the prompt, decode at batch 1, 8 and 64 after 1,024-token prompts); ``--no-shapes`` leaves
+them out.  ``--only sample`` times the sampler alone at the real vocabulary.
 """
 from __future__ import annotations
 
@@ -126,6 +131,59 @@ def measure_read_gbs(repeats=5):
     return x.numel() * 2 / best / 1e9
 
 
+def measure_matrix_tflops(n=8192, repeats=5):
+    """TFLOP/s of one n x n x n bfloat16 product on the matrix cores (the tiled kernel of this library and the
+    library's own, whichever is faster), best of ``repeats``."""
+    import torch
+
+    from llm_infrence_engine_amd.kernels import ops
+
+    g = torch.Generator(device="cuda:0").manual_seed(0)
+    a = torch.randn(n, n, generator=g, device="cuda:0").bfloat16()
+    w = torch.randn(n, n, generator=g, device="cuda:0").bfloat16()
+    best = None
+    for fn in (lambda: ops.gemm_tiled(a, w), lambda: torch.mm(a, w.t())):
+        for i in range(repeats + 1):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            fn()
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            if i > 0:
+                best = dt if best is None else min(best, dt)
+    return 2.0 * n ** 3 / best / 1e12
+
+
+def run_sampler(vocab, batches=(8, 64), repeats=20):
+    """Microseconds one call of the sampling kernel takes for a batch of rows at the real vocabulary: greedy, and
+    temperature 0.8 with top-k 50 and top-p 0.9."""
+    import torch
+
+    from llm_infrence_engine_amd.kernels import ops
+
+    out = {}
+    g = torch.Generator(device="cuda:0").manual_seed(1)
+    for b in batches:
+        logits = torch.randn(b, vocab, generator=g, device="cuda:0") * 3.0
+        tok = torch.empty(b, dtype=torch.int32, device="cuda:0")
+        temp = torch.full((b,), 0.8, device="cuda:0")
+        top_k = torch.full((b,), 50, dtype=torch.int32, device="cuda:0")
+        top_p = torch.full((b,), 0.9, device="cuda:0")
+        seeds = torch.arange(b, dtype=torch.int64, device="cuda:0") + 7
+        draw = torch.zeros(b, dtype=torch.int32, device="cuda:0")
+        for name, fn in (("greedy", lambda: ops.sample(logits, tok)),
+                         ("top_k50_top_p0.9", lambda: ops.sample(logits, tok, temp, top_k, top_p, seeds, draw)),
+                         ("temperature_only", lambda: ops.sample(logits, tok, temp, None, None, seeds, draw))):
+            fn()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(repeats):
+                fn()
+            torch.cuda.synchronize()
+            out[f"b{b}_{name}_us"] = round((time.perf_counter() - t0) / repeats * 1e6, 1)
+    return out
+
+
 def run_prefill(eng_mod, model, vocab, seed, repeats=5):
     import numpy as np
     import torch
@@ -192,9 +250,11 @@ def main() -> int:
                     help="fewer layers than the configuration has, if memory or time needs it (both numbers are reported)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 decode points and the prefill")
     ap.add_argument("--prompt-len", type=int, default=PROMPT_LEN, help="prompt length of the decode run (default 512)")
-    ap.add_argument("--only", choices=["prefill", "serve"],
-                    help="run one part alone: the 2,048-token prefill (for profiles), or a queue of 64 requests with "
-                         "prompts of 128 to 4,096 tokens and 256 decoded tokens each through the scheduler")
+    ap.add_argument("--no-shapes", action="store_true", help="skip the 7B and 32B shapes that follow the headline")
+    ap.add_argument("--only", choices=["prefill", "serve", "sample"],
+                    help="run one part alone: the 2,048-token prefill (for profiles), a queue of 64 requests with "
+                         "prompts of 128 to 4,096 tokens and 256 decoded tokens each through the scheduler, or the "
+                         "sampling kernel at the real vocabulary")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(f"bench.py measures one GPU; --gpus {a.gpus} is not supported by this single-GPU engine")
@@ -224,6 +284,10 @@ def main() -> int:
         print(json.dumps({"serving": run_serving(eng, model, vocab, seed=5)}), flush=True)
         return 0
 
+    if a.only == "sample":
+        print(json.dumps({"sampler": run_sampler(vocab)}), flush=True)
+        return 0
+
     dt, ctx, launch = run_decode(eng, model, a.batch, a.steps, a.warmup, vocab, seed=1, prompt_len=a.prompt_len)
     value = a.batch / dt
     gbs = decode_bytes(cfg, a.batch, ctx) / dt / 1e9
@@ -249,18 +313,64 @@ def main() -> int:
         "launch": launch,
     }
     if not a.no_points:
-        pt = run_prefill(eng, model, vocab, seed=2)
-        tf = prefill_flops(cfg, PREFILL_TOKENS) / pt / 1e12
-        out["prefill"] = {"value": round(PREFILL_TOKENS / pt, 1), "tokens": PREFILL_TOKENS, "ms": round(pt * 1e3, 3),
-                          "frac": round(tf / PEAK_TFLOPS["bf16"], 4)}
-        points = {}
+        out["prefill"] = prefill_point(eng, model, cfg, vocab)
+        out["prefill"]["measured_peak_tflops"] = round(measure_matrix_tflops(), 1)
+        out["points"] = {}
         for b in (1, 64):
-            steps = min(a.steps, 128)
-            dtb, _, _ = run_decode(eng, model, b, steps, min(a.warmup, 8), vocab, seed=3 + b)
-            points[f"decode_b{b}"] = round(b / dtb, 1)
-        out["points"] = points
+            out["points"].update(decode_point(eng, model, cfg, b, min(a.steps, 128), min(a.warmup, 8), vocab, a.prompt_len))
+        out["sampler"] = run_sampler(vocab)
+    if a.shape == "0.5b" and not a.no_points and not a.no_shapes and a.layers == shape["num_hidden_layers"]:
+        del model
+        out["shapes"] = {}
+        for name, prompt_len, batches, serve in (("7b", PROMPT_LEN, (8, 64), True), ("32b", 1024, (1, 8, 64), False)):
+            out["shapes"][name] = measure_shape(eng, name, prompt_len, batches, serve)
     print(json.dumps(out), flush=True)
     return 0
+
+
+def prefill_point(eng, model, cfg, vocab):
+    pt = run_prefill(eng, model, vocab, seed=2)
+    tf = prefill_flops(cfg, PREFILL_TOKENS) / pt / 1e12
+    return {"value": round(PREFILL_TOKENS / pt, 1), "tokens": PREFILL_TOKENS, "ms": round(pt * 1e3, 3),
+            "frac": round(tf / PEAK_TFLOPS["bf16"], 4)}
+
+
+def decode_point(eng, model, cfg, batch, steps, warmup, vocab, prompt_len):
+    """decode_b<batch>: tokens a second, with the step's time and its fraction of the published HBM bandwidth."""
+    dt, ctx, _ = run_decode(eng, model, batch, steps, warmup, vocab, seed=3 + batch, prompt_len=prompt_len)
+    gbs = decode_bytes(cfg, batch, ctx) / dt / 1e9
+    return {f"decode_b{batch}": round(batch / dt, 1), f"decode_b{batch}_ms_per_step": round(dt * 1e3, 4),
+            f"decode_b{batch}_frac": round(gbs / HBM_GBS, 4)}
+
+
+def measure_shape(eng, name, prompt_len, batches, serve):
+    """Another shape measured as the headline is: all its layers, weights drawn on the GPU."""
+    import gc
+
+    import torch
+
+    from llm_infrence_engine_amd.config import config_from_dict, preset
+
+    gc.collect()
+    torch.cuda.empty_cache()
+    cfg = config_from_dict(preset(name))
+    t0 = time.perf_counter()
+    model = eng.load_random_model(cfg, seed=0, dtype="bfloat16", device="cuda:0")
+    torch.cuda.synchronize()
+    out = {"layers": cfg.num_hidden_layers, "hidden": cfg.hidden_size, "prompt_len": prompt_len,
+           "load_s": round(time.perf_counter() - t0, 1), "roofline_bound": "hbm", "roofline_peak_gbs": HBM_GBS}
+    out["prefill"] = prefill_point(eng, model, cfg, cfg.vocab_size)
+    for b in batches:
+        out.update(decode_point(eng, model, cfg, b, 64, 8, cfg.vocab_size, prompt_len))
+    if serve:
+        run_serving(eng, model, cfg.vocab_size, seed=4, n_requests=8, new_tokens=16)       # warms up graphs and the library
+        sv = run_serving(eng, model, cfg.vocab_size, seed=5)
+        out["serve_64_mixed"] = {k: sv[k] for k in ("seconds", "prompt_tokens", "new_tokens", "all_tokens_per_s",
+                                                    "new_tokens_per_s", "preemptions", "ttft_p50_s", "tpot_mean_ms")}
+    del model
+    gc.collect()
+    torch.cuda.empty_cache()
+    return out
 
 
 if __name__ == "__main__":
