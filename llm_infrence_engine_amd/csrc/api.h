@@ -126,8 +126,11 @@ void ms_argmax_static_limits(int* max_rows, int* max_chunks);
 int ms_argmax_static(const float* logits, long long ld, int n_rows, int vocab, int n_chunks, int* out,
                      hipStream_t stream);
 
+// workspace: ms_sample_workspace_bytes(n_rows) bytes of device memory (any contents); use_top_k / use_top_p: 0 if
+// no row has a top_k in (0, vocab) / a top_p below 1.
+long long ms_sample_workspace_bytes(int n_rows);
 int ms_sample(const float* logits, long long ld, int n_rows, int vocab, const float* temperature, const int* top_k,
-              const float* top_p, const unsigned long long* seeds, const int* draw_index, int* out,
-              hipStream_t stream);
+              const float* top_p, const unsigned long long* seeds, const int* draw_index, int* out, void* workspace,
+              int use_top_k, int use_top_p, hipStream_t stream);
 
 }  // extern "C"

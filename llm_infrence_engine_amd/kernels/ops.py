@@ -64,7 +64,9 @@ _SIGNATURES = {
                                        _c_ll, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
                                        _c_int, _c_int, _c_int, _c_ptr],
     "ms_argmax": [_c_ptr, _c_ll, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr],
-    "ms_sample": [_c_ptr, _c_ll, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
+    "ms_sample": [_c_ptr, _c_ll, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
+                  _c_ptr],
+    "ms_sample_workspace_bytes": [_c_int],
 }
 
 _fn = {}
@@ -720,13 +722,18 @@ def paged_attention_mfma(q: torch.Tensor, k_pages: torch.Tensor, vt_pages: torch
 
 def sample(logits: torch.Tensor, out: torch.Tensor, temperature: Optional[torch.Tensor] = None,
            top_k: Optional[torch.Tensor] = None, top_p: Optional[torch.Tensor] = None,
-           seeds: Optional[torch.Tensor] = None, draw_index: Optional[torch.Tensor] = None) -> torch.Tensor:
+           seeds: Optional[torch.Tensor] = None, draw_index: Optional[torch.Tensor] = None,
+           use_top_k: bool = True, use_top_p: bool = True) -> torch.Tensor:
     """One token per row of float32 logits [M, V].  Without ``temperature`` (or where it is <= 0) the first
-    maximum; else a draw after top-k and top-p, repeatable from (seeds[r], draw_index[r])."""
+    maximum; else a draw after top-k and top-p, repeatable from (seeds[r], draw_index[r]).  ``use_top_k`` /
+    ``use_top_p`` False: the caller knows that no row has a top_k in (0, V) / a top_p below 1, and the kernels
+    that look for those thresholds are left out."""
     _check(logits, "logits", torch.float32)
     M, V = logits.shape
     _check(out, "out", torch.int32, (M,))
-    if temperature is None and M <= 65535:
+    if M > 65535:
+        raise ValueError("at most 65,535 rows to a call")
+    if temperature is None:
         n_chunks = max(1, min(128, V // 1024))
         val = torch.empty((M, n_chunks), dtype=torch.float32, device=logits.device)
         idx = torch.empty((M, n_chunks), dtype=torch.int32, device=logits.device)
@@ -737,8 +744,12 @@ def sample(logits: torch.Tensor, out: torch.Tensor, temperature: Optional[torch.
                         (draw_index, "draw_index", torch.int32)):
         if t is not None:
             _check(t, name, dt, (M,))
-    _call("ms_sample", logits.data_ptr(), V, M, V, _ptr(temperature), _ptr(top_k), _ptr(top_p), _ptr(seeds),
-          _ptr(draw_index), out.data_ptr(), _stream())
+    f = _get("ms_sample_workspace_bytes")
+    f.restype = _c_ll
+    work = torch.empty(int(f(M)), dtype=torch.uint8, device=logits.device)
+    _call("ms_sample", logits.data_ptr(), V, M, V, temperature.data_ptr(), _ptr(top_k), _ptr(top_p), _ptr(seeds),
+          _ptr(draw_index), out.data_ptr(), work.data_ptr(), int(use_top_k and top_k is not None),
+          int(use_top_p and top_p is not None), _stream())
     return out
 
 

@@ -45,6 +45,8 @@ class Sampler:
             f = torch.tensor([[r.temperature, r.top_p] for r in requests], dtype=torch.float32).to(dev)
             i = torch.tensor([[r.top_k, len(r.output_ids)] for r in requests], dtype=torch.int32).to(dev)
             seeds = torch.tensor([r.sample_seed & 0x7FFFFFFFFFFFFFFF for r in requests], dtype=torch.int64).to(dev)
+            V = logits.shape[1]
             ops.sample(logits, out, f[:, 0].contiguous(), i[:, 0].contiguous(), f[:, 1].contiguous(), seeds,
-                       i[:, 1].contiguous())
+                       i[:, 1].contiguous(), use_top_k=any(0 < r.top_k < V for r in requests),
+                       use_top_p=any(r.top_p < 1.0 for r in requests))
         return out.tolist()

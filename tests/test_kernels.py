@@ -247,6 +247,84 @@ def test_sample_greedy_and_vectors(ops):
     assert out.tolist() == big.argmax(-1).tolist()
 
 
+def _draws_of_row(ops, row, n, temperature, top_k, top_p, seed=5, first_draw=0):
+    """``n`` draws from one row of logits: the row repeated, each copy with a draw index of its own."""
+    V = row.numel()
+    lg = row.to(DEV).float().expand(n, V).contiguous()
+    out = torch.empty(n, dtype=torch.int32, device=DEV)
+    ops.sample(lg, out, torch.full((n,), temperature, device=DEV), torch.full((n,), top_k, dtype=torch.int32, device=DEV),
+               torch.full((n,), top_p, device=DEV), torch.full((n,), seed, dtype=torch.int64, device=DEV),
+               torch.arange(first_draw, first_draw + n, dtype=torch.int32, device=DEV))
+    return out.cpu().long()
+
+
+@pytest.mark.parametrize("V", [50, 1000, 151936])
+@pytest.mark.parametrize("temperature,top_k,top_p", [(0.8, 50, 0.9), (1.3, 0, 0.7), (1.0, 5, 1.0), (1.0, 0, 1.0), (0.5, 7, 0.3)])
+def test_sampler_draws_from_the_plain_distribution(ops, V, temperature, top_k, top_p):
+    """Draws land only on tokens the plain rule keeps (temperature, top-k, top-p in the reference's order,
+    src/miniserve/sampler.py:23-41) and as often as its probabilities say."""
+    from tests.plain import qwen2_plain as P
+
+    g = torch.Generator().manual_seed(V + top_k)
+    row = torch.randn(V, generator=g) * 2.5
+    want = P.logits_to_probs(row[None], temperature, top_k, top_p)[0]
+    n = 8192
+    got = _draws_of_row(ops, row, n, temperature, top_k, top_p)
+    kept = (want > 0).nonzero().flatten()
+    assert set(got.tolist()) <= set(kept.tolist()), "a token was drawn that the plain rule drops"
+    freq = torch.bincount(got, minlength=V).double() / n
+    # the tokens that carry the mass: each within five standard deviations of its probability
+    for tok in want.topk(min(20, kept.numel())).indices.tolist():
+        pr = float(want[tok])
+        assert abs(float(freq[tok]) - pr) < 5 * math.sqrt(pr * (1 - pr) / n) + 2e-4, (tok, pr, float(freq[tok]))
+    if kept.numel() <= 64:                                  # few enough that every kept token should appear
+        assert (freq[kept] > 0).all() or float(want[kept].min()) * n < 8
+
+
+def test_sampler_ties_thresholds_and_mixed_rows(ops):
+    """Ties at the k-th value are all kept; the token at which the running mass reaches top_p is kept with all its
+    equals; top_k = 1 and a tiny top_p are the greedy choice; rows without temperature take the first maximum
+    beside rows that draw; and a draw does not depend on the rows beside it (nor on how many blocks a row is
+    spread over)."""
+    row = torch.tensor([1.0, 3.0, 2.0, 2.0, 0.5, 2.0, -1.0, 3.0])
+    got = _draws_of_row(ops, row, 2048, 1.0, 3, 1.0)               # the third largest is 2.0, three times: five tokens stay
+    assert set(got.tolist()) == {1, 2, 3, 5, 7}
+    got = _draws_of_row(ops, row, 2048, 1.0, 0, 0.59)              # the two 3.0s hold 0.599 of the mass: they stay, nothing else
+    assert set(got.tolist()) == {1, 7}
+    got = _draws_of_row(ops, row, 2048, 1.0, 0, 0.61)              # a little more: the three 2.0s come in together
+    assert set(got.tolist()) == {1, 2, 3, 5, 7}
+    assert set(_draws_of_row(ops, row, 256, 2.0, 1, 1.0).tolist()) == {1, 7}      # both maxima tie at k = 1
+    g = torch.Generator().manual_seed(3)
+    big = torch.randn(151936, generator=g) * 3
+    assert set(_draws_of_row(ops, big, 64, 1.5, 1, 1.0).tolist()) == {int(big.argmax())}
+    assert set(_draws_of_row(ops, big, 64, 1.0, 0, 1e-6).tolist()) == {int(big.argmax())}
+    # mixed rows, and the same draws alone and in company
+    rows = torch.stack([big, big.flip(0), big * 0.5, big])
+    lg = rows.to(DEV)
+    temp = torch.tensor([0.9, 0.0, 1.2, -1.0], device=DEV)
+    k = torch.tensor([40, 40, 0, 3], dtype=torch.int32, device=DEV)
+    pp = torch.tensor([0.95, 0.5, 0.8, 0.9], device=DEV)
+    seeds = torch.tensor([11, 12, 13, 14], dtype=torch.int64, device=DEV)
+    draw = torch.tensor([3, 3, 9, 0], dtype=torch.int32, device=DEV)
+    out = torch.empty(4, dtype=torch.int32, device=DEV)
+    ops.sample(lg, out, temp, k, pp, seeds, draw)
+    together = out.tolist()
+    assert together[1] == int(rows[1].argmax()) and together[3] == int(rows[3].argmax())
+    for r in (0, 2):
+        alone = torch.empty(1, dtype=torch.int32, device=DEV)
+        ops.sample(lg[r:r + 1].contiguous(), alone, temp[r:r + 1], k[r:r + 1], pp[r:r + 1], seeds[r:r + 1], draw[r:r + 1])
+        assert alone.item() == together[r]
+        many = torch.empty(200, dtype=torch.int32, device=DEV)          # 200 rows: fewer blocks to a row
+        ops.sample(lg[r:r + 1].expand(200, -1).contiguous(), many, temp[r:r + 1].expand(200).contiguous(),
+                   k[r:r + 1].expand(200).contiguous(), pp[r:r + 1].expand(200).contiguous(),
+                   seeds[r:r + 1].expand(200).contiguous(), draw[r:r + 1].expand(200).contiguous())
+        assert set(many.tolist()) == {together[r]}
+    # a row that holds nothing to draw from falls back to index 0, like the greedy choice
+    nothing = torch.full((1, 5000), float("-inf"), device=DEV)
+    ops.sample(nothing, alone, temp[:1], k[:1], pp[:1], seeds[:1], draw[:1])
+    assert alone.item() == 0
+
+
 def test_argmax_in_two_stages(ops):
     """Ties across and inside the slices of the first stage go to the smallest index; a row of -inf or NaN gives
     index 0; vocabularies that are no multiple of the slice count."""
@@ -338,6 +416,320 @@ def test_table_update_and_zero_rows(ops):
         assert live.tolist() == [True, True, False, True, False, True, True, False, True]
         ops.zero_rows(t, rows)
         assert float(t.reshape(9, -1)[0].float().abs().sum()) == 0
+
+
+def _draws(ops, logits, n, temperature=1.0, top_k=0, top_p=1.0, seed=0):
+    M = n
+    lg = logits.to(DEV).expand(M, -1).contiguous()
+    out = torch.empty(M, dtype=torch.int32, device=DEV)
+    ops.sample(lg, out, torch.full((M,), temperature, device=DEV), torch.full((M,), top_k, dtype=torch.int32, device=DEV),
+               torch.full((M,), top_p, device=DEV), torch.full((M,), seed, dtype=torch.int64, device=DEV),
+               torch.arange(M, dtype=torch.int32, device=DEV))
+    return out.cpu()
+
+
+def test_sample_distribution_and_filters(ops):
+    # vectors of the reference's tests/test_sampler.py
+    assert set(_draws(ops, torch.tensor([[0.1, 2.0, 0.5]]), 20, top_k=1).tolist()) == {1}
+    assert set(_draws(ops, torch.tensor([[2.0, 1.0, 0.0, -1.0]]), 300, top_p=0.7).tolist()) == {0, 1}
+    assert set(_draws(ops, torch.tensor([[10.0, 0.0, 0.0]]), 50, top_p=1e-4).tolist()) == {0}
+    d = _draws(ops, torch.log(torch.tensor([[0.7, 0.2, 0.1]])), 4000, seed=123)
+    freq = torch.bincount(d, minlength=3).float() / 4000
+    assert torch.allclose(freq, torch.tensor([0.7, 0.2, 0.1]), atol=0.03)
+    # temperature sharpens: T = 0.5 squares the odds
+    d = _draws(ops, torch.log(torch.tensor([[0.5, 0.5 / 3]])), 4000, temperature=0.5, seed=5)
+    assert abs((d == 0).float().mean().item() - 0.9) < 0.03
+    # same seed and draw index, same token; top-k = 2 on a wide row leaves two tokens
+    row = torch.randn(1, 5000, generator=torch.Generator().manual_seed(8))
+    a, b = _draws(ops, row, 64, seed=9), _draws(ops, row, 64, seed=9)
+    assert torch.equal(a, b) and len(set(a.tolist())) > 10
+    top2 = set(row[0].topk(2).indices.tolist())
+    assert set(_draws(ops, row, 200, top_k=2, seed=1).tolist()) == top2
+
+
+def test_ops_refuse_cpu_tensors_and_wrong_shapes(ops):
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        ops.silu_mul(torch.zeros(2, 4), torch.zeros(2, 2))
+    with pytest.raises(ValueError):
+        ops.silu_mul(torch.zeros(2, 4, device=DEV), torch.zeros(2, 3, device=DEV))
+    with pytest.raises(RuntimeError, match="unsupported"):
+        kp = torch.zeros(2, 1, 4, 6, device=DEV)  # head size 6 is no multiple of 4
+        ops.paged_attention_generic(torch.zeros(1, 6, device=DEV), kp, kp, torch.zeros(1, 1, dtype=torch.int32, device=DEV),
+                                    torch.zeros(1, dtype=torch.int32, device=DEV), torch.zeros(1, dtype=torch.int32, device=DEV),
+                                    torch.zeros(1, 6, device=DEV), 1, 1.0)
+
+
+@pytest.mark.parametrize("M", [1, 8, 16, 17, 33, 64])
+@pytest.mark.parametrize("N,K", [(1152, 896), (331, 72), (896, 4864), (50, 200), (9728, 104), (17000, 64)])
+def test_gemm_skinny(ops, M, N, K):
+    g = torch.Generator().manual_seed(M * 1000 + N)
+    a = torch.randn(M, K, generator=g).bfloat16().to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16().to(DEV)
+    bias = torch.randn(N, generator=g).to(DEV)
+    want = a.double() @ w.double().T
+    out = ops.gemm_skinny(a, w, bias)
+    torch.testing.assert_close(out.double(), want + bias.double(), **tol(torch.bfloat16))
+    f = ops.gemm_skinny(a, w, None, out_dtype=torch.float32)
+    assert f.dtype == torch.float32
+    torch.testing.assert_close(f.double(), want, atol=2e-5, rtol=2e-5)
+    x = torch.randn(M, N, generator=g).to(DEV)
+    x0 = x.clone()
+    ops.gemm_skinny(a, w, bias, ops.EPI_RESIDUAL, residual=x)
+    torch.testing.assert_close(x.double(), x0.double() + want + bias.double(), atol=2e-5, rtol=2e-5)
+    if N % 2 == 0:
+        act = ops.gemm_skinny(a, w, None, ops.EPI_SWIGLU)
+        wantact = torch.nn.functional.silu(want[:, 0::2]) * want[:, 1::2]
+        torch.testing.assert_close(act.double(), wantact, **tol(torch.bfloat16))
+    # a row slice of a wider matrix, and the same row alone: the same bits whatever else is in the batch
+    wide = torch.zeros(M, K + 8, dtype=torch.bfloat16, device=DEV)
+    wide[:, :K] = a
+    assert torch.equal(ops.gemm_skinny(wide[:, :K], w, bias), out)
+    assert torch.equal(ops.gemm_skinny(a[M - 1:], w, bias), out[M - 1:])
+
+
+@pytest.mark.parametrize("M", [3, 40])
+@pytest.mark.parametrize("shape", [(4, 4, 0), (4, 8, 0), (3, 4, 0), (3, 8, 0), (2, 8, 0), (2, 16, 0), (1, 8, 0), (1, 16, 0),
+                                   (4, 8, 1), (3, 8, 1), (2, 8, 2)])
+def test_gemm_skinny_block_shapes(ops, M, shape):
+    """Every block shape on offer (tiles per block, waves, token groups per block) gives the same numbers (to
+    float rounding of another summation order), also with the gated epilogue and the folded norm.  A forced
+    shape also keeps few rows in this kernel; unforced they go to the streaming kernel, which must agree."""
+    from llm_infrence_engine_amd.kernels import build
+
+    lib = build.load()
+    g = torch.Generator().manual_seed(sum(shape) + M)
+    N, K = 1000, 1544
+    a = torch.randn(M, K, generator=g).bfloat16().to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16().to(DEV)
+    bias = torch.randn(N, generator=g).to(DEV)
+    want = a.double() @ w.double().T + bias.double()
+    x0 = torch.randn(M, N, generator=g).to(DEV)
+    try:
+        lib.ms_gemm_skinny_force(*shape)
+        x = x0.clone()
+        try:
+            ops.gemm_skinny(a, w, bias, ops.EPI_RESIDUAL, residual=x)
+        except RuntimeError as e:      # a shape that does not fit LDS with this many token groups is refused
+            assert "unsupported" in str(e) and (shape[1] - 1) * shape[0] * (shape[2] or (1 if M <= 16 else 4)) > 60
+            return
+        torch.testing.assert_close(x.double(), x0.double() + want, atol=3e-5, rtol=3e-5)
+        f = ops.gemm_skinny(a, w, bias, out_dtype=torch.float32)
+        torch.testing.assert_close(f.double(), want, atol=3e-5, rtol=3e-5)
+        # gated epilogue over interleaved rows, norm folded in: against the default shape
+        x32 = torch.randn(M, K, generator=g).to(DEV)
+        nw = (1 + 0.1 * torch.randn(K, generator=g)).to(DEV)
+        got = ops.gemm_skinny_norm(x32, nw, 1e-6, w, None, ops.EPI_SWIGLU)
+        lib.ms_gemm_skinny_force(0, 0, 0)
+        ref = ops.gemm_skinny_norm(x32, nw, 1e-6, w, None, ops.EPI_SWIGLU)
+        torch.testing.assert_close(got.double(), ref.double(), atol=1e-2, rtol=1e-2)
+    finally:
+        lib.ms_gemm_skinny_force(0, 0, 0)
+
+
+@pytest.mark.parametrize("M", [1, 5, 8, 16])
+@pytest.mark.parametrize("N,K", [(896, 4864), (1152, 896), (330, 72), (52, 200), (9728, 904), (1000, 9000), (4000, 2056),
+                                 (16384, 64)])
+def test_gemm_stream(ops, M, N, K):
+    """The streaming kernel at every shape it can compute: one or several stages, a last k-step that K fills in
+    part, one to four tiles of rows to a block, rows that run out in the last block; every epilogue, the folded
+    norm with gathered rows; a row's numbers do not depend on the rest of the batch."""
+    g = torch.Generator().manual_seed(M * 1000 + N + K)
+    a = torch.randn(M, K, generator=g).bfloat16().to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16().to(DEV)
+    bias = torch.randn(N, generator=g).to(DEV)
+    want = a.double() @ w.double().T
+    out = ops.gemm_stream(a, w, bias)
+    torch.testing.assert_close(out.double(), want + bias.double(), **tol(torch.bfloat16))
+    f = ops.gemm_stream(a, w, None, out_dtype=torch.float32)
+    torch.testing.assert_close(f.double(), want, atol=3e-5, rtol=3e-5)
+    x = torch.randn(M, N, generator=g).to(DEV)
+    x0 = x.clone()
+    ops.gemm_stream(a, w, bias, ops.EPI_RESIDUAL, residual=x)
+    torch.testing.assert_close(x.double(), x0.double() + want + bias.double(), atol=3e-5, rtol=3e-5)
+    act = ops.gemm_stream(a, w, None, ops.EPI_SWIGLU)
+    torch.testing.assert_close(act.double(), torch.nn.functional.silu(want[:, 0::2]) * want[:, 1::2], **tol(torch.bfloat16))
+    assert torch.equal(ops.gemm_stream(a[M - 1:], w, bias), out[M - 1:])
+    # the folded norm over gathered rows of a taller residual stream
+    xs = torch.randn(M + 3, K, generator=g).to(DEV)
+    nw = (1 + 0.1 * torch.randn(K, generator=g)).to(DEV)
+    rows = torch.randperm(M + 3, generator=g)[:M].to(torch.int32).to(DEV)
+    xr = xs[rows.long()].double()
+    h = (xr * nw.double()).float().bfloat16().double() * torch.rsqrt((xr * xr).mean(-1, keepdim=True) + 1e-5)
+    got = ops.gemm_stream(xs, w, bias, out_dtype=torch.float32, norm_weight=nw, eps=1e-5, rows=rows)
+    torch.testing.assert_close(got.double(), h @ w.double().T + bias.double(), atol=2e-4, rtol=2e-4)
+    gated = ops.gemm_stream(xs, w, None, ops.EPI_SWIGLU, norm_weight=nw, eps=1e-5, rows=rows)
+    hw = h @ w.double().T
+    torch.testing.assert_close(gated.double(), torch.nn.functional.silu(hw[:, 0::2]) * hw[:, 1::2], **tol(torch.bfloat16))
+
+
+def test_gemm_stream_refuses_what_it_cannot_take(ops):
+    w = torch.zeros(64, 64, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(RuntimeError, match="unsupported"):
+        ops.gemm_stream(torch.zeros(17, 64, dtype=torch.bfloat16, device=DEV), w)            # more than 16 rows
+    with pytest.raises(RuntimeError, match="unsupported"):
+        ops.gemm_stream(torch.zeros(2, 36, dtype=torch.bfloat16, device=DEV),
+                        torch.zeros(8, 36, dtype=torch.bfloat16, device=DEV))                 # K no multiple of 8
+    with pytest.raises(RuntimeError, match="unsupported"):                                   # not the shape it is for
+        ops.gemm_stream(torch.zeros(2, 64, dtype=torch.bfloat16, device=DEV), w, any_shape=False)
+
+
+@pytest.mark.parametrize("M", [17, 32, 41, 64])
+@pytest.mark.parametrize("N,K", [(7000, 96), (4100, 200), (330, 256), (48, 896), (16 * 256 * 17 + 6, 64), (1000, 1000)])
+def test_gemm_panel(ops, M, N, K):
+    """The kernel that holds the activations in LDS, at every shape it can compute: blocks of one tile, of a few
+    tiles whose k-steps several waves share, and of more tiles than waves; a last k-step that K fills in part;
+    rows of W that run out inside the last tile; every epilogue, the folded norm with gathered rows; a row's
+    numbers do not depend on the rest of the batch."""
+    g = torch.Generator().manual_seed(M * 1000 + N + K)
+    a = torch.randn(M, K, generator=g).bfloat16().to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16().to(DEV)
+    bias = torch.randn(N, generator=g).to(DEV)
+    want = a.double() @ w.double().T
+    out = ops.gemm_panel(a, w, bias)
+    torch.testing.assert_close(out.double(), want + bias.double(), **tol(torch.bfloat16))
+    f = ops.gemm_panel(a, w, None, out_dtype=torch.float32)
+    torch.testing.assert_close(f.double(), want, atol=3e-5, rtol=3e-5)
+    x = torch.randn(M, N, generator=g).to(DEV)
+    x0 = x.clone()
+    ops.gemm_panel(a, w, bias, ops.EPI_RESIDUAL, residual=x)
+    torch.testing.assert_close(x.double(), x0.double() + want + bias.double(), atol=3e-5, rtol=3e-5)
+    act = ops.gemm_panel(a, w, None, ops.EPI_SWIGLU)
+    torch.testing.assert_close(act.double(), torch.nn.functional.silu(want[:, 0::2]) * want[:, 1::2], **tol(torch.bfloat16))
+    assert torch.equal(ops.gemm_panel(a[M - 3:], w, bias), out[M - 3:])
+    # the folded norm over gathered rows of a taller residual stream
+    xs = torch.randn(M + 3, K, generator=g).to(DEV)
+    nw = (1 + 0.1 * torch.randn(K, generator=g)).to(DEV)
+    rows = torch.randperm(M + 3, generator=g)[:M].to(torch.int32).to(DEV)
+    xr = xs[rows.long()].double()
+    h = (xr * nw.double()).float().bfloat16().double() * torch.rsqrt((xr * xr).mean(-1, keepdim=True) + 1e-5)
+    got = ops.gemm_panel(xs, w, bias, out_dtype=torch.float32, norm_weight=nw, eps=1e-5, rows=rows)
+    torch.testing.assert_close(got.double(), h @ w.double().T + bias.double(), atol=2e-4, rtol=2e-4)
+    gated = ops.gemm_panel(xs, w, None, ops.EPI_SWIGLU, norm_weight=nw, eps=1e-5, rows=rows)
+    hw = h @ w.double().T
+    torch.testing.assert_close(gated.double(), torch.nn.functional.silu(hw[:, 0::2]) * hw[:, 1::2], **tol(torch.bfloat16))
+
+
+@pytest.mark.parametrize("M,N,K", [(20, 300, 1200), (33, 4100, 1528), (18, 500, 2040),
+                                   (64, 4300, 3584), (40, 700, 5120), (64, 4096 + 16 * 256 * 2, 2600), (17, 90, 4872),
+                                   (50, 16 * 256 * 33 + 40, 2400), (40, 16 * 256 * 50, 1840)])
+def test_gemm_panel_long_rows(ops, M, N, K):
+    """Rows of three and four 512-column parts (with three a quarter of the waves sit the loading out), and rows
+    that do not fit LDS whole and go through it in chunks: a last chunk that is shorter, blocks with whole and
+    shared tiles, two and three whole tiles to a wave."""
+    g = torch.Generator().manual_seed(K)
+    xs = torch.randn(M, K, generator=g).to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16().to(DEV)
+    nw = (1 + 0.1 * torch.randn(K, generator=g)).to(DEV)
+    h = (xs.double() * nw.double()).float().bfloat16().double() * torch.rsqrt((xs.double() ** 2).mean(-1, keepdim=True) + 1e-6)
+    got = ops.gemm_panel(xs, w, None, out_dtype=torch.float32, norm_weight=nw, eps=1e-6)
+    torch.testing.assert_close(got.double(), h @ w.double().T, atol=2e-4, rtol=2e-4)
+    a = xs.bfloat16()
+    plain = ops.gemm_panel(a, w, None, out_dtype=torch.float32)
+    torch.testing.assert_close(plain.double(), a.double() @ w.double().T, atol=3e-5, rtol=3e-5)
+
+
+@pytest.mark.parametrize("M,N,K", [(8, 5120, 13824), (64, 3584, 18944), (33, 5120, 27648), (17, 900, 8200), (64, 16, 9000),
+                                   (5, 8192, 16384)])
+def test_gemm_with_the_columns_split_over_blocks(ops, M, N, K):
+    """Long rows against few of them: blocks take parts of the columns, a second kernel adds the partial sums in
+    order.  Every epilogue that has no gate; a row's numbers do not depend on the rest of the batch; parts of
+    uneven length, a vocabulary-free odd N, one tile only."""
+    from llm_infrence_engine_amd.kernels import build
+    assert build.load().ms_gemm_panel_splitk_parts(M, N, K) > 1
+    g = torch.Generator().manual_seed(M + N + K)
+    a = torch.randn(M, K, generator=g).bfloat16().to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16().to(DEV)
+    bias = torch.randn(N, generator=g).to(DEV)
+    want = a.double() @ w.double().T
+    out = ops.gemm_skinny(a, w, bias)
+    torch.testing.assert_close(out.double(), want + bias.double(), **tol(torch.bfloat16))
+    f = ops.gemm_skinny(a, w, None, out_dtype=torch.float32)
+    torch.testing.assert_close(f.double(), want, atol=5e-5, rtol=5e-5)
+    x = torch.randn(M, N, generator=g).to(DEV)
+    x0 = x.clone()
+    ops.gemm_skinny(a, w, bias, ops.EPI_RESIDUAL, residual=x)
+    torch.testing.assert_close(x.double(), x0.double() + want + bias.double(), atol=5e-5, rtol=5e-5)
+    assert torch.equal(ops.gemm_skinny(a[M - 1:], w, bias), out[M - 1:]) or M > 16   # the same kernel for one row
+    unsplit = ops.gemm_skinny(a, w, None, out_dtype=torch.float32, split_columns=False)
+    torch.testing.assert_close(unsplit.double(), want, atol=5e-5, rtol=5e-5)
+
+
+def test_columns_are_split_only_where_it_pays(ops):
+    from llm_infrence_engine_amd.kernels import build
+    parts = build.load().ms_gemm_panel_splitk_parts
+    assert parts(8, 896, 4864) == 0          # rows too short
+    assert parts(8, 3584, 18944) == 0        # few tokens and a tile for nearly every CU: as well unsplit
+    assert parts(8, 37888, 3584) == 0        # and here, with tiles enough for every CU besides
+    assert parts(65, 3584, 18944) == 0       # too many tokens
+    assert parts(8, 16384, 18944) == 0       # more than two tiles per CU
+
+
+def test_gemm_panel_refuses_what_it_cannot_take(ops):
+    w = torch.zeros(64, 64, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(RuntimeError, match="unsupported"):
+        ops.gemm_panel(torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV), w)             # more than 64 rows
+    with pytest.raises(RuntimeError, match="unsupported"):           # in chunks, and too many tiles to a block
+        ops.gemm_panel(torch.zeros(64, 2400, dtype=torch.bfloat16, device=DEV),
+                       torch.zeros(16 * 256 * 48, 2400, dtype=torch.bfloat16, device=DEV))
+    with pytest.raises(RuntimeError, match="unsupported"):                                   # not the shape it is for
+        ops.gemm_panel(torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV), w, any_shape=False)
+
+
+def test_gemm_skinny_refuses_what_it_cannot_take(ops):
+    a = torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(32, 64, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(ValueError, match="at most 64 rows"):
+        ops.gemm_skinny(a, w)
+    with pytest.raises(ValueError, match="multiple of 8"):
+        ops.gemm_skinny(a[:4, :60], w[:, :60].contiguous())
+
+
+@pytest.mark.parametrize("tile", [1, 2])
+@pytest.mark.parametrize("M,N,K", [(65, 662, 64), (300, 2 * 331, 192), (257, 130, 896), (1000, 2 * 4864, 896), (2051, 1026, 128),
+                                   (130, 16, 64), (513, 4100, 1536)])
+def test_gemm_tiled(ops, M, N, K, tile):
+    """The many-rows product and its gated epilogue with either tile shape: rows and features that fill no
+    whole tile, one step of 64 columns and many."""
+    force = ops._get("ms_gemm_tiled_force")
+    force.restype = None
+    g = torch.Generator().manual_seed(M + N)
+    a = torch.randn(M, K, generator=g).bfloat16().to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).bfloat16().to(DEV)
+    a[M - 1] *= 3.0                                        # the last row is told apart from a repeated one before it
+    want = a.double() @ w.double().T
+    force(tile)
+    try:
+        out = ops.gemm_tiled(a, w)
+        act = ops.gemm_tiled(a, w, ops.EPI_SWIGLU)
+    finally:
+        force(0)
+    assert out.shape == (M, N) and act.shape == (M, N // 2) and out.dtype == act.dtype == torch.bfloat16
+    torch.testing.assert_close(out.double(), want, **tol(torch.bfloat16))
+    torch.testing.assert_close(act.double(), torch.nn.functional.silu(want[:, 0::2]) * want[:, 1::2], **tol(torch.bfloat16))
+    # a row's result does not depend on what else is in the batch
+    assert torch.equal(ops.gemm_tiled(a[M - 70:], w), out[M - 70:])
+
+
+def test_gemm_tiled_refuses_what_it_cannot_take_and_linear_goes_on(ops):
+    from llm_infrence_engine_amd.kernels import linear
+
+    g = torch.Generator().manual_seed(5)
+    a = torch.randn(100, 72, generator=g).bfloat16().to(DEV)
+    w = (torch.randn(60, 72, generator=g) / 8).bfloat16().to(DEV)
+    with pytest.raises(ops.UnsupportedShape):
+        ops.gemm_tiled(a, w)                               # 72 columns: no multiple of 64
+    assert not ops.gemm_tiled_pays(a, w)
+    with pytest.raises(TypeError):
+        ops.gemm_tiled(a.float(), w)
+    # the dispatcher: wide enough rows of a narrow model go to the tiled kernel, others to the library
+    a2 = torch.randn(200, 128, generator=g).bfloat16().to(DEV)
+    w2 = (torch.randn(96, 128, generator=g) / 11).bfloat16().to(DEV)
+    assert ops.gemm_tiled_pays(a2, w2)
+    got = linear.linear_swiglu(a2, w2)
+    ref = a2.double() @ w2.double().T
+    torch.testing.assert_close(got.double(), torch.nn.functional.silu(ref[:, 0::2]) * ref[:, 1::2], **tol(torch.bfloat16))
+    assert torch.equal(got, ops.gemm_tiled(a2, w2, ops.EPI_SWIGLU))
+    assert linear.fallback_count() == 0 or all(k[3] != "tiled gated product" for k in linear.fallbacks)
 
 
 def test_linear_picks_a_kernel_for_every_shape(ops):
