@@ -509,7 +509,14 @@ int plan(const void* A, size_t lda, const bf16* W, size_t ldw, const float* bias
 int splitk_parts(int M, int N, int K) {
   const int cus = ms_compute_units();
   const int tiles = (N + 15) / 16;
-  if (M <= 0 || M > MAX_TOKENS || K < 8192 || K % 8 || tiles > 2 * cus) return 0;
+  if (M <= 0 || M > MAX_TOKENS || K % 8 || tiles > 2 * cus) return 0;
+  // Rows of 8,192 columns or more (down projections) always; with more than 32 tokens also rows from 3,072
+  // columns on against a W of about a tile per CU (the o and q/k/v products of the 7B and 32B shapes), where an
+  // unsplit block reads all activations, four times its weights, for a single tile (64 tokens, 3,584 x 3,584:
+  // 21.5 -> 16.9 us in four parts; 4,608 x 3,584: 23.8 -> 18.3; 5,120 x 5,120: 31.7 -> 24.1; with 32 tokens, or
+  // rows of 2,048 columns, splitting is no faster or slower)
+  const bool long_rows = K >= 8192;
+  if (!long_rows && !(M > 32 && K >= 3072 && tiles * 4 >= cus * 3)) return 0;
   // up to 16 tokens a W with a tile for (nearly) every CU and no more is served as well unsplit (7B shape's down
   // projection, 224 tiles, at 8 tokens: 34 us unsplit, 39 split; 320 tiles of the 14B and 32B shapes: 47 -> 39
   // and 93 -> 64 us split, for the second round of blocks that unsplit they need)
@@ -518,7 +525,7 @@ int splitk_parts(int M, int N, int K) {
   for (int parts = 2; parts <= 16; parts *= 2) {
     const int row_blocks = cus / parts;
     if (row_blocks < 1 || (tiles + row_blocks - 1) / row_blocks > WAVES) continue;
-    if (K / parts < 1024) break;
+    if (K / parts < (long_rows ? 1024 : 768)) break;
     best = parts;
   }
   return best;

@@ -629,7 +629,7 @@ def test_gemm_panel_long_rows(ops, M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(8, 5120, 13824), (64, 3584, 18944), (33, 5120, 27648), (17, 900, 8200), (64, 16, 9000),
-                                   (5, 8192, 16384)])
+                                   (5, 8192, 16384), (64, 3584, 3584), (40, 4608, 3584), (64, 7168, 5120), (33, 3100, 3080)])
 def test_gemm_with_the_columns_split_over_blocks(ops, M, N, K):
     """Long rows against few of them: blocks take parts of the columns, a second kernel adds the partial sums in
     order.  Every epilogue that has no gate; a row's numbers do not depend on the rest of the batch; parts of
@@ -662,6 +662,8 @@ def test_columns_are_split_only_where_it_pays(ops):
     assert parts(8, 37888, 3584) == 0        # and here, with tiles enough for every CU besides
     assert parts(65, 3584, 18944) == 0       # too many tokens
     assert parts(8, 16384, 18944) == 0       # more than two tiles per CU
+    assert parts(64, 3584, 3584) == 4 and parts(64, 5120, 5120) == 4   # shorter rows: only with more than 32 tokens ...
+    assert parts(32, 3584, 3584) == 0 and parts(64, 2048, 2048) == 0 and parts(64, 896, 4864) == 0   # ... long enough, and a tile to most CUs
 
 
 def test_gemm_panel_refuses_what_it_cannot_take(ops):
