@@ -218,7 +218,7 @@ int launch(const bf16* A, size_t lda, const bf16* W, size_t ldw, TO* out, size_t
   return ms_launch_status();
 }
 
-int g_tile = 0;   // measurements: 0 leaves the choice of tile, 1 and 2 force one
+int g_tile = 0;   // measurements: 0 leaves the choice of tile, 1, 2 and 3 force one
 
 // Tiles of 256 x 256 (a byte loaded does 128 multiply-adds; one block to a CU, 1.7 us a step of 64 columns, in
 // whole rounds over the CUs) or of 128 x 128 (two blocks to a CU, 1.26 us a step each; they end at different
@@ -228,6 +228,10 @@ int choose_tile(int M, int N) {
   const long long cus = ms_compute_units();
   const long long big = (long long)((N + 255) / 256) * ((M + 255) / 256);
   const long long small = (long long)((N + 127) / 128) * ((M + 127) / 128);
+  // fewer tiles of 128 x 128 than CUs: tiles of 64 x 64 (four waves) put four times as many CUs to work, and a
+  // tile's time is the time its CU needs to draw its rows (q/k/v of the 0.5B shape, 512 tokens: 11.3 -> 8.7 us;
+  // gate/up at 128 tokens 16.6 -> 12.9, at 256 tokens 16.0 -> 14.9; from 512 tokens on 20.4 against 25.5)
+  if (small < cus) return 3;
   const double t_big = (double)((big + cus - 1) / cus) * 1.70;
   const double t_small = ((double)small / (double)(2 * cus) + 0.3) * 1.26;
   return t_big <= t_small ? 1 : 2;
@@ -266,6 +270,7 @@ extern "C" int ms_gemm_tiled(const void* A, long long lda, const void* W, long l
 #define GO(WF, WT, FT, TT) return epilogue == EPI_SWIGLU ? launch<WF, WT, FT, TT, EPI_SWIGLU, bf16>(a, lda, w, ldw, o, ldo, M, N, K, stream) \
                                                         : launch<WF, WT, FT, TT, EPI_STORE, bf16>(a, lda, w, ldw, o, ldo, M, N, K, stream)
   if (tile == 1) GO(2, 4, 8, 4);   // 256 x 256
+  if (tile == 3) GO(1, 4, 4, 1);   // 64 x 64, four waves
   GO(2, 4, 4, 2);                  // 128 x 128
 #undef GO
 }

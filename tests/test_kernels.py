@@ -686,7 +686,7 @@ def test_gemm_skinny_refuses_what_it_cannot_take(ops):
         ops.gemm_skinny(a[:4, :60], w[:, :60].contiguous())
 
 
-@pytest.mark.parametrize("tile", [1, 2])
+@pytest.mark.parametrize("tile", [1, 2, 3])
 @pytest.mark.parametrize("M,N,K", [(65, 662, 64), (300, 2 * 331, 192), (257, 130, 896), (1000, 2 * 4864, 896), (2051, 1026, 128),
                                    (130, 16, 64), (513, 4100, 1536)])
 def test_gemm_tiled(ops, M, N, K, tile):
