@@ -238,12 +238,23 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
     for (int s = 0; s < D / 32; ++s) qv[t][s] = *reinterpret_cast<const bf16x8*>(qp + s * 32);
   }
 
-  float m[NT], l[NT];
-  f32x4 o[CT][NT];
+  // The sums of the exponentials come from the matrix cores too: one more product per column tile, of P^T with
+  // a V^T of ones, gives every lane its columns' sums over all 32 keys of the block (of the same bfloat16 values
+  // that the weighted sum of the values uses), where adding them up lane by lane took 32 additions and, at the
+  // end, two exchanges between lanes; the matrix pipe has the time.
+  // (The widest tile at head size 64 has no registers left for it and adds its exponentials up on the vector
+  // pipe, a lane's share at a time, with two exchanges between lanes at the end.)
+  constexpr bool SUMS_BY_MATRIX = !(D == 64 && NT == 4);
+  float m[NT], lvec[NT];
+  f32x4 o[CT][NT], lsum[SUMS_BY_MATRIX ? NT : 1];
+  bf16x8 ones;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) ones[i] = (__bf16)1.0f;
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     m[t] = -INFINITY;
-    l[t] = 0.f;
+    lvec[t] = 0.f;
+    if (SUMS_BY_MATRIX) lsum[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int c = 0; c < CT; ++c) o[c][t] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
@@ -252,10 +263,13 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
   // block's values early, together with its keys.  A wide tile fetches values at the top of the pass that
   // uses them (the score products and the softmax run meanwhile, and so does the SIMD's other wave).
   constexpr bool VALUES_EARLY = NT == 1;
-  KeyBlock<D> cur_k, nxt_k;
-  ValueBlock<CT> cur_v, nxt_v;
-  BlockPlace cur_at, nxt_at;
+  KeyBlock<D> buf_k[2];
+  ValueBlock<CT> buf_v[2];
+  BlockPlace buf_at[2];
   if (blk_begin + wave < blk_end) {
+    KeyBlock<D>& cur_k = buf_k[0];
+    ValueBlock<CT>& cur_v = buf_v[0];
+    BlockPlace& cur_at = buf_at[0];
     const int base = (blk_begin + wave) * 32;
     int pages[2];
     if (early) {  // blk_begin is 0 here; halves past the last key fall back to the null page
@@ -274,7 +288,10 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
   // dropped: a decode tile's time is what its CU can draw, 102 KB at about 43 GB/s at 640 keys, not its waits.)
   int ahead_pages[2] = {0, 0};
   if (blk_begin + wave + WAVES < blk_end) pages_of(table, (blk_begin + wave + WAVES) * 32, key_hi, pg, ahead_pages);
-  for (int blk = blk_begin + wave; blk < blk_end; blk += WAVES) {
+  // One block of 32 keys: the step works on the buffers it is handed as current and fills those it is handed
+  // as next; the loop below calls it with the two sets of buffers in turn, so nothing is copied between them.
+  auto step = [&](int blk, KeyBlock<D>& cur_k, ValueBlock<CT>& cur_v, BlockPlace& cur_at, KeyBlock<D>& nxt_k,
+                  ValueBlock<CT>& nxt_v, BlockPlace& nxt_at) __attribute__((always_inline)) {
     const int base = blk * 32;
     if (!VALUES_EARLY) load_values<CT>(cur_v, vt_pages, cur_at, pg, dim0, lane);
     if (blk + WAVES < blk_end) {
@@ -361,24 +378,25 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
     }
     if (NT == 1 || __builtin_amdgcn_ballot_w64(moved) != 0) {   // the same branch for the whole wave
 #pragma unroll
-      for (int t = 0; t < NT; ++t)
+      for (int t = 0; t < NT; ++t) {
+        if (SUMS_BY_MATRIX) lsum[t] *= corr[t]; else lvec[t] *= corr[t];
 #pragma unroll
         for (int c = 0; c < CT; ++c) o[c][t] *= corr[t];
+      }
     }
     // column by column, so that the products of one column run on the matrix cores while the next column's
     // exponentials are taken
 #pragma unroll
     for (int t = 0; t < NT; ++t) {
-      float ls = 0.f;
 #pragma unroll
       for (int u = 0; u < 2; ++u)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const float e = fast_exp2(fmaf(s[u][t][i], scale_log2e, -m_safe[t]));
-          ls += e;
+          if (!SUMS_BY_MATRIX) lvec[t] += e;
           p[t][u * 4 + i] = (__bf16)e;
         }
-      l[t] = l[t] * corr[t] + ls;
+      if (SUMS_BY_MATRIX) lsum[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones, p[t], lsum[t], 0, 0, 0);
 #pragma unroll
       for (int c = 0; c < CT; ++c) {
         bf16x8 vv;
@@ -387,17 +405,21 @@ attention_mfma_kernel(const bf16* __restrict__ q, size_t q_stride, const bf16* _
         o[c][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vv, p[t], o[c][t], 0, 0, 0);
       }
     }
-    if (blk + WAVES < blk_end) {
-      cur_k = nxt_k;
-      cur_at = nxt_at;
-      if (VALUES_EARLY) cur_v = nxt_v;
-    }
+  };
+  for (int blk = blk_begin + wave; blk < blk_end; blk += 2 * WAVES) {
+    step(blk, buf_k[0], buf_v[0], buf_at[0], buf_k[1], buf_v[1], buf_at[1]);
+    if (blk + WAVES < blk_end) step(blk + WAVES, buf_k[1], buf_v[1], buf_at[1], buf_k[0], buf_v[0], buf_at[0]);
   }
 
+  float l[NT];
 #pragma unroll
-  for (int t = 0; t < NT; ++t) {  // a column's sum is spread over the four lane groups
-    l[t] += __shfl_xor(l[t], 16, MS_WAVE);
-    l[t] += __shfl_xor(l[t], 32, MS_WAVE);
+  for (int t = 0; t < NT; ++t) {
+    if (SUMS_BY_MATRIX) {
+      l[t] = lsum[t][0];   // every row of the product of ones is the column's sum
+    } else {               // a column's sum is spread over the four lane groups
+      l[t] = lvec[t] + __shfl_xor(lvec[t], 16, MS_WAVE);
+      l[t] += __shfl_xor(l[t], 32, MS_WAVE);
+    }
   }
   if (WAVES > 1) {
     // merge the waves' partial results (each relative to its own maximum) in wave order
