@@ -309,11 +309,39 @@ class Block(Part):
     def mixers(self) -> List[Mixer]:
         return [p for p in self.built.values() if isinstance(p, Mixer)]
 
+    def _caching_mixers(self) -> Dict[str, CacheNeed]:
+        out = {}
+        for name, p in self.built.items():
+            if isinstance(p, Mixer):
+                need = p.cache_need()
+                if need is not None:
+                    out[name] = need
+        return out
+
     def cache_need(self) -> Optional[CacheNeed]:
-        needs = [n for n in (m.cache_need() for m in self.mixers()) if n is not None]
-        if len(needs) > 1:
-            raise ValueError("a run of a layer has one cache; a block with two caching mixers must merge their needs itself")
-        return needs[0] if needs else None
+        """What a run of this layer keeps per token.  One caching mixer: its need as it states it.  Several: one
+        need that holds all their page tensors, each under ``<part name>.<tensor name>`` (a run has one cache
+        group, so the mixers must keep their tokens for the same span); ``kv_of`` hands every mixer its own."""
+        needs = self._caching_mixers()
+        if len(needs) <= 1:
+            return next(iter(needs.values()), None)
+        windows = {n.window for n in needs.values()}
+        if len(windows) > 1:
+            raise ValueError(f"the caching mixers {sorted(needs)} of one layer keep their tokens for different spans "
+                             f"({sorted(windows, key=str)}); the pages of a run are given back together")
+        tensors = tuple(PageTensor(f"{name}.{t.name}", t.heads, t.width, t.transpose_at, t.transpose_in)
+                        for name, need in needs.items() for t in need.tensors)
+        return CacheNeed(tensors, windows.pop())
+
+    def kv_of(self, name: str, kv: Optional[KVView]) -> Optional[KVView]:
+        """The part of the run's cache view that belongs to the mixer ``name``, under the tensor names the mixer
+        declared (the whole view when the layer has one caching mixer)."""
+        if kv is None or len(self._caching_mixers()) <= 1:
+            return kv
+        prefix = name + "."
+        return KVView({k[len(prefix):]: v for k, v in kv.pages.items() if k.startswith(prefix)},
+                      {k[len(prefix):]: v for k, v in kv.transposed.items() if k.startswith(prefix)},
+                      kv.block_table, kv.slot_mapping, kv.store, kv.window, kv.table_rows)
 
     def state_need(self):
         needs = []

@@ -479,6 +479,100 @@ def test_toy_architecture_is_registered_built_and_stepped(fw, tmp_path):
     assert all(g.allocator.num_in_use() == 0 for g in runner.manager.groups)
 
 
+def test_a_layer_with_two_caching_mixers(fw, tmp_path):
+    """An arrangement of its own with two attention mixers of different head counts and sizes side by side: the
+    layer's cache need holds both their page tensors under the parts' names, each mixer is handed its own, the
+    model decodes from graphs in bfloat16 and follows the plain computation in both types."""
+    from dataclasses import dataclass
+
+    parts, cfgm, ops = fw.parts, fw.config, fw.ops
+
+    class Twin(parts.Block):
+        """x += wide(norm(x)) + narrow(norm(x))"""
+
+        takes = {"norm": "norm", "wide": "mixer", "narrow": "mixer"}
+
+        def forward(self, x, pending, ctx, kv, state):
+            if pending is not None:
+                ops.residual_add(x, pending)
+            h = self.norm.forward(x)
+            a = self.wide.forward(h, ctx, self.kv_of("wide", kv), None)
+            b = self.narrow.forward(h, ctx, self.kv_of("narrow", kv), None)
+            ops.residual_add(x, a)
+            return b                                   # the next norm (or the head's) adds it
+
+    @dataclass(frozen=True)
+    class TwinConfig:
+        vocab_size: int = 90
+        width: int = 64
+
+        @classmethod
+        def from_dict(cls, d):
+            return cls(d["vocab_size"], d["width"])
+
+        def to_dict(self):
+            return {"vocab_size": self.vocab_size, "width": self.width, "architectures": ["TwinForCausalLM"]}
+
+        def to_spec(self):
+            H = self.width
+            PartSpec = cfgm.PartSpec
+
+            def attn(p, nh, nkv, d):
+                return PartSpec("gqa_attention", p, {"hidden_size": H, "num_heads": nh, "num_kv_heads": nkv, "head_dim": d,
+                                                      "scale": d ** -0.5, "qkv_bias": True, "out_bias": False, "window": None})
+            layers = tuple(cfgm.layer("twin", norm=PartSpec("rms_norm", f"l{i}.n.", {"size": H, "eps": 1e-6}),
+                                      wide=attn(f"l{i}.wide.", 4, 2, 32), narrow=attn(f"l{i}.narrow.", 2, 1, 64))
+                           for i in range(2))
+            return cfgm.ModelSpec("TwinForCausalLM", H, self.vocab_size,
+                                  PartSpec("token_embedding", "emb.", {"vocab_size": self.vocab_size, "hidden_size": H}),
+                                  layers, (cfgm.Run(0), cfgm.Run(1)), PartSpec("rms_norm", "final.", {"size": H, "eps": 1e-6}),
+                                  PartSpec("lm_head", "head.", {"hidden_size": H, "vocab_size": self.vocab_size, "tied_to": None}))
+
+    parts.register_part("block", "twin", Twin)
+    cfgm.register_architecture("TwinForCausalLM", TwinConfig)
+    cfg = TwinConfig()
+    d = fw.root.write_random_model(tmp_path / "twin", cfg, seed=8, dtype="float32", std=0.2)
+    w = P.read_weights(d, torch.float64)
+
+    def plain(ids):
+        T = len(ids)
+        x = w["emb.weight"][ids]
+        for i in range(2):
+            h = P.rms_norm(x, w[f"l{i}.n.weight"], 1e-6)
+            for name, nh, nkv, hd in (("wide", 4, 2, 32), ("narrow", 2, 1, 64)):
+                p = f"l{i}.{name}."
+                q = (h @ w[p + "q_proj.weight"].T + w[p + "q_proj.bias"]).view(T, nh, hd).transpose(0, 1)
+                k = (h @ w[p + "k_proj.weight"].T + w[p + "k_proj.bias"]).view(T, nkv, hd).transpose(0, 1)
+                v = (h @ w[p + "v_proj.weight"].T + w[p + "v_proj.bias"]).view(T, nkv, hd).transpose(0, 1)
+                o = P.causal_attention(q, k, v).transpose(0, 1).reshape(T, nh * hd)     # no position encoding
+                x = x + o @ w[p + "o_proj.weight"].T
+        return P.rms_norm(x, w["final.weight"], 1e-6) @ w["head.weight"].T
+
+    rng = np.random.default_rng(2)
+    seq = [int(t) for t in rng.integers(0, 90, 45)]
+    want = plain(torch.tensor(seq)).numpy()
+    Entry = fw.engine.StepEntry
+    for dtype, bound in (("float32", 1e-3), ("bfloat16", 0.15)):
+        runner = fw.engine.load_runner(d, dtype=dtype, page_size=16, num_pages=8, max_requests=2, max_len=64,
+                                       hip_graphs=dtype == "bfloat16")
+        need = runner.model.layers[0].cache_need()
+        assert [t.name for t in need.tensors] == ["wide.k", "wide.v", "narrow.k", "narrow.v"]
+        assert [(t.heads, t.width) for t in need.tensors] == [(2, 32), (2, 32), (1, 64), (1, 64)]
+        assert len(runner.layout.group_keys) == 1 and runner.manager.bytes_per_token(1) == 2 * (2 * 2 * 32 + 2 * 64)
+        got = [runner.step([Entry("x", seq[:30], list(range(30)))]).float().cpu().numpy()]
+        for t in range(30, 45):
+            got.append(runner.step([Entry("x", [seq[t]], [0])]).float().cpu().numpy())
+        assert np.abs(np.concatenate(got) - want).max() < bound, dtype
+        if dtype == "bfloat16":
+            assert runner.graphs is not None and runner.graphs.launches == 16
+    # mixers that keep their tokens for different spans cannot share a layer
+    bad = Twin.build({"norm": cfg.to_spec().layers[0].parts["norm"], "wide": cfg.to_spec().layers[0].parts["wide"],
+                      "narrow": cfgm.PartSpec("gqa_attention", "n.", {"hidden_size": 64, "num_heads": 2, "num_kv_heads": 1,
+                                                                    "head_dim": 64, "scale": 0.125, "window": 7})})
+    with pytest.raises(ValueError, match="different spans"):
+        bad.cache_need()
+
+
 def test_a_mixer_with_state_that_says_so_decodes_from_graphs(fw, tmp_path):
     """The decaying-state mixer handles single tokens with device tensors only and declares ``graph_safe``: a model of
     it, attention and dense feed-forwards decodes from captured graphs, several steps to a launch too, rows that

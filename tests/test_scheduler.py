@@ -291,3 +291,38 @@ def test_batch_size_buckets_of_the_decode_graphs():
     assert default_batch_sizes(64) == [1, 2, 4, 8, 16, 32, 64]
     with pytest.raises(ValueError):
         default_batch_sizes(0)
+
+
+def test_memory_beside_the_pages_is_taken_off_the_budget():
+    """The pool sized from a share of the device's memory leaves room for what the engine holds beside weights and
+    pages: state slots (one more than requests), block tables, the logits of the graph buckets and activations."""
+    import torch
+
+    from llm_infrence_engine_amd.config import config_from_dict, preset
+    from llm_infrence_engine_amd.engine.engine import memory_beside_the_pages
+    from llm_infrence_engine_amd.parts.base import Runtime, StateNeed
+    from llm_infrence_engine_amd.parts.model import Model
+
+    model = Model(config_from_dict(preset("tinyB")).to_spec())
+    model.rt = Runtime(torch.device("cpu"), torch.bfloat16)
+    plain = CacheLayout(model.run_needs())
+    stateful = CacheLayout([(kv, (StateNeed((1000,), torch.float32), StateNeed((), torch.int32)) if i == 0 else None, c)
+                            for i, (kv, _, c) in enumerate(model.run_needs())])
+    cfg = EngineConfig(dtype="bfloat16", max_seqs=7, max_len=64, block_size=16, max_num_batched_tokens=128,
+                       gpu_memory_fraction=0.5, hip_graphs=False)
+    a, b = memory_beside_the_pages(cfg, model, plain), memory_beside_the_pages(cfg, model, stateful)
+    assert b - a == 8 * (1000 * 4 + 4)                      # eight slots of 1,000 floats and an int
+    tables = 1 * 8 * 4 * 4                                  # one group, eight rows of four pages
+    widest = max(320 * 2, 192 * 4)                          # the widest checkpoint matrix's rows in bfloat16, or the float stream
+    assert a == tables + 10 * 128 * widest
+    with_graphs = EngineConfig(dtype="bfloat16", max_seqs=7, max_len=64, block_size=16, max_num_batched_tokens=128,
+                               gpu_memory_fraction=0.5, hip_graphs=True)
+    assert memory_beside_the_pages(with_graphs, model, plain) == tables + (1 + 2 + 4 + 7) * 384 * 4 + 10 * (128 + 7) * widest
+    # and it comes off the pool
+    per_token = plain.bytes_per_token(2)
+    total = 1 << 24
+    free_pool = cfg.resolved_num_blocks(per_token, total, 0)
+    assert cfg.resolved_num_blocks(per_token, total, 0, other_bytes=b) <= free_pool
+    tight = EngineConfig(dtype="bfloat16", max_seqs=64, max_len=4096, block_size=16, gpu_memory_fraction=0.5)
+    most = tight.resolved_num_blocks(per_token, total, 0)
+    assert tight.resolved_num_blocks(per_token, total, 0, other_bytes=1 << 20) == most - (1 << 20) // (per_token * 16)
