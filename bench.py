@@ -62,7 +62,7 @@ def prefill_flops(cfg, tokens):
     return linear + attention
 
 
-def run_decode(eng_mod, model, batch, steps, warmup, vocab, seed, prompt_len=PROMPT_LEN):
+def run_decode(eng_mod, model, batch, steps, warmup, vocab, seed, prompt_len=PROMPT_LEN, sampling=None):
     """Prefill ``batch`` prompts, then time ``steps`` decode steps of the engine.  Returns seconds per step, the
     mean context length of the timed steps, and what a graph launch cost the host against the whole launch."""
     import numpy as np
@@ -79,9 +79,9 @@ def run_decode(eng_mod, model, batch, steps, warmup, vocab, seed, prompt_len=PRO
     # every graph this run can reach, before any timer: all requests stay alive, so the one bucket of ``batch``
     # rows, in both context classes and every launch size (an engine that serves captures all buckets itself)
     e.runner.graphs.warm_up(e.launch_sizes(), batch_sizes=[batch], portion_tokens=())
-    for _ in range(batch):
+    for i in range(batch):
         e.add_request(eng_mod.Request([int(t) for t in rng.integers(0, vocab, prompt_len)],
-                                      max_new_tokens=warmup + steps + extra))
+                                      max_new_tokens=warmup + steps + extra, **dict(sampling or {}, **({"seed": i} if sampling else {}))))
     while any(r.num_tokens - r.num_computed > 1 for r in e.running) or e.waiting:
         e.step()                                   # prompts in portions under the budget; first tokens sampled
     def run(n):   # exactly n decode steps, several to a graph launch
@@ -93,7 +93,7 @@ def run_decode(eng_mod, model, batch, steps, warmup, vocab, seed, prompt_len=PRO
     run(warmup)
     assert len(e.running) == batch and all(r.num_tokens - r.num_computed == 1 for r in e.running)
     graphs = e.runner.graphs
-    held = len(graphs.buckets)
+    held = len(graphs.buckets)      # (graphs that draw tokens are captured at their first use: the warm-up steps)
     torch.cuda.synchronize()
     q0, n0 = graphs.enqueue_seconds, graphs.launches
     t0 = time.perf_counter()
@@ -318,6 +318,10 @@ def main() -> int:
         out["points"] = {}
         for b in (1, 64):
             out["points"].update(decode_point(eng, model, cfg, b, min(a.steps, 128), min(a.warmup, 8), vocab, a.prompt_len))
+        # the same batch as the headline with every request drawing its tokens (temperature 0.8, top-k 50, top-p 0.9)
+        dts, _, _ = run_decode(eng, model, a.batch, min(a.steps, 128), 16, vocab, seed=9, prompt_len=a.prompt_len,
+                               sampling=dict(temperature=0.8, top_k=50, top_p=0.9))
+        out["points"][f"decode_b{a.batch}_sampled"] = round(a.batch / dts, 1)
         out["sampler"] = run_sampler(vocab)
     if a.shape == "0.5b" and not a.no_points and not a.no_shapes and a.layers == shape["num_hidden_layers"]:
         del model

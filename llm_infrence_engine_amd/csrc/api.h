@@ -15,12 +15,12 @@ int ms_rms_norm(float* x, const void* delta, int delta_dtype, int n_partials, lo
 int ms_bias_add(void* x, const float* bias, int n_rows, int width, int dtype, hipStream_t stream);
 
 // tables / slots: host arrays of n_groups device pointers (block table int32 [table rows, table_stride], slot
-// mapping int32 [n_rows]); table_rows int32 [n_rows]: the table's row of each row of the batch.  At most
-// ms_max_cache_groups() groups.
+// mapping int32 [n_rows]); table_rows int32 [n_rows]: the table's row of each row of the batch; draw_index int32
+// [n_rows] (may be null): counted up by one for every live row.  At most ms_max_cache_groups() groups.
 int ms_max_cache_groups();
 int ms_decode_advance(const int* prev_tokens, int* token_ids, int* positions, int* context_lens, const int* n_live,
-                      const int* table_rows, const int* const* tables, int* const* slots, int n_groups,
-                      int table_stride, int page_size, int n_rows, hipStream_t stream);
+                      const int* table_rows, int* draw_index, const int* const* tables, int* const* slots,
+                      int n_groups, int table_stride, int page_size, int n_rows, hipStream_t stream);
 
 // Block tables kept on the device: tables[g][index[g][i]] = value[g][i] for i < counts[g] (counts: device ints),
 // every index at most once per group; max_updates bounds counts, table_elems bounds the indices.

@@ -402,8 +402,8 @@ extern "C" int ms_rope_store(void* qkv, const float* bias, const int* positions,
 
 // ------------------------------------------------------------------------------------------------
 // Between two decode steps that run back to back on the device: every live request (row < *n_live) moves one
-// position on, takes the token the step before chose as its input, and gets the slots its new key and value
-// go to, from its block tables.  One thread per row; up to MS_MAX_GROUPS cache groups.
+// position on, takes the token the step before chose as its input, counts its draws on (draw_index, may be
+// null) and gets the slots its new key and value go to, from its block tables.  One thread per row; up to MS_MAX_GROUPS cache groups.
 struct AdvanceArgs {
   const int* prev_tokens;
   int* token_ids;
@@ -411,6 +411,7 @@ struct AdvanceArgs {
   int* context_lens;
   const int* n_live;
   const int* table_rows;
+  int* draw_index;
   const int* tables[MS_MAX_GROUPS];
   int* slots[MS_MAX_GROUPS];
   int n_groups, table_stride, page_size, n_rows;
@@ -423,6 +424,7 @@ __global__ void decode_advance_kernel(AdvanceArgs a) {
   a.positions[r] = pos;
   a.context_lens[r] = pos + 1;
   a.token_ids[r] = a.prev_tokens[r];
+  if (a.draw_index) a.draw_index[r] += 1;     // the next draw of a request that samples is its next
   const size_t row = a.table_rows ? a.table_rows[r] : r;
   for (int g = 0; g < a.n_groups; ++g)
     a.slots[g][r] = a.tables[g][row * a.table_stride + pos / a.page_size] * a.page_size + pos % a.page_size;
@@ -431,14 +433,14 @@ __global__ void decode_advance_kernel(AdvanceArgs a) {
 extern "C" int ms_max_cache_groups() { return MS_MAX_GROUPS; }
 
 extern "C" int ms_decode_advance(const int* prev_tokens, int* token_ids, int* positions, int* context_lens,
-                                 const int* n_live, const int* table_rows, const int* const* tables,
-                                 int* const* slots, int n_groups, int table_stride, int page_size, int n_rows,
-                                 hipStream_t stream) {
+                                 const int* n_live, const int* table_rows, int* draw_index,
+                                 const int* const* tables, int* const* slots, int n_groups, int table_stride,
+                                 int page_size, int n_rows, hipStream_t stream) {
   if (n_rows <= 0) return MS_OK;
   if (n_groups < 0 || n_groups > MS_MAX_GROUPS || table_stride <= 0 || page_size <= 0) return MS_BAD_ARG;
   AdvanceArgs a;
   a.prev_tokens = prev_tokens; a.token_ids = token_ids; a.positions = positions; a.context_lens = context_lens;
-  a.n_live = n_live; a.table_rows = table_rows; a.n_groups = n_groups; a.table_stride = table_stride;
+  a.n_live = n_live; a.table_rows = table_rows; a.draw_index = draw_index; a.n_groups = n_groups; a.table_stride = table_stride;
   a.page_size = page_size; a.n_rows = n_rows;
   for (int g = 0; g < MS_MAX_GROUPS; ++g) { a.tables[g] = g < n_groups ? tables[g] : nullptr; a.slots[g] = g < n_groups ? slots[g] : nullptr; }
   decode_advance_kernel<<<dim3((n_rows + 63) / 64), dim3(64), 0, stream>>>(a);

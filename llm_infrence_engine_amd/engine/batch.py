@@ -53,7 +53,13 @@ class StepLayout:
                    ("update_counts", n_groups)]
         for g in range(n_groups):
             fields += [(f"update_index{g}", n_updates), (f"update_value{g}", n_updates)]
+        # how each request's next token is chosen, for steps that choose it on the device: float fields hold the
+        # bits of a float32, "seeds" two ints to a request (one int64, at an even offset)
+        fields += [("seeds", 2 * n_requests), ("temperature", n_requests), ("top_p", n_requests), ("top_k", n_requests),
+                   ("draw_index", n_requests)]
         for name, n in fields:
+            if name == "seeds":
+                o += o & 1
             self.at[name] = slice(o, o + n)
             o += n
         self.size = o
@@ -83,7 +89,10 @@ class StepBuffers:
         self._sent.record()
 
     def views(self, layout: StepLayout) -> Dict[str, torch.Tensor]:
-        return {name: self.dev[sl] for name, sl in layout.at.items()}
+        v = {name: self.dev[sl] for name, sl in layout.at.items()}
+        v["temperature"], v["top_p"] = v["temperature"].view(torch.float32), v["top_p"].view(torch.float32)
+        v["seeds"] = v["seeds"].view(torch.int64)
+        return v
 
 
 @dataclass
@@ -103,6 +112,18 @@ class _Described:
     logit_rows: np.ndarray
     q_lens: List[int]
     starts: np.ndarray
+    sampling: Optional[Sequence] = None    # per request (temperature, top_k, top_p, seed, draw index), or None: greedy
+
+
+@dataclass
+class Sampling:
+    """How one request's next token is chosen on the device (``sampling/sampler.py`` has the rules)."""
+
+    temperature: float = 0.0
+    top_k: int = 0
+    top_p: float = 1.0
+    seed: int = 0
+    draw_index: int = 0
 
 
 @dataclass
@@ -194,6 +215,14 @@ class BatchBuilder:
         put("logit_rows", d.logit_rows if d else empty, 0)
         a[at["n_live"]] = R
         a[at["n_fresh"]] = d.fresh_rows.size if d else 0
+        how = list(d.sampling) if d is not None and d.sampling is not None else []
+        if how and len(how) != R:
+            raise ValueError("one Sampling per request of the step, or none")
+        put("temperature", np.asarray([h.temperature for h in how], dtype=np.float32).view(np.int32), 0)
+        put("top_p", np.asarray([h.top_p for h in how], dtype=np.float32).view(np.int32), 0)
+        put("top_k", np.asarray([h.top_k for h in how], dtype=np.int32), 0)
+        put("draw_index", np.asarray([h.draw_index for h in how], dtype=np.int32), 0)
+        put("seeds", np.asarray([h.seed & 0x7FFFFFFFFFFFFFFF for h in how], dtype=np.int64).view(np.int32), 0)
         most = 0
         if m.pending_updates() > layout.n_updates:
             raise RuntimeError("more table entries changed than the layout has room for; flush them first")

@@ -18,7 +18,7 @@ from ..cache.allocator import OutOfPages
 from ..config.engine_config import EngineConfig
 from ..parts.model import Model
 from ..sampling import Sampler
-from .batch import StepEntry
+from .batch import Sampling, StepEntry
 from .request import Request, StepRecord
 from .runner import ModelRunner
 from .scheduler import Scheduler
@@ -65,10 +65,10 @@ class Engine:
         With ``hip_graphs`` every graph that serving can reach is captured here, before the first request
         (as the reference's constructor does, src/miniserve/graph_decode.py:46-47), unless ``capture_at_start``
         is False: then a graph is captured when a step first needs it.
-        ``decode_steps_per_launch`` > 1 (with ``hip_graphs``): while every running request is decoding
-        greedily and nobody waits, up to that many decode steps run in one graph launch, each fed the argmax of
-        the one before on the device; a stop id is then noticed up to that many steps late (the surplus tokens
-        are dropped), so outputs do not change.
+        ``decode_steps_per_launch`` > 1 (with ``hip_graphs``): while every running request is decoding and
+        nobody waits, up to that many decode steps run in one graph launch, each fed the token the one before
+        chose on the device (the argmax, or the request's own draw); a stop id is then noticed up to that many
+        steps late (the surplus tokens are dropped), so outputs do not change.
         ``graph_portion_tokens`` (with ``hip_graphs``): steps with prompt portions of up to that many tokens are
         replayed from graphs too (None: as far as the host would otherwise be what such a step waits for)."""
         dtype = {torch.float32: "float32", torch.bfloat16: "bfloat16"}[model.rt.dtype]
@@ -146,14 +146,18 @@ class Engine:
 
     def _steps_ahead(self, sched, limit: int) -> int:
         """How many decode steps the next launch may hold: a power of two within the configured limit and
-        within what every request still has to generate, if all of them decode greedily and nobody waits."""
+        within what every request still has to generate, if all of them decode and nobody waits; 0 if the step
+        is not one of single decoded tokens that a graph launch can take."""
+        if self.runner.graphs is None or len(sched) > self.runner.graphs.max_batch:
+            return 0
+        for s in sched:
+            if s.count != 1 or s.start == 0 or not s.sample:
+                return 0
         limit = min(limit, self.decode_steps_per_launch)
-        if limit < 2 or self.scheduler.waiting or len(sched) > self.runner.graphs.max_batch:
+        if limit < 2 or self.scheduler.waiting:
             return 1
         for s in sched:
             r = s.request
-            if s.count != 1 or s.start == 0 or not s.sample or r.temperature > 0.0:
-                return 1
             limit = min(limit, r.max_new_tokens - len(r.output_ids), self.config.max_len - r.num_computed)
         k = 1
         while k * 2 <= limit:
@@ -173,11 +177,16 @@ class Engine:
         useful = 0
         if not sched and self.scheduler.has_work():
             raise RuntimeError("the scheduler could place no request although work is waiting")
-        ahead = self._steps_ahead(sched, max_decode_steps) if sched and self.decode_steps_per_launch > 1 else 1
-        if ahead > 1:
+        ahead = self._steps_ahead(sched, max_decode_steps) if sched else 0
+        sampled = any(s.request.temperature > 0.0 for s in sched)
+        if ahead > 1 or (ahead == 1 and sampled):
             # a request's newest token: its last output, or its prompt's last token when a portion left only that
             entries = [StepEntry(s.request.id, [(s.request.output_ids or s.request.prompt_ids)[-1]]) for s in sched]
-            tokens = self.runner.decode_steps(entries, ahead)
+            how = None
+            if sampled:       # the draws happen on the device too, by each request's own rule, seed and count
+                how = [Sampling(r.temperature, r.top_k, r.top_p, r.sample_seed, len(r.output_ids))
+                       for r in (s.request for s in sched)]
+            tokens = self.runner.decode_steps(entries, ahead, how)
             for k in range(ahead):      # as the single steps would have: a finished request drops its later tokens
                 for i, s in enumerate(sched):
                     if s.request.state == "running":
@@ -194,13 +203,13 @@ class Engine:
             logits = self.runner.step(entries)
             greedy = self.runner.greedy_tokens
             if greedy is not None and len(rows) == len(entries) and all(r.temperature <= 0.0 for r in rows):
-                sampled = greedy.tolist()       # the captured graph has already taken the argmax
+                chosen = greedy.tolist()       # the captured graph has already taken the argmax
             else:
-                sampled = self.sampler.sample(logits, rows)
-            useful = self.scheduler.commit(sched, sampled)
+                chosen = self.sampler.sample(logits, rows)
+            useful = self.scheduler.commit(sched, chosen)
         n_decode = sum(1 for s in sched if s.count == 1 and s.start > 0)
         n_prefill = sum(s.count for s in sched) - n_decode
-        decode_steps = ahead if n_decode else 0
+        decode_steps = max(ahead, 1) if n_decode else 0
         self.prefill_tokens_computed += n_prefill
         self.peak_running = max(self.peak_running, len(self.scheduler.running))
         in_use = max((g.allocator.num_in_use() for g in self.runner.manager.groups), default=0)

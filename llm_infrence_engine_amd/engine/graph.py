@@ -71,6 +71,7 @@ class _Bucket:
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.logits: Optional[torch.Tensor] = None       # decode: [rows, V] of the last step
         self.hidden = None                                # portions: (residual stream, unsummed addend)
+        self.sampled = False                              # decode: False, or (top-k, top-p): tokens are drawn, not the argmax
         self.tokens = torch.zeros((steps, layout.n_requests), dtype=torch.int32, device=device)   # the argmax of every step
 
 
@@ -129,14 +130,18 @@ class StepGraphs:
         return len(self.buckets) + len(self.portion_buckets)
 
     # ------------------------------------------------------------------ buckets
-    def _bucket(self, n: int, long_context: bool, steps: int = 1) -> _Bucket:
+    def _bucket(self, n: int, long_context: bool, steps: int = 1, sampled=False) -> _Bucket:
+        """``sampled``: False (the graph takes the argmax), or which thresholds the sampling kernels look for,
+        (top-k, top-p): a graph of its own for each, so that rows which only have a temperature do not pay for
+        the search."""
         B = next(b for b in self.sizes if b >= n)
-        key = (B, long_context, steps)
+        key = (B, long_context, steps) + (("sampled",) + tuple(sampled) if sampled else ())
         bk = self.buckets.get(key)
         if bk is None:
             ps = self.manager.page_size
             layout = StepLayout(B, B, B, len(self.manager.groups), B * (steps // ps + 2))
             bk = self.buckets[key] = _Bucket(layout, self.runner.rt.device, steps)
+            bk.sampled = sampled
             cap = self.width * ps
             self._capture(bk, max_q_len=1, max_context_len=cap if long_context else min(cap, ops.LONG_CONTEXT))
         return bk
@@ -181,9 +186,14 @@ class StepGraphs:
             for k in range(bk.steps):
                 if k > 0:      # n_live is 0 in the buffer while capturing and warming up: nothing moves
                     ops.decode_advance(bk.tokens[k - 1], f["token_ids"], f["positions"], f["context_lens"], f["n_live"],
-                                       f["state_slots"], runner.pools.tables, bk.slots, self.manager.page_size)
+                                       f["state_slots"], runner.pools.tables, bk.slots, self.manager.page_size,
+                                       f["draw_index"] if bk.sampled else None)
                 bk.logits = model.head_logits(*model.forward_hidden(ctx, caches), ctx.logit_rows)
-                ops.sample(bk.logits, bk.tokens[k])
+                if bk.sampled:     # rows without a temperature (padding rows too) take the first maximum
+                    ops.sample(bk.logits, bk.tokens[k], f["temperature"], f["top_k"], f["top_p"], f["seeds"], f["draw_index"],
+                               use_top_k=bk.sampled[0], use_top_p=bk.sampled[1])
+                else:
+                    ops.sample(bk.logits, bk.tokens[k])
 
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
@@ -221,10 +231,12 @@ class StepGraphs:
             return "portions"
         return None
 
-    def _fill_and_replay(self, bk: _Bucket, entries: List[StepEntry], steps: int, every_row: bool = False):
+    def _fill_and_replay(self, bk: _Bucket, entries: List[StepEntry], steps: int, every_row: bool = False,
+                         sampling=None):
         if self.manager.pending_updates() > bk.layout.n_updates:
             self.builder.flush_updates()
         d = self.builder.describe(entries, steps)
+        d.sampling = sampling
         if every_row:     # a decode graph works out the logits and the greedy choice of every request, wanted or not
             d.logit_rows = np.arange(d.n_requests, dtype=np.int32)
         bk.buf.wait_until_sent()
@@ -233,15 +245,20 @@ class StepGraphs:
         bk.graph.replay()
         return d
 
-    def run(self, entries: List[StepEntry], steps: int = 1):
+    def run(self, entries: List[StepEntry], steps: int = 1, sampling=None):
         """``steps`` decode steps for ``entries`` (one token each, pages already grown for all the steps).
-        Returns (logits [R, V] of the last step, greedy tokens int32 [steps, R]); both are views of static
-        buffers that the next replay overwrites."""
+        ``sampling``: one ``batch.Sampling`` per entry if any of them draws its tokens (the graph then holds the
+        sampling kernels instead of the argmax), else None.  Returns (logits [R, V] of the last step, chosen
+        tokens int32 [steps, R]); both are views of static buffers that the next replay overwrites."""
         t_begin = time.perf_counter()
         R = len(entries)
         longest = max(self.manager.computed(e.req_id) for e in entries) + steps
-        bk = self._bucket(R, longest > ops.LONG_CONTEXT, steps)
-        self._fill_and_replay(bk, entries, steps, every_row=True)
+        sampled = False
+        if sampling is not None:
+            V = self.runner.model.spec.vocab_size
+            sampled = (any(0 < h.top_k < V for h in sampling), any(h.top_p < 1.0 for h in sampling))
+        bk = self._bucket(R, longest > ops.LONG_CONTEXT, steps, sampled=sampled)
+        self._fill_and_replay(bk, entries, steps, every_row=True, sampling=sampling)
         self.enqueue_seconds += time.perf_counter() - t_begin
         self.launches += 1
         return bk.logits[:R], bk.tokens[:, :R]

@@ -95,10 +95,11 @@ class ModelRunner:
         return logits
 
     @torch.inference_mode()
-    def decode_steps(self, entries: List[StepEntry], steps: int) -> List[List[int]]:
-        """``steps`` greedy decode steps in one launch of a captured graph: every request of ``entries`` (one
-        token each, the one it is to be fed next) runs ``steps`` tokens ahead, each step fed the argmax of the
-        one before on the device.  Returns the chosen tokens, [steps][len(entries)]."""
+    def decode_steps(self, entries: List[StepEntry], steps: int, sampling=None) -> List[List[int]]:
+        """``steps`` decode steps in one launch of a captured graph: every request of ``entries`` (one token
+        each, the one it is to be fed next) runs ``steps`` tokens ahead, each step fed the token the one before
+        chose on the device: the argmax, or with ``sampling`` (one ``batch.Sampling`` per entry) a draw by each
+        request's own rule, seed and count of draws.  Returns the chosen tokens, [steps][len(entries)]."""
         if self.graphs is None:
             raise RuntimeError("several decode steps per launch need hip_graphs")
         m = self.manager
@@ -106,7 +107,7 @@ class ModelRunner:
             if len(e.tokens) != 1:
                 raise ValueError("decode_steps takes one token per request")
             m.grow(e.req_id, m.computed(e.req_id) + steps)
-        _, tokens = self.graphs.run(entries, steps)
+        _, tokens = self.graphs.run(entries, steps, sampling)
         out = tokens.tolist()
         for e in entries:
             m.advance(e.req_id, m.computed(e.req_id) + steps)

@@ -27,8 +27,8 @@ _SIGNATURES = {
                             _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "ms_qkv_rope_store": [_c_ptr, _c_ll, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                           _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
-    "ms_decode_advance": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int,
-                          _c_ptr],
+    "ms_decode_advance": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int,
+                          _c_int, _c_ptr],
     "ms_max_cache_groups": [],
     "ms_table_update": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ll, _c_ptr],
     "ms_zero_rows": [_c_ptr, _c_ll, _c_ptr, _c_ptr, _c_int, _c_ptr],
@@ -218,10 +218,10 @@ def _pointer_array(tensors):
 
 def decode_advance(prev_tokens: torch.Tensor, token_ids: torch.Tensor, positions: torch.Tensor,
                    context_lens: torch.Tensor, n_live: torch.Tensor, table_rows: Optional[torch.Tensor], tables, slots,
-                   page_size: int) -> None:
+                   page_size: int, draw_index: Optional[torch.Tensor] = None) -> None:
     """Between two decode steps queued back to back: rows below ``n_live[0]`` move one position on, take
-    ``prev_tokens`` as their input and get their new slots from ``tables`` (one [table rows, width] per cache
-    group; row r of the batch has the table row ``table_rows[r]``, or r without it)."""
+    ``prev_tokens`` as their input, count ``draw_index`` up by one and get their new slots from ``tables`` (one
+    [table rows, width] per cache group; row r of the batch has the table row ``table_rows[r]``, or r without it)."""
     R = token_ids.numel()
     for t, name in ((prev_tokens, "prev_tokens"), (token_ids, "token_ids"), (positions, "positions"),
                     (context_lens, "context_lens")):
@@ -232,14 +232,16 @@ def decode_advance(prev_tokens: torch.Tensor, token_ids: torch.Tensor, positions
     width = tables[0].shape[1] if tables else 1
     if table_rows is not None:
         _check(table_rows, "table_rows", torch.int32, (R,))
+    if draw_index is not None:
+        _check(draw_index, "draw_index", torch.int32, (R,))
     for t, sl in zip(tables, slots):
         _check(t, "table", torch.int32, (None if table_rows is not None else R, width))
         _check(sl, "slots", torch.int32, (R,))
     keep_t, tp = _pointer_array(tables)
     keep_s, sp = _pointer_array(slots)
     _call("ms_decode_advance", prev_tokens.data_ptr(), token_ids.data_ptr(), positions.data_ptr(),
-          context_lens.data_ptr(), n_live.data_ptr(), _ptr(table_rows), tp, sp, len(tables), width, page_size, R,
-          _stream())
+          context_lens.data_ptr(), n_live.data_ptr(), _ptr(table_rows), _ptr(draw_index), tp, sp, len(tables), width,
+          page_size, R, _stream())
 
 
 def table_update(tables, index, value, counts: torch.Tensor, max_updates: int) -> None:

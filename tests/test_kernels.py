@@ -373,8 +373,11 @@ def test_decode_advance(ops, page_size, through_rows):
     slots = [torch.full((R,), -7, dtype=torch.int32) for _ in range(2)]
     dev = lambda t: t.clone().to(DEV)
     d_tok, d_pos, d_ctx, d_slots = dev(toks), dev(pos), dev(ctx), [dev(s_) for s_ in slots]
+    draws = torch.arange(10, 10 + R, dtype=torch.int32, device=DEV)
     ops.decode_advance(dev(prev), d_tok, d_pos, d_ctx, torch.tensor([live], dtype=torch.int32, device=DEV),
-                       dev(rows) if through_rows else None, [dev(t) for t in tables], d_slots, page_size)
+                       dev(rows) if through_rows else None, [dev(t) for t in tables], d_slots, page_size,
+                       draws if through_rows else None)
+    assert draws.tolist() == [10 + r + (1 if r < live and through_rows else 0) for r in range(R)]
     for r in range(R):
         if r < live:
             p = int(pos[r]) + 1

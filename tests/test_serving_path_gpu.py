@@ -192,12 +192,18 @@ def test_sampled_tokens_do_not_depend_on_graphs(tiny_d, eng):
     with_graphs = eng.LLM(model, hip_graphs=True, decode_steps_per_launch=8, **kw)
     without = eng.LLM(model, hip_graphs=False, **kw)
     a = with_graphs.generate(prompts, sp)
+    # the draws happened on the device, eight steps to a launch, from graphs that hold the sampling kernels
+    assert any(rec.decode_steps == 8 for rec in with_graphs.engine.steps)
+    assert (4, False, 8, "sampled", True, True) in with_graphs.engine.runner.graphs.buckets
     b = without.generate(prompts, sp)
     assert [o.token_ids for o in a] == [o.token_ids for o in b]
     assert len({tuple(o.token_ids) for o in a}) == 4
     assert with_graphs.engine.runner.graphs.launches > 0
     other = with_graphs.generate(prompts[:1], eng.SamplingParams(max_new_tokens=20, temperature=0.8, top_k=20, top_p=0.9, seed=7))
     assert other[0].token_ids != a[0].token_ids
+    t_only = eng.SamplingParams(max_new_tokens=20, temperature=0.9, seed=3)
+    assert [o.token_ids for o in with_graphs.generate(prompts, t_only)] == [o.token_ids for o in without.generate(prompts, t_only)]
+    assert (4, False, 8, "sampled", False, False) in with_graphs.engine.runner.graphs.buckets
     greedy = with_graphs.generate(prompts, eng.SamplingParams(max_new_tokens=20))
     assert any(rec.decode_steps == 8 for rec in with_graphs.engine.steps)
     k1 = with_graphs.generate(prompts, eng.SamplingParams(max_new_tokens=20, temperature=1.3, top_k=1, seed=5))
