@@ -43,6 +43,9 @@ int ms_rope_store(void* qkv, const float* bias, const int* positions, const floa
                   void* v_pages, int n_tokens, int num_heads, int num_kv_heads, int head_dim, int rot_dim,
                   int page_size, int v_transposed, int dtype, hipStream_t stream);
 
+// table float [n_tokens, half, 2] = (cos, sin) of float(positions[n]) * inv_freq[j]
+int ms_rope_table(const int* positions, const float* inv_freq, float* table, int n_tokens, int half, hipStream_t stream);
+
 int ms_gemm_generic(const void* A, const void* W, const float* bias, void* C, int M, int N, int K, long long lda,
                     long long ldw, long long ldc, int in_dtype, int out_dtype, int accumulate, hipStream_t stream);
 
@@ -73,6 +76,14 @@ int ms_gemm_tiled(const void* A, long long lda, const void* W, long long ldw, vo
 void ms_gemm_tiled_force(int tile);
 int ms_gemm_tiled_pays(int M, int N, int K);
 int ms_gemm_tiled_plain_pays(int M, int N, int K);   // the same question for a plain product (epilogue 0)
+
+// The q/k/v product of many tokens with bias, rotation (whole heads, pairs (j, j + d/2)) and the store of k and v
+// into the cache pages as its epilogue: A [M, lda] bfloat16, W [(nh + 2 nkv) d, ldw], q_out [M, nh d] bfloat16;
+// head_dim 64 or 128; rope_table float [M, d / 2, 2] from ms_rope_table.  Pages as in ms_rope_store.  ms_gemm_tiled_qkv_pays: where it beats product + rotation kernel.
+int ms_gemm_tiled_qkv(const void* A, long long lda, const void* W, long long ldw, const float* bias,
+                      const float* rope_table, const int* slot_mapping, void* q_out, void* k_pages, void* v_pages, int M,
+                      int K, int nh, int nkv, int head_dim, int page_size, int v_transposed, hipStream_t stream);
+int ms_gemm_tiled_qkv_pays(int M, int N, int K, int head_dim);
 
 int ms_gemm_skinny_norm(const float* x, long long ldx, const int* rows, const float* norm_w, float eps, const void* W,
                         long long ldw, const float* bias, void* out, long long ldo, int M, int N, int K, int epilogue,

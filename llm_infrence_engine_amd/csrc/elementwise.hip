@@ -368,6 +368,29 @@ rope_store_vec_kernel(T* __restrict__ qkv, const float* __restrict__ bias, const
   }
 }
 
+// table[n][j] = (cos, sin) of float(positions[n]) * inv_freq[j], by the short routine that the rotation kernels for
+// bfloat16 use: worked out once a step, the same for every layer.
+__global__ void rope_table_kernel(const int* __restrict__ positions, const float* __restrict__ inv_freq,
+                                  float2* __restrict__ table, int n_tokens, int half) {
+  const int id = blockIdx.x * blockDim.x + threadIdx.x;
+  if (id >= n_tokens * half) return;
+  const int n = id / half, j = id - n * half;
+  float sn, cs;
+  ms_sincos_rot((float)positions[n] * inv_freq[j], &sn, &cs);
+  table[id] = make_float2(cs, sn);
+}
+
+extern "C" int ms_rope_table(const int* positions, const float* inv_freq, float* table, int n_tokens, int half,
+                             hipStream_t stream) {
+  if (n_tokens <= 0 || half <= 0) return MS_OK;
+  if (!positions || !inv_freq || !table || (uintptr_t)table % 8) return MS_BAD_ARG;
+  const long long total = (long long)n_tokens * half;
+  if (total > 0x7fffffffLL) return MS_UNSUPPORTED;
+  rope_table_kernel<<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream>>>(positions, inv_freq, (float2*)table,
+                                                                                   n_tokens, half);
+  return ms_launch_status();
+}
+
 extern "C" int ms_rope_store(void* qkv, const float* bias, const int* positions, const float* inv_freq, const int* slot_mapping,
                              void* k_pages, void* v_pages, int n_tokens, int num_heads, int num_kv_heads,
                              int head_dim, int rot_dim, int page_size, int v_transposed, int dtype,

@@ -175,6 +175,7 @@ class StepGraphs:
         bk.buf.send()
 
         def body():
+            ctx.shared.clear()     # what parts derive from the step's tensors is worked out inside every run
             if G:
                 runner.pools.apply_updates([f[f"update_index{g}"] for g in range(G)],
                                            [f[f"update_value{g}"] for g in range(G)], f["update_counts"], lay.n_updates)
@@ -188,6 +189,7 @@ class StepGraphs:
                     ops.decode_advance(bk.tokens[k - 1], f["token_ids"], f["positions"], f["context_lens"], f["n_live"],
                                        f["state_slots"], runner.pools.tables, bk.slots, self.manager.page_size,
                                        f["draw_index"] if bk.sampled else None)
+                    ctx.shared.clear()
                 bk.logits = model.head_logits(*model.forward_hidden(ctx, caches), ctx.logit_rows)
                 if bk.sampled:     # rows without a temperature (padding rows too) take the first maximum
                     ops.sample(bk.logits, bk.tokens[k], f["temperature"], f["top_k"], f["top_p"], f["seeds"], f["draw_index"],

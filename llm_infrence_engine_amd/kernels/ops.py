@@ -46,6 +46,10 @@ _SIGNATURES = {
     "ms_gemm_tiled_force": [_c_int],
     "ms_gemm_tiled_pays": [_c_int, _c_int, _c_int],
     "ms_gemm_tiled_plain_pays": [_c_int, _c_int, _c_int],
+    "ms_gemm_tiled_qkv": [_c_ptr, _c_ll, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int,
+                          _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "ms_rope_table": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
+    "ms_gemm_tiled_qkv_pays": [_c_int, _c_int, _c_int, _c_int],
     "ms_read_probe_blocks": [],
     "ms_read_probe": [_c_ptr, _c_ll, _c_ptr, _c_ptr],
     "ms_residual_add": [_c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr],
@@ -450,6 +454,49 @@ def gemm_tiled(a: torch.Tensor, w: torch.Tensor, epilogue: int = EPI_STORE) -> t
     out = torch.empty((M, N // 2 if epilogue == EPI_SWIGLU else N), dtype=torch.bfloat16, device=a.device)
     _call("ms_gemm_tiled", a.data_ptr(), K, w.data_ptr(), K, out.data_ptr(), out.shape[1], M, N, K, epilogue, _stream())
     return out
+
+
+def gemm_tiled_qkv_pays(a, w: torch.Tensor, head_dim: int, rot_dim: int, k_pages: torch.Tensor) -> bool:
+    """Whether ``gemm_tiled_qkv`` takes these operands (bfloat16 rows, heads of 64 or 128 rotated whole) and is the
+    faster way from a portion's normed rows to q and the cache."""
+    return (isinstance(a, torch.Tensor) and a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.dim() == 2
+            and a.is_contiguous() and w.is_contiguous() and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
+            and rot_dim == head_dim and k_pages.dtype == torch.bfloat16
+            and bool(_get("ms_gemm_tiled_qkv_pays")(a.shape[0], w.shape[0], a.shape[1], head_dim)))
+
+
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
+    """float [N, half, 2]: (cos, sin) of float(positions[n]) * inv_freq[j], for ``gemm_tiled_qkv``."""
+    _check(positions, "positions", torch.int32)
+    _check(inv_freq, "inv_freq", torch.float32)
+    n, half = positions.numel(), inv_freq.numel()
+    table = torch.empty((n, half, 2), dtype=torch.float32, device=positions.device)
+    _call("ms_rope_table", positions.data_ptr(), inv_freq.data_ptr(), table.data_ptr(), n, half, _stream())
+    return table
+
+
+def gemm_tiled_qkv(a: torch.Tensor, w_qkv: torch.Tensor, bias: Optional[torch.Tensor], nh: int, nkv: int, d: int,
+                   table: torch.Tensor, slot_mapping: torch.Tensor, k_pages: torch.Tensor,
+                   v_pages: torch.Tensor, v_transposed: bool = False) -> torch.Tensor:
+    """a [M, K] @ w_qkv [(nh + 2 nkv) d, K].T (+ bias) on the matrix cores with the rotation of q and k and the
+    store of k and v into the pages as the product's epilogue; returns q [M, nh d].  ``table`` is
+    ``rope_table(positions, inv_freq)`` with d / 2 frequencies (whole heads are rotated); pages as in
+    ``rope_store``."""
+    _check(a, "a", torch.bfloat16)
+    M, K = a.shape
+    _check(w_qkv, "w_qkv", torch.bfloat16, ((nh + 2 * nkv) * d, K))
+    _check(table, "table", torch.float32, (M, d // 2, 2))
+    _check(slot_mapping, "slot_mapping", torch.int32, (M,))
+    if bias is not None:
+        _check(bias, "bias", torch.float32, ((nh + 2 * nkv) * d,))
+    _check(k_pages, "k_pages", torch.bfloat16, (None, nkv, None, d))
+    page_size = k_pages.shape[2]
+    _check(v_pages, "v_pages", torch.bfloat16, _v_shape(k_pages, v_transposed))
+    q = torch.empty((M, nh * d), dtype=torch.bfloat16, device=a.device)
+    _call("ms_gemm_tiled_qkv", a.data_ptr(), K, w_qkv.data_ptr(), K, _ptr(bias), table.data_ptr(),
+          slot_mapping.data_ptr(), q.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(), M, K, nh,
+          nkv, d, page_size, int(bool(v_transposed)), _stream())
+    return q
 
 
 def skinny_norm_ok(x: torch.Tensor, w: torch.Tensor, n_rows: int) -> bool:

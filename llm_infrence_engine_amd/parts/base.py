@@ -151,6 +151,9 @@ class StepContext:
     q_lens_host: List[int] = field(default_factory=list)
     start_pos_host: List[int] = field(default_factory=list)
     state_slots_host: List[int] = field(default_factory=list)
+    # what a part derives from the step's tensors once for all layers that hold a part like it (key: the part's
+    # choice); whoever changes ``positions`` in place empties it
+    shared: dict = field(default_factory=dict)
 
     @property
     def decode_only(self) -> bool:

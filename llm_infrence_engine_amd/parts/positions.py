@@ -27,6 +27,16 @@ class RotaryHalf(PositionEncoding):
         self.inv_freq = (1.0 / (self.theta ** (j / self.rotary_dim))).to(torch.float32).to(rt.device)
 
     def project_encode_store(self, h, w_qkv, bias, num_heads, num_kv_heads, head_dim, ctx, kv):
+        if (kv is not None and kv.store
+                and ops.gemm_tiled_qkv_pays(h, w_qkv, head_dim, self.rotary_dim, kv.k_pages)):
+            # a portion of a prompt: rotation and cache store are the product's epilogue; the cosines and sines of
+            # the step's positions are worked out by the first layer that comes here and shared by the others
+            key = ("rotary_half", self.rotary_dim, self.theta)
+            table = ctx.shared.get(key)
+            if table is None:
+                table = ctx.shared[key] = ops.rope_table(ctx.positions, self.inv_freq)
+            return ops.gemm_tiled_qkv(h, w_qkv, bias, num_heads, num_kv_heads, head_dim, table, kv.slot_mapping,
+                                      kv.k_pages, kv.v_pages, kv.v_transposed)
         if not (isinstance(h, linear.LazyNorm) and h.rows is None and kv is not None and kv.store
                 and ops.qkv_rope_store_ok(h.x, w_qkv, head_dim, self.rotary_dim) and ops.qkv_rope_store_pays(h.x, w_qkv)):
             return None

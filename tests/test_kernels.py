@@ -689,12 +689,13 @@ def test_gemm_skinny_refuses_what_it_cannot_take(ops):
         ops.gemm_skinny(a[:4, :60], w[:, :60].contiguous())
 
 
-@pytest.mark.parametrize("tile", [1, 2, 3])
+@pytest.mark.parametrize("tile", [1, 2, 3, 4, 5])
 @pytest.mark.parametrize("M,N,K", [(65, 662, 64), (300, 2 * 331, 192), (257, 130, 896), (1000, 2 * 4864, 896), (2051, 1026, 128),
                                    (130, 16, 64), (513, 4100, 1536)])
 def test_gemm_tiled(ops, M, N, K, tile):
-    """The many-rows product and its gated epilogue with either tile shape: rows and features that fill no
-    whole tile, one step of 64 columns and many."""
+    """The many-rows product and its gated epilogue with every tile shape (256, 128, 64, 192 and 160 features wide:
+    the last two store a lane's results in pieces of 8 and 4 bytes): rows and features that fill no whole tile, rows
+    of the result that start at odd addresses, one step of 64 columns and many."""
     force = ops._get("ms_gemm_tiled_force")
     force.restype = None
     g = torch.Generator().manual_seed(M + N)
@@ -1054,6 +1055,59 @@ def _qkv_fused_case(ops, M, nh, nkv, d, K, v_transposed):
     untouched = torch.ones(pages * page_size, dtype=torch.bool)
     untouched[slots[slots >= 0].long().cpu()] = False
     assert (kp1.permute(0, 2, 1, 3).reshape(pages * page_size, -1)[untouched.to(DEV)] == 0).all()
+
+
+@pytest.mark.parametrize("M", [65, 130, 700])
+@pytest.mark.parametrize("nh,nkv,d,K,v_transposed,tile", [(14, 2, 64, 896, True, 0), (3, 1, 64, 128, False, 2),
+                                                            (5, 5, 64, 192, True, 3), (3, 1, 128, 256, True, 0),
+                                                            (2, 2, 128, 64, False, 0)])
+def test_gemm_tiled_qkv_equals_product_rotation_and_store(ops, M, nh, nkv, d, K, v_transposed, tile):
+    """The many-rows q/k/v product with bias, rotation and cache store as its epilogue, against a double product
+    and the plain rotation: every tile shape, tokens and heads that fill no whole tile, one token not stored, pages
+    plain and transposed, positions up to thousands."""
+    g = torch.Generator().manual_seed(M + d + K)
+    page_size = 16
+    pages = (M + page_size - 1) // page_size + 3
+    a = torch.randn(M, K, generator=g).bfloat16().to(DEV)
+    w = (torch.randn((nh + 2 * nkv) * d, K, generator=g) / math.sqrt(K)).bfloat16().to(DEV)
+    bias = torch.randn((nh + 2 * nkv) * d, generator=g).to(DEV) if K != 128 else None
+    pos = torch.randint(0, 3000, (M,), generator=g).to(torch.int32).to(DEV)
+    slots = torch.randperm(pages * page_size, generator=g)[:M].to(torch.int32)
+    slots[2] = -1
+    slots = slots.to(DEV)
+    inv_freq = (1.0 / (1e6 ** (torch.arange(0, d, 2, dtype=torch.float64) / d))).float().to(DEV)
+    vshape = (pages, nkv, d, page_size) if v_transposed else (pages, nkv, page_size, d)
+    kp = torch.zeros(pages, nkv, page_size, d, dtype=torch.bfloat16, device=DEV)
+    vp = torch.zeros(vshape, dtype=torch.bfloat16, device=DEV)
+    assert ops.gemm_tiled_qkv_pays(a, w, d, d, kp)
+    assert not ops.gemm_tiled_qkv_pays(a, w, d, d // 2, kp)       # a rotation over part of the head is not taken
+    force = ops._get("ms_gemm_tiled_force")
+    force(tile)
+    try:
+        table = ops.rope_table(pos, inv_freq)
+        q = ops.gemm_tiled_qkv(a, w, bias, nh, nkv, d, table, slots, kp, vp, v_transposed)
+    finally:
+        force(0)
+    ang = pos.cpu().float()[:, None] * inv_freq.cpu()[None]      # the float product, as the kernel forms it
+    torch.testing.assert_close(table.cpu().double(), torch.stack((ang.double().cos(), ang.double().sin()), -1),
+                               atol=1e-6, rtol=0)
+    exact = a.double().cpu() @ w.double().cpu().T
+    if bias is not None:
+        exact = exact + bias.double().cpu()
+    exact = exact.view(M, nh + 2 * nkv, d)
+    rot = rope_reference(exact[:, :nh + nkv], pos.cpu(), d, inv_freq.double().cpu())
+    t = dict(atol=3e-2, rtol=1.6e-2)
+    torch.testing.assert_close(q.double().cpu().view(M, nh, d), rot[:, :nh], **t)
+    sl = slots.cpu()
+    stored = sl >= 0
+    pg, off = (sl[stored] // page_size).long(), (sl[stored] % page_size).long()
+    torch.testing.assert_close(kp.cpu()[pg, :, off].double(), rot[stored][:, nh:], **t)
+    v = vp.cpu().permute(0, 1, 3, 2) if v_transposed else vp.cpu()
+    torch.testing.assert_close(v[pg, :, off].double(), exact[stored][:, nh + nkv:], **t)
+    untouched = torch.ones(pages * page_size, dtype=torch.bool)
+    untouched[sl[stored].long()] = False
+    assert (kp.cpu().permute(0, 2, 1, 3).reshape(pages * page_size, -1)[untouched] == 0).all()
+    assert (v.permute(0, 2, 1, 3).reshape(pages * page_size, -1)[untouched] == 0).all()
 
 
 # the products of a decode step at the shapes of the published checkpoints: (rows of W, columns) of the packed
