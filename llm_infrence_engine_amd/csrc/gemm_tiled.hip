@@ -86,7 +86,7 @@ __device__ __forceinline__ void store_run(bf16* o, const float* v, int valid) {
 template <int WF, int WT, int FT, int TT, int EPI, typename TO>
 __global__ void __launch_bounds__(WF * WT * MS_WAVE)
 gemm_tiled_kernel(const bf16* __restrict__ A, size_t lda, const bf16* __restrict__ W, size_t ldw,
-                  TO* __restrict__ out, size_t ldo, int M, int N, int K, int m_tiles, int n_tiles, QkvEpilogue qkv) {
+                  TO* __restrict__ out, size_t ldo, int M, int N, int K, int m_tiles, int n_tiles, int xm, QkvEpilogue qkv) {
   constexpr int NWAVES = WF * WT, THREADS = NWAVES * MS_WAVE;
   constexpr int BN = WF * FT * 16, BM = WT * TT * 16, ROWS = BN + BM;
   constexpr int LOADS = (ROWS / 8 + NWAVES - 1) / NWAVES;   // loads of 8 rows (1 KB) a wave makes per step at most
@@ -95,12 +95,16 @@ gemm_tiled_kernel(const bf16* __restrict__ A, size_t lda, const bf16* __restrict
   extern __shared__ __align__(16) unsigned char lds_raw[];
   bf16* lds = reinterpret_cast<bf16*>(lds_raw);          // two buffers of ROWS x PITCH
 
-  // Blocks with consecutive ids go to consecutive XCDs, each with an L2 of its own: an XCD takes every eighth
-  // tile of W with all token tiles (those fastest), so a tile of W is read from memory by one XCD only.  The
-  // host launches 8 * ceil(n_tiles / 8) * m_tiles blocks; one without a tile leaves.
-  const int nt = ((int)(blockIdx.x >> 3) / m_tiles) * 8 + (blockIdx.x & 7);
-  const int mt = (int)(blockIdx.x >> 3) % m_tiles;
-  if (nt >= n_tiles) return;
+  // Blocks with consecutive ids go to consecutive XCDs, each with an L2 of its own.  The 8 XCDs are laid over the
+  // tiles as xm x (8 / xm): an XCD takes every xm-th token tile and every (8 / xm)-th tile of W, its token tiles
+  // running fastest (they share a tile of W at the same time).  With xm = 1 a tile of W is read from memory by
+  // one XCD only and every XCD reads all of A; a larger xm leaves an XCD 1 / xm of A to keep in its L2.  The host
+  // launches 8 * ceil(m_tiles / xm) * ceil(n_tiles / (8 / xm)) blocks; one without a tile leaves.
+  const int xcd = blockIdx.x & 7, local = (int)(blockIdx.x >> 3);
+  const int xn = 8 / xm, mi = (m_tiles + xm - 1) / xm;
+  const int nt = (local / mi) * xn + xcd / xm;
+  const int mt = (local % mi) * xm + xcd % xm;
+  if (nt >= n_tiles || mt >= m_tiles) return;
   const int n0 = nt * BN, m0 = mt * BM;
   const int lane = threadIdx.x & (MS_WAVE - 1), wave = threadIdx.x / MS_WAVE;
   const int wf = wave % WF, wt = wave / WF;
@@ -268,6 +272,17 @@ gemm_tiled_kernel(const bf16* __restrict__ A, size_t lda, const bf16* __restrict
   }
 }
 
+int g_xcd_split = 0;   // measurements: 0 leaves the choice, 1, 2, 4, 8 force the number of XCD rows
+
+// Over how many XCDs the token tiles are spread (see the kernel).  Measured at the gate/up shapes of 0.5B to 32B:
+// no difference up to 4,096 tokens; at 8,192 tokens of the 0.5B and 1.5B shapes four rows of XCDs take 143 against
+// 155 us and 406 against 425 (an XCD then keeps a quarter of A in its L2 instead of fetching all of it again and
+// again), two rows lie between.
+int choose_xcd_split(int M) {
+  if (g_xcd_split) return g_xcd_split;
+  return M >= 6144 ? 4 : (M >= 4096 ? 2 : 1);
+}
+
 template <int WF, int WT, int FT, int TT, int EPI, typename TO>
 int launch(const bf16* A, size_t lda, const bf16* W, size_t ldw, TO* out, size_t ldo, int M, int N, int K,
            hipStream_t stream, const QkvEpilogue& qkv = QkvEpilogue{}) {
@@ -281,10 +296,11 @@ int launch(const bf16* A, size_t lda, const bf16* W, size_t ldw, TO* out, size_t
     raised = true;
   }
   const int n_tiles = (N + BN - 1) / BN, m_tiles = (M + BM - 1) / BM;
-  const long long blocks = (long long)((n_tiles + 7) / 8) * 8 * m_tiles;
+  const int xm = choose_xcd_split(M);
+  const long long blocks = 8LL * ((m_tiles + xm - 1) / xm) * ((n_tiles + 8 / xm - 1) / (8 / xm));
   if (blocks > 0x7fffffffLL) return MS_UNSUPPORTED;
   gemm_tiled_kernel<WF, WT, FT, TT, EPI, TO><<<dim3((unsigned)blocks), dim3(WF * WT * MS_WAVE), lds, stream>>>(
-      A, lda, W, ldw, out, ldo, M, N, K, m_tiles, n_tiles, qkv);
+      A, lda, W, ldw, out, ldo, M, N, K, m_tiles, n_tiles, xm, qkv);
   return ms_launch_status();
 }
 
@@ -325,6 +341,7 @@ TileChoice choose_tile(int M, int N, int K) {
 }  // namespace
 
 extern "C" void ms_gemm_tiled_force(int tile) { g_tile = tile; }
+extern "C" void ms_gemm_tiled_force_xcd_split(int xm) { g_xcd_split = xm; }
 
 // Whether the gated product of M tokens is faster here than as the library's product and an activation kernel
 // (measured with a different W every call, 65 to 8,192 tokens): up to 1,536 columns always (0.5 to 0.98 of the

@@ -44,6 +44,7 @@ _SIGNATURES = {
                              _c_ptr, _c_int, _c_ptr],
     "ms_gemm_tiled": [_c_ptr, _c_ll, _c_ptr, _c_ll, _c_ptr, _c_ll, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "ms_gemm_tiled_force": [_c_int],
+    "ms_gemm_tiled_force_xcd_split": [_c_int],
     "ms_gemm_tiled_pays": [_c_int, _c_int, _c_int],
     "ms_gemm_tiled_plain_pays": [_c_int, _c_int, _c_int],
     "ms_gemm_tiled_qkv": [_c_ptr, _c_ll, _c_ptr, _c_ll, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int,

@@ -691,11 +691,12 @@ def test_gemm_skinny_refuses_what_it_cannot_take(ops):
 
 @pytest.mark.parametrize("tile", [1, 2, 3, 4, 5])
 @pytest.mark.parametrize("M,N,K", [(65, 662, 64), (300, 2 * 331, 192), (257, 130, 896), (1000, 2 * 4864, 896), (2051, 1026, 128),
-                                   (130, 16, 64), (513, 4100, 1536)])
+                                   (130, 16, 64), (513, 4100, 1536), (4100, 2 * 331, 64), (6200, 1300, 128)])
 def test_gemm_tiled(ops, M, N, K, tile):
     """The many-rows product and its gated epilogue with every tile shape (256, 128, 64, 192 and 160 features wide:
     the last two store a lane's results in pieces of 8 and 4 bytes): rows and features that fill no whole tile, rows
-    of the result that start at odd addresses, one step of 64 columns and many."""
+    of the result that start at odd addresses, one step of 64 columns and many, and so many tokens that the tiles are
+    laid over the XCDs in two and in four rows."""
     force = ops._get("ms_gemm_tiled_force")
     force.restype = None
     g = torch.Generator().manual_seed(M + N)
