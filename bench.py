@@ -39,6 +39,8 @@ PROMPT_LEN = 512
 CONTEXT_LIMIT = 8192
 BLOCK_SIZE = 16
 PREFILL_TOKENS = 2048
+LONG_PROMPT = 7600          # a further point: decoding behind prompts of this length
+LONG_PREFILL = 8192         # and a prompt step of this many tokens
 DECODE_STEPS_PER_LAUNCH = 8   # decode steps queued in one graph launch (a stop id is noticed that many steps late at most)
 # the reference's own decode at batch 8: CUDA-graph step of 6.0 ms on an A10, context 128 (docs/RESULTS.md:38)
 REFERENCE_TOKS = 8 / 6.0e-3
@@ -184,20 +186,20 @@ def run_sampler(vocab, batches=(8, 64), repeats=20):
     return out
 
 
-def run_prefill(eng_mod, model, vocab, seed, repeats=5):
+def run_prefill(eng_mod, model, vocab, seed, repeats=5, tokens=PREFILL_TOKENS):
     import numpy as np
     import torch
 
     from llm_infrence_engine_amd.engine import ModelRunner, StepEntry
 
     rng = np.random.default_rng(seed)
-    runner = ModelRunner(model, BLOCK_SIZE, PREFILL_TOKENS // BLOCK_SIZE + 1, 1, PREFILL_TOKENS + BLOCK_SIZE)
+    runner = ModelRunner(model, BLOCK_SIZE, tokens // BLOCK_SIZE + 1, 1, tokens + BLOCK_SIZE)
     best = None
     for i in range(repeats + 1):
-        toks = [int(t) for t in rng.integers(0, vocab, PREFILL_TOKENS)]
+        toks = [int(t) for t in rng.integers(0, vocab, tokens)]
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        runner.step([StepEntry("p", toks, [PREFILL_TOKENS - 1])])
+        runner.step([StepEntry("p", toks, [tokens - 1])])
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         runner.free_request("p")
@@ -322,6 +324,15 @@ def main() -> int:
         dts, _, _ = run_decode(eng, model, a.batch, min(a.steps, 128), 16, vocab, seed=9, prompt_len=a.prompt_len,
                                sampling=dict(temperature=0.8, top_k=50, top_p=0.9))
         out["points"][f"decode_b{a.batch}_sampled"] = round(a.batch / dts, 1)
+        if a.shape == "0.5b":       # a long context: decoding behind 7,600-token prompts, and a prompt of 8,192 tokens
+            dtl, ctxl, _ = run_decode(eng, model, a.batch, 64, 8, vocab, seed=11, prompt_len=LONG_PROMPT)
+            out["points"].update({f"decode_b{a.batch}_ctx{LONG_PROMPT}_ms_per_step": round(dtl * 1e3, 4),
+                                  f"decode_b{a.batch}_ctx{LONG_PROMPT}_frac":
+                                      round(decode_bytes(cfg, a.batch, ctxl) / dtl / 1e9 / HBM_GBS, 4)})
+            ptl = run_prefill(eng, model, vocab, seed=12, repeats=3, tokens=LONG_PREFILL)
+            out["points"].update({f"prefill_{LONG_PREFILL}_ms": round(ptl * 1e3, 3),
+                                  f"prefill_{LONG_PREFILL}_frac":
+                                      round(prefill_flops(cfg, LONG_PREFILL) / ptl / 1e12 / PEAK_TFLOPS["bf16"], 4)})
         out["sampler"] = run_sampler(vocab)
     if a.shape == "0.5b" and not a.no_points and not a.no_shapes and a.layers == shape["num_hidden_layers"]:
         del model
