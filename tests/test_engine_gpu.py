@@ -133,6 +133,48 @@ def test_mid_flight_join_and_cancel(tiny, eng):
     assert all(g.allocator.num_in_use() == 0 for g in e.runner.manager.groups)
 
 
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_random_arrivals_cancels_and_scarce_pages_keep_outputs(tiny, eng, seed):
+    """Requests of random lengths that arrive at random steps, some cancelled on the way, under a random token
+    budget and a pool that cannot hold them all: whatever the scheduler does (portions, preemption, recomputation,
+    pages used again), every request that finishes has the plain implementation's tokens, the cache manager's
+    books balance after every step, and every page and slot comes back."""
+    name, d, cfg, w = tiny
+    rng = np.random.default_rng(100 + seed)
+    n = 9
+    prompts = [[int(t) for t in rng.integers(0, cfg["vocab_size"], int(rng.integers(1, 30)))] for _ in range(n)]
+    new = [int(rng.integers(1, 14)) for _ in range(n)]
+    arrive = sorted(int(rng.integers(0, 25)) for _ in range(n))
+    cancel_at = {int(i): int(rng.integers(2, 30)) for i in rng.choice(n, 2, replace=False)}
+    model = eng.load_model(d, "float32")
+    block = int(rng.choice([2, 4, 8]))
+    longest = max(len(p) + k for p, k in zip(prompts, new))
+    pages_of_longest = -(-longest // block) + 1
+    e = eng.Engine(model, num_blocks=pages_of_longest + int(rng.integers(1, 2 * pages_of_longest)), block_size=block,
+                   max_seqs=int(rng.integers(2, 5)), max_len=64, max_num_batched_tokens=int(rng.integers(6, 40)))
+    reqs, step = {}, 0
+    while step < 400 and (len(reqs) < n or e.has_work()):
+        for i in range(n):
+            if i not in reqs and arrive[i] <= step:
+                reqs[i] = e.add_request(eng.Request(prompts[i], max_new_tokens=new[i]))
+        for i, at in cancel_at.items():
+            if at == step and i in reqs:
+                e.cancel(reqs[i])
+        if e.has_work():
+            e.step()
+            e.runner.manager.check_invariants()
+        step += 1
+    assert len(reqs) == n and not e.has_work()
+    for i, r in reqs.items():
+        want = P.greedy_generate(w, cfg, prompts[i], new[i])
+        if r.finish_reason == "abort":
+            assert r.output_ids == want[:len(r.output_ids)]      # what it got before the cancel was right
+        else:
+            assert r.finish_reason == "length" and r.output_ids == want, (seed, i)
+    assert sum(r.finish_reason != "abort" for r in reqs.values()) >= n - 2
+    assert all(g.allocator.num_in_use() == 0 for g in e.runner.manager.groups)
+
+
 def test_long_decoding_and_first_tokens(tiny, eng):
     """Decode 150 tokens one by one from a 3-token prompt in bfloat16 and float32: the first tokens of a
     sequence and positions far past several pages, checked against the plain logits along the way."""
