@@ -3,7 +3,8 @@
 // interleaved gate/up weight never goes to memory, which saves the write of [M, 2I], its read and a kernel.
 //
 // A block of 8 waves owns a tile of BN features by BM tokens, as large as registers allow (256 x 256: a byte
-// loaded does 128 multiply-adds; a CU draws some 80 GB/s from L2).  Per step of 64 columns the tile's rows of W
+// loaded does 128 multiply-adds; a CU draws 100 GB/s and more from its XCD's L2 but 27 GB/s from beyond it, some
+// 40 GB/s in this kernel, where a fifth of the requests miss).  Per step of 64 columns the tile's rows of W
 // and A go from memory straight to LDS (global_load_lds, 16 bytes a lane: no registers, no LDS write
 // instructions) into one of two buffers, a step before they are multiplied.  LDS rows are 128 bytes with their
 // eight 16-byte pieces permuted by the row number (piece c at place c ^ (row & 7)): fragment reads then run at
