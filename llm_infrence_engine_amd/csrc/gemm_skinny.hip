@@ -26,8 +26,10 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 enum { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_RESIDUAL = 3 };
 
-// The tiles are dealt out evenly: the first `rem` blocks take q + 1 tiles, the others q (at most NTILE), so that
-// every CU streams about the same share of W.
+// The rows of W are dealt out evenly in units of four (what a lane holds of a tile): the first `rem` blocks take
+// q + 1 units, the others q, at most NTILE tiles of 16 rows either way, the last of them filled in part.  A CU
+// draws from memory at a rate of its own, so a product is as slow as its block with the most rows: whole tiles
+// would leave 3 against 2 of them (0.5B gate/up, 608 tiles for 256 CUs) or 2 against 1 (32B o, 320 tiles).
 template <int MT, int NTILE, int WAVES, int EPI, typename TO, bool NORM>
 __global__ void __launch_bounds__(WAVES * MS_WAVE)
 gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restrict__ W, size_t ldw,
@@ -40,15 +42,19 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
   const float* X = (const float*)Av;
   const int lane = threadIdx.x & (MS_WAVE - 1), wave = threadIdx.x / MS_WAVE;
   const int col = lane & 15, kq = lane >> 4;
-  const int nt = q + ((int)blockIdx.x < rem ? 1 : 0);   // tiles of this block, at most NTILE
-  const int n0 = ((int)blockIdx.x * q + min((int)blockIdx.x, rem)) * 16;
+  const int n0 = ((int)blockIdx.x * q + min((int)blockIdx.x, rem)) * 4;
+  const int n1 = min(N, n0 + (q + ((int)blockIdx.x < rem ? 1 : 0)) * 4);   // this block's rows: n0 .. n1 - 1
+  const int nt = (n1 - n0 + 15) / 16;                                      // in tiles, at most NTILE
   const int m0 = blockIdx.y * 16 * MT;   // token groups beyond MT per block go to further blocks along y
   const int total_steps = (K + 31) / 32;
 
   const bf16* wrow[NTILE];
+  bool mine[NTILE];                // rows past the block's last are not loaded (their products are zero and not stored)
 #pragma unroll
-  for (int u = 0; u < NTILE; ++u)  // rows past the end repeat the last one; their results are not stored
+  for (int u = 0; u < NTILE; ++u) {
+    mine[u] = n0 + u * 16 + col < n1;
     wrow[u] = W + (size_t)min(n0 + u * 16 + col, N - 1) * ldw + kq * 8;
+  }
   size_t arow[MT];  // element offset of this lane's activation row and k slice
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
@@ -71,11 +77,11 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
   f32x4 bv[NTILE];        // bias of this lane's 4 features per tile
 #pragma unroll
   for (int u = 0; u < NTILE; ++u) {
-    const int nb = u < nt ? n0 + u * 16 + kq * 4 : N;   // N: nothing of this tile is this block's
+    const int nb = n0 + u * 16 + kq * 4;
     bv[u] = f32x4{0.f, 0.f, 0.f, 0.f};
     if (bias && EPI != EPI_SWIGLU) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) if (nb + r < N) bv[u][r] = bias[nb + r];
+      for (int r = 0; r < 4; ++r) if (nb + r < n1) bv[u][r] = bias[nb + r];
     }
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
@@ -83,7 +89,7 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
       if (EPI == EPI_RESIDUAL && wave == (u * MT + t) % WAVES && m0 + t * 16 + col < M) {
         const float* o = reinterpret_cast<const float*>(out) + (size_t)(m0 + t * 16 + col) * ldo + nb;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) if (nb + r < N) pre[u][t][r] = o[r];
+        for (int r = 0; r < 4; ++r) if (nb + r < n1) pre[u][t][r] = o[r];
       }
     }
   }
@@ -98,7 +104,7 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
 #pragma unroll
     for (int u = 0; u < NTILE; ++u) {
       wv[u] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
-      if (in && u < nt) wv[u] = *reinterpret_cast<const bf16x8*>(wrow[u] + k);
+      if (in && mine[u]) wv[u] = *reinterpret_cast<const bf16x8*>(wrow[u] + k);
     }
     f32x4 nw0 = {0.f, 0.f, 0.f, 0.f}, nw1 = {0.f, 0.f, 0.f, 0.f};
     if (NORM && in) {
@@ -170,7 +176,7 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
         // rows nb, nb+1 are (gate, up) of feature nb/2; rows nb+2, nb+3 of feature nb/2 + 1
 #pragma unroll
         for (int p = 0; p < 2; ++p) {
-          if (nb + 2 * p + 1 < N) {
+          if (nb + 2 * p + 1 < n1) {
             const float g = sum[2 * p], up = sum[2 * p + 1];
             out[(size_t)m * ldo + nb / 2 + p] = from_float<TO>(fast_silu(g) * up);
           }
@@ -181,7 +187,7 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
         // against 64 us)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          if (nb + r < N) o[r] = from_float<TO>(sum[r] + bv[u][r] + pre[u][t][r]);
+          if (nb + r < n1) o[r] = from_float<TO>(sum[r] + bv[u][r] + pre[u][t][r]);
         }
       }
     }
@@ -202,20 +208,22 @@ int launch_cfg(const void* A, size_t lda, const bf16* W, size_t ldw, const float
   const int steps = (K + 31) / 32;
   const int groups = (M + 16 * MT - 1) / (16 * MT);
   const int cus = ms_compute_units();
-  // Every CU should stream an equal share of the matrix: the tiles are dealt out evenly over a whole number of
-  // blocks per CU, of up to four tiles each (no last round that only some CUs take part in); an output with
-  // fewer tiles than CUs has a block per tile; with several token groups four tiles go to a block.
+  // Every CU should stream an equal share of the matrix: the rows are dealt out in units of four over a whole
+  // number of blocks per CU, of up to four tiles each (no last round that only some CUs take part in); an output
+  // with fewer tiles than CUs has a block per tile; with several token groups four tiles go to a block.
   // (Measured on the 0.5B shapes at 8 and 64 rows and on the 7B shapes at 8.)
-  int ntile, blocks;
-  if (tiles <= cus) { ntile = 1; blocks = tiles; }
-  else if (groups == 1 && tiles <= 16 * cus) {   // a whole number of blocks per CU, of up to four tiles each
-    blocks = cus * ((tiles + 4 * cus - 1) / (4 * cus));
-    ntile = (tiles + blocks - 1) / blocks;
-  } else { ntile = 4; blocks = (tiles + 3) / 4; }   // many rounds: the last one matters little (measured: the head)
+  const int units = (N + 3) / 4;
+  int blocks;
+  if (tiles <= cus) blocks = tiles;
+  else if (groups == 1 && tiles <= 16 * cus) blocks = cus * ((tiles + 4 * cus - 1) / (4 * cus));
+  else blocks = (tiles + 3) / 4;      // many rounds: the last one matters little (measured: the head)
+  if (g_force_ntile) blocks = (tiles + g_force_ntile - 1) / g_force_ntile;
+  const int q = units / blocks, rem = units % blocks;   // blocks * q + rem units
+  int ntile = (q + (rem ? 1 : 0) + 3) / 4;              // tiles of the block with the most rows
+  if (g_force_ntile && ntile <= g_force_ntile) ntile = g_force_ntile;
   int waves = ntile >= 3 ? (MT <= 2 && (MT == 1 || tiles < 1024) ? 8 : 4) : ((steps >= 32 || MT > 1) ? 16 : 8);
-  if (g_force_ntile) { ntile = g_force_ntile; waves = g_force_waves; blocks = (tiles + ntile - 1) / ntile; }
-  const int q = tiles / blocks, rem = tiles % blocks;   // blocks * q + rem tiles; q + (rem > 0) <= ntile
-  if (q + (rem ? 1 : 0) > ntile || (waves - 1) * ntile * MT > 60) return MS_UNSUPPORTED;  // LDS
+  if (g_force_ntile) waves = g_force_waves;
+  if (ntile > 4 || (waves - 1) * ntile * MT > 60) return MS_UNSUPPORTED;  // LDS
 #define GO(NT, WV) if (ntile == NT && waves == WV) { if constexpr ((WV - 1) * NT * MT <= 60) { gemm_skinny_kernel<MT, NT, WV, EPI, TO, NORM><<<dim3(blocks, groups), dim3(WV * MS_WAVE), 0, stream>>>(A, lda, W, ldw, bias, out, ldo, M, N, K, norm_w, eps, rows, q, rem); return ms_launch_status(); } }
   GO(4, 4) GO(4, 8) GO(3, 4) GO(3, 8) GO(2, 8) GO(2, 16) GO(1, 8) GO(1, 16)
 #undef GO
