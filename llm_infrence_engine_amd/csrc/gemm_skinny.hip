@@ -18,6 +18,7 @@
 // epilogue: norm(x) . W^T = rsqrt(..) * ((x * w) . W^T).
 #include "common.h"
 #include "api.h"
+#include <algorithm>
 
 namespace {
 
@@ -26,8 +27,10 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 enum { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_RESIDUAL = 3 };
 
-// The rows of W are dealt out evenly in units of four (what a lane holds of a tile): the first `rem` blocks take
-// q + 1 units, the others q, at most NTILE tiles of 16 rows either way, the last of them filled in part.  A CU
+constexpr int UNIT = 2;   // rows of W are dealt out in units of two (a gate/up pair)
+
+// The rows of W are dealt out evenly in units of two (a gate/up pair): the first `rem` blocks take q + 1 units,
+// the others q, at most NTILE tiles of 16 rows either way, the last of them filled in part.  A CU
 // draws from memory at a rate of its own, so a product is as slow as its block with the most rows: whole tiles
 // would leave 3 against 2 of them (0.5B gate/up, 608 tiles for 256 CUs) or 2 against 1 (32B o, 320 tiles).
 template <int MT, int NTILE, int WAVES, int EPI, typename TO, bool NORM>
@@ -42,8 +45,8 @@ gemm_skinny_kernel(const void* __restrict__ Av, size_t lda, const bf16* __restri
   const float* X = (const float*)Av;
   const int lane = threadIdx.x & (MS_WAVE - 1), wave = threadIdx.x / MS_WAVE;
   const int col = lane & 15, kq = lane >> 4;
-  const int n0 = ((int)blockIdx.x * q + min((int)blockIdx.x, rem)) * 4;
-  const int n1 = min(N, n0 + (q + ((int)blockIdx.x < rem ? 1 : 0)) * 4);   // this block's rows: n0 .. n1 - 1
+  const int n0 = ((int)blockIdx.x * q + min((int)blockIdx.x, rem)) * UNIT;
+  const int n1 = min(N, n0 + (q + ((int)blockIdx.x < rem ? 1 : 0)) * UNIT);   // this block's rows: n0 .. n1 - 1
   const int nt = (n1 - n0 + 15) / 16;                                      // in tiles, at most NTILE
   const int m0 = blockIdx.y * 16 * MT;   // token groups beyond MT per block go to further blocks along y
   const int total_steps = (K + 31) / 32;
@@ -208,18 +211,21 @@ int launch_cfg(const void* A, size_t lda, const bf16* W, size_t ldw, const float
   const int steps = (K + 31) / 32;
   const int groups = (M + 16 * MT - 1) / (16 * MT);
   const int cus = ms_compute_units();
-  // Every CU should stream an equal share of the matrix: the rows are dealt out in units of four over a whole
-  // number of blocks per CU, of up to four tiles each (no last round that only some CUs take part in); an output
-  // with fewer tiles than CUs has a block per tile; with several token groups four tiles go to a block.
-  // (Measured on the 0.5B shapes at 8 and 64 rows and on the 7B shapes at 8.)
-  const int units = (N + 3) / 4;
+  // Every CU should stream an equal share of the matrix: the rows are dealt out in units of two over a whole
+  // number of blocks per CU, of up to four tiles each (no last round that only some CUs take part in); with
+  // several token groups four tiles go to a block.  An output with fewer tiles than CUs has a block per tile,
+  // or, with up to 16 tokens, blocks of at least 8 rows on as many CUs as that gives (every block reads all the
+  // activations, which is little then; with 32 tokens and more it costs more than the spread saves.  At 8
+  // tokens: o of the 1.5B and 3B shapes 5.1 -> 4.8 and 5.9 -> 5.4 us, down of 3B and 7B 20.2 -> 18.8 and
+  // 36.9 -> 35.5; the 0.5B shapes the same).
+  const int units = (N + UNIT - 1) / UNIT;
   int blocks;
-  if (tiles <= cus) blocks = tiles;
+  if (tiles <= cus) blocks = M <= 16 ? std::max(tiles, std::min(cus, N / 8)) : tiles;
   else if (groups == 1 && tiles <= 16 * cus) blocks = cus * ((tiles + 4 * cus - 1) / (4 * cus));
   else blocks = (tiles + 3) / 4;      // many rounds: the last one matters little (measured: the head)
   if (g_force_ntile) blocks = (tiles + g_force_ntile - 1) / g_force_ntile;
   const int q = units / blocks, rem = units % blocks;   // blocks * q + rem units
-  int ntile = (q + (rem ? 1 : 0) + 3) / 4;              // tiles of the block with the most rows
+  int ntile = ((q + (rem ? 1 : 0)) * UNIT + 15) / 16;   // tiles of the block with the most rows
   if (g_force_ntile && ntile <= g_force_ntile) ntile = g_force_ntile;
   int waves = ntile >= 3 ? (MT <= 2 && (MT == 1 || tiles < 1024) ? 8 : 4) : ((steps >= 32 || MT > 1) ? 16 : 8);
   if (g_force_ntile) waves = g_force_waves;
