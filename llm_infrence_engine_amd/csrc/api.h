@@ -69,11 +69,12 @@ int ms_gemm_panel_splitk(const void* A, long long lda, const void* W, long long 
                          hipStream_t stream);
 
 // Many rows (prompt portions): the tiled matrix-core product, bfloat16 in and out, with the gated activation
-// as epilogue 1; K a multiple of 64 (ms_gemm_tiled_force: measurements, 0 leaves the choice of tile;
+// as epilogue 1; K a multiple of 64 (ms_gemm_tiled_force: measurements, 0 leaves the choice of tile, 1 to 5 force one;
 // ms_gemm_tiled_pays: whether the gated product is faster here than as library product and activation kernel).
 int ms_gemm_tiled(const void* A, long long lda, const void* W, long long ldw, void* out, long long ldo, int M, int N,
                   int K, int epilogue, hipStream_t stream);
 void ms_gemm_tiled_force(int tile);
+void ms_gemm_tiled_force_xcd_split(int xm);   // measurements: rows of XCDs over the tiles (1, 2, 4, 8); 0 leaves the choice
 int ms_gemm_tiled_pays(int M, int N, int K);
 int ms_gemm_tiled_plain_pays(int M, int N, int K);   // the same question for a plain product (epilogue 0)
 

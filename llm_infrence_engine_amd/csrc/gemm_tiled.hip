@@ -305,7 +305,7 @@ int launch(const bf16* A, size_t lda, const bf16* W, size_t ldw, TO* out, size_t
   return ms_launch_status();
 }
 
-int g_tile = 0;   // measurements: 0 leaves the choice of tile, 1, 2 and 3 force one
+int g_tile = 0;   // measurements: 0 leaves the choice of tile; 1 to 5 force one (256, 128, 64, 192, 160 features wide)
 
 // The tile that takes the least time by a model of the measurements.  A block of 256 tokens by 256, 192 or 160
 // features has a CU to itself; its time is what the CU needs to draw its rows (some 40 GB/s whatever the tile), so
