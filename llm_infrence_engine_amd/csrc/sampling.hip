@@ -408,11 +408,25 @@ argmax_chunks_kernel(const float* __restrict__ logits, size_t ld, int V, int n_c
                      int* __restrict__ idx) {
   __shared__ MaxIdx red[4];
   const int r = blockIdx.y, c = blockIdx.x;
-  const int len = (V + n_chunks - 1) / n_chunks;
-  const int begin = c * len, end = min(V, begin + len);
+  const int len = ((V + n_chunks - 1) / n_chunks + 3) & ~3;   // slices start at a multiple of four logits
+  const int begin = min(V, c * len), end = min(V, begin + len);
   const float* row = logits + (size_t)r * ld;
   MaxIdx best = {-INFINITY, 0x7fffffff};
-  for (int i = begin + threadIdx.x; i < end; i += blockDim.x) best = better(best, MaxIdx{row[i], i});
+  if ((((uintptr_t)row) & 15) == 0) {   // four logits a load, and a thread's loads all asked for before the first is used
+    for (int i = begin + threadIdx.x * 4; i < end; i += blockDim.x * 4) {
+      if (i + 3 < end) {
+        const float4 v = *reinterpret_cast<const float4*>(row + i);
+        best = better(best, MaxIdx{v.x, i});
+        best = better(best, MaxIdx{v.y, i + 1});
+        best = better(best, MaxIdx{v.z, i + 2});
+        best = better(best, MaxIdx{v.w, i + 3});
+      } else {
+        for (int j = i; j < end; ++j) best = better(best, MaxIdx{row[j], j});
+      }
+    }
+  } else {
+    for (int i = begin + threadIdx.x; i < end; i += blockDim.x) best = better(best, MaxIdx{row[i], i});
+  }
   for (int o = MS_WAVE / 2; o > 0; o >>= 1) {
     MaxIdx other = {__shfl_xor(best.v, o, MS_WAVE), __shfl_xor(best.i, o, MS_WAVE)};
     best = better(best, other);
