@@ -911,6 +911,20 @@ def test_split_decode_attention_of_very_long_contexts(ops, longest, splits_windo
     torch.testing.assert_close(_run_mfma(ops, c, nh, d, ctx, qlen, splits_window), want, **tol(torch.bfloat16))
 
 
+@pytest.mark.parametrize("nh,nkv,d,window", [(4, 2, 64, None), (2, 1, 128, None), (4, 4, 32, None), (4, 2, 64, 700)])
+def test_prompt_attention_of_thousands_of_tokens(ops, nh, nkv, d, window):
+    """A whole prompt of 3,300 tokens in one step (more column tiles than CUs, late tiles first, every wave of a
+    block many key blocks deep) beside a portion of 1,500 tokens behind a prefix of 1,100, with a far key that
+    stands out for the last query of each."""
+    g = torch.Generator().manual_seed(d + nh)
+    ctx, qlen = [3300, 2600], [3300, 1500]
+    c = _paged_case(g, torch.bfloat16, nh, nkv, d, 16, ctx, qlen, float("nan"))
+    scale = 1.0 / math.sqrt(d)
+    want = torch.cat([attention_reference(q.double(), k.double(), v.double(), scale, window).transpose(0, 1).reshape(-1, nh * d)
+                      for q, k, v in zip(c["qs"], c["ks"], c["vs"])])
+    torch.testing.assert_close(_run_mfma(ops, c, nh, d, ctx, qlen, window), want, **tol(torch.bfloat16))
+
+
 def _run_mfma(ops, c, nh, d, ctx, qlen, window=None):
     N = c["q"].shape[0]
     out = torch.full((N, nh * d), float("nan"), dtype=torch.bfloat16, device=DEV)
